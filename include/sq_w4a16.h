@@ -1,0 +1,110 @@
+/* sq_w4a16.h -- C ABI of libsq_w4a16.so: W4A16 quantized linear on MI355X (gfx950).
+ *
+ * Every entry point takes plain device pointers and sizes, launches on the
+ * given HIP stream (a hipStream_t passed as void*; NULL = the null stream),
+ * never allocates or frees device memory, never synchronises, never throws.
+ * The return value is 0 on success or one of the SQ_ERR_* codes; on any error
+ * nothing has been launched.  All matrices are dense and row-major.
+ *
+ * Weight layouts
+ *   SQ_LAYOUT_L1  weight  uint8 [N, K/2] == uint32 [N, K/8]; the nibbles of a
+ *                 word, least significant first, hold k0,k2,k4,k6,k1,k3,k5,k7
+ *                 of 8 consecutive k.  zeros_scales fp16 [N, 2K/g]: pairs
+ *                 (zero + 64, scale) per (row, group).
+ *                 (reference: test/muxi/utils/quant_funcs.py:75-83,116-127,142-174)
+ *   SQ_LAYOUT_L2  weight  int32 [K, N/8] in the tensor-core tile order produced
+ *                 by convert_ours_to_awq + convert_awq_to_lmdeploy;
+ *                 zeros_scales fp16 [K/g, 2N]: pairs (zero + 64, scale) per
+ *                 (group, column).  Group size must be 128.
+ *                 (reference: test/nvidia/utils/quant_dequant_nvidia.py:5-32)
+ */
+#ifndef SQ_W4A16_H
+#define SQ_W4A16_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SQ_OK 0
+#define SQ_ERR_NULL_POINTER 1    /* a required pointer is NULL */
+#define SQ_ERR_BAD_SHAPE 2       /* M/N/K out of range or not a supported multiple */
+#define SQ_ERR_BAD_GROUP 3       /* unsupported group size */
+#define SQ_ERR_BAD_LAYOUT 4      /* unknown layout id */
+#define SQ_ERR_BAD_ALGO 5        /* unknown or inapplicable kernel id */
+#define SQ_ERR_MISALIGNED 6      /* pointer not 16-byte aligned */
+#define SQ_ERR_LAUNCH 7          /* the HIP runtime rejected the launch */
+#define SQ_ERR_WORKSPACE 8       /* workspace missing or too small */
+
+#define SQ_LAYOUT_L1 1
+#define SQ_LAYOUT_L2 2
+
+/* Kernel selection for sq_w4a16_gemm_ex (SQ_ALGO_AUTO is what sq_w4a16_gemm uses). */
+#define SQ_ALGO_AUTO 0
+#define SQ_ALGO_GEMV 1           /* M <= 8: lane-private rows on 4x4x4 MFMA, exact W_hat */
+#define SQ_ALGO_GEMV_FIXUP 2     /* M <= 8: same, zero/scale applied per group in fp32 */
+#define SQ_ALGO_SKINNY 3         /* M <= 64: 16-column MFMA tiles, weights straight from registers */
+#define SQ_ALGO_GEMM 4           /* any M: LDS-tiled MFMA GEMM */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int sq_version(void);
+
+/* Static, human-readable text for an SQ_ERR_* code. */
+const char* sq_strerror(int code);
+
+/* Y[M,N] (fp16) = X[M,K] (fp16) * W_hat^T, W_hat[n,k] = (q - z) * s, fp32
+ * accumulation.  Replaces the body of gemm_awq_ut / Gemm_awq_pure
+ * (reference: quantization/muxi/backend/gemm_quant.cu:12-59,84-109;
+ * quantization/nvidia/kernel/gemm_quant.cu:13-40,98-123).
+ * Requirements: M >= 1; N % 8 == 0; K % 32 == 0; K % g == 0; g in {32,64,128}
+ * for L1 (g == 128 for L2, plus K % 32 == 0 and N % 32 == 0); x, w, zs, y
+ * 16-byte aligned.  M == 0 is accepted and launches nothing. */
+int sq_w4a16_gemm(const void* x, const void* w, const void* zs, void* y,
+                  int M, int N, int K, int group_size, int layout, void* stream);
+
+/* Same with an explicit kernel choice (tests and benchmarks). */
+int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y,
+                     int M, int N, int K, int group_size, int layout, int algo,
+                     void* stream);
+
+/* out[N,K] (fp16) = W_hat in natural k order, bit-identical to fp16
+ * (q_fp16 - z_fp16) * s_fp16.  Replaces dequant
+ * (reference: quantization/tianshu/backend/gemm_quant.cu:153-164 and
+ * quantization/tianshu/backend/w4a16_gemm.cuh:1060-1154). */
+int sq_w4a16_dequant(const void* w, const void* zs, void* out, int N, int K,
+                     int group_size, int layout, void* stream);
+
+/* zeros, scales fp16 [N, K/g] (zeros without the +64) -> zs fp16 [K/g, 2N]
+ * = pairs (zero + 64, scale).  Replaces transpose_merge_zeros_scales
+ * (reference: quantization/nvidia/kernel/gemm_s4_f16/format.cu:206-239). */
+int sq_transpose_merge_zeros_scales(const void* zeros, const void* scales, void* zs,
+                                    int in_features, int out_features, int group_size,
+                                    void* stream);
+
+/* src uint8 [N, K/2] (even k in the high nibble) -> dst uint32 [K, N/8], word
+ * (k,c) holding columns 8c + {0,2,4,6,1,3,5,7}.  Replaces convert_ours_to_awq
+ * (reference: quantization/nvidia/kernel/gemm_s4_f16/format.cu:151-201). */
+int sq_convert_ours_to_awq(const void* src, void* dst, int in_features, int out_features,
+                           void* stream);
+
+/* src uint32 [K, N/8] (AWQ order) -> dst int32 [K, N/8] storage in layout L2.
+ * Replaces convert_awq_to_lmdeploy
+ * (reference: quantization/nvidia/kernel/gemm_s4_f16/format.cu:24-57,66-71,135-149).
+ * Needs K % 32 == 0 and N % 32 == 0; src and dst must not overlap. */
+int sq_convert_awq_to_lmdeploy(const void* src, void* dst, int in_features, int out_features,
+                               void* stream);
+
+/* Layout L2 -> layout L1 (weight and zeros_scales), so that an L2 checkpoint
+ * can be served by the L1 kernels.  No counterpart in the reference (its
+ * back-ends each accept one layout only). */
+int sq_repack_l2_to_l1(const void* w_l2, const void* zs_l2, void* w_l1, void* zs_l1,
+                       int N, int K, int group_size, void* stream);
+
+/* 2-bit packed weight uint8 [N, K/4] -> 4-bit packed uint8 [N, K/2] (layout
+ * L1 nibbles).  Replaces WALinear.convert_2bit_to_4bit
+ * (reference: test/muxi/module/qlinear/qlinear.py:93-103). */
+int sq_convert_2bit_to_4bit(const void* src, void* dst, int N, int K, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SQ_W4A16_H */

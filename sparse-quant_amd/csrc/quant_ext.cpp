@@ -1,0 +1,270 @@
+// `quant`: the PyTorch-ROCm extension module the reference's Python code imports
+// (`from quant import gemm_awq_ut, dequant, transpose_merge_zeros_scales, ...`).
+// Host C++ only: it validates tensors the way the reference does, takes torch's
+// current HIP stream and forwards raw pointers to the C ABI of libsq_w4a16.so.
+//
+// Reference interfaces mirrored here:
+//   gemm_awq_ut / Gemm_awq_pure   quantization/nvidia/kernel/gemm_quant.cu:42-123,
+//                                 quantization/muxi/backend/gemm_quant.cu:12-109
+//   dequant                       quantization/tianshu/backend/gemm_quant.cu:153-164
+//   transpose_merge_zeros_scales, convert_ours_to_awq, convert_awq_to_lmdeploy
+//                                 quantization/nvidia/kernel/gemm_s4_f16/format.cu:135-239
+//   module definition             quantization/{nvidia/kernel,muxi/backend,tianshu/backend}/pybind.cpp
+#include <torch/extension.h>
+
+#include <c10/core/DeviceGuard.h>
+#include <c10/hip/HIPStream.h>
+
+#include <mutex>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+
+#include "sq_w4a16.h"
+
+namespace {
+
+#define SQ_CHECK_DEVICE(x) TORCH_CHECK((x).is_cuda(), "Tensor " #x " must be on CUDA")
+#define SQ_CHECK_CONTIGUOUS(x) TORCH_CHECK((x).is_contiguous(), "Tensor " #x " must be contiguous")
+#define SQ_CHECK_DTYPE(x, t) TORCH_CHECK((x).dtype() == (t), "Tensor " #x " must have dtype (" #t ")")
+#define SQ_CHECK_DIMS(x, d) TORCH_CHECK((x).dim() == (d), "Tensor " #x " must have dimension number (" #d ")")
+
+void* current_stream(const at::Tensor& t) {
+    return static_cast<void*>(c10::hip::getCurrentHIPStream(t.device().index()).stream());
+}
+
+void raise_if_error(int code, const char* what) {
+    if (code == SQ_OK) return;
+    const std::string msg = std::string(what) + ": " + sq_strerror(code);
+    // Shape / group complaints surface as ValueError like the wave64 back-ends'
+    // std::invalid_argument; everything else as RuntimeError like TORCH_CHECK.
+    if (code == SQ_ERR_BAD_SHAPE) throw std::invalid_argument(msg);
+    throw std::runtime_error(msg);
+}
+
+int layout_of(const at::Tensor& W) {
+    if (W.scalar_type() == at::kByte) return SQ_LAYOUT_L1;
+    if (W.scalar_type() == at::kInt) return SQ_LAYOUT_L2;
+    TORCH_CHECK(false, "Tensor W must have dtype uint8 ([N, K/2], wave64 layout) or int32 ([K, N/8], "
+                       "tensor-core layout)");
+    return 0;
+}
+
+// Layout-L2 weights are converted to L1 once and kept while the source tensor
+// lives.  The key is the source's data pointer; an entry is valid only while the
+// source storage is alive (weak reference) and unmodified (version counter).
+struct RepackEntry {
+    c10::weak_intrusive_ptr<c10::StorageImpl> src_storage;
+    int64_t version;
+    at::Tensor w_l1, zs_l1;
+};
+std::mutex g_cache_mutex;
+std::unordered_map<const void*, RepackEntry> g_repack_cache;
+
+void sweep_cache_locked() {
+    for (auto it = g_repack_cache.begin(); it != g_repack_cache.end();) {
+        if (it->second.src_storage.expired())
+            it = g_repack_cache.erase(it);
+        else
+            ++it;
+    }
+}
+
+std::pair<at::Tensor, at::Tensor> l1_view_of_l2(const at::Tensor& W, const at::Tensor& ZS, int N, int K, int g) {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    const void* key = W.data_ptr();
+    auto it = g_repack_cache.find(key);
+    if (it != g_repack_cache.end() && !it->second.src_storage.expired() &&
+        it->second.version == W._version() && it->second.w_l1.size(0) == N && it->second.w_l1.size(1) == K / 2)
+        return {it->second.w_l1, it->second.zs_l1};
+    sweep_cache_locked();
+    at::Tensor w1 = torch::empty({N, K / 2}, W.options().dtype(at::kByte));
+    at::Tensor zs1 = torch::empty({N, 2 * (K / g)}, ZS.options());
+    raise_if_error(sq_repack_l2_to_l1(W.data_ptr(), ZS.data_ptr(), w1.data_ptr(), zs1.data_ptr(), N, K, g,
+                                      current_stream(W)),
+                   "repack");
+    RepackEntry e{c10::weak_intrusive_ptr<c10::StorageImpl>(W.storage().getWeakStorageImpl()), W._version(), w1, zs1};
+    g_repack_cache.erase(key);
+    g_repack_cache.emplace(key, std::move(e));
+    return {w1, zs1};
+}
+
+at::Tensor gemm_impl(const at::Tensor& I, const at::Tensor& W, const at::Tensor& ZS, int N, int group_size,
+                     int algo) {
+    SQ_CHECK_DEVICE(I);
+    SQ_CHECK_DEVICE(W);
+    SQ_CHECK_DEVICE(ZS);
+    SQ_CHECK_CONTIGUOUS(I);
+    SQ_CHECK_CONTIGUOUS(W);
+    SQ_CHECK_CONTIGUOUS(ZS);
+    SQ_CHECK_DTYPE(I, at::kHalf);
+    SQ_CHECK_DTYPE(ZS, at::kHalf);
+    SQ_CHECK_DIMS(I, 3);
+    SQ_CHECK_DIMS(W, 2);
+    SQ_CHECK_DIMS(ZS, 2);
+    const int layout = layout_of(W);
+    const int64_t M = I.size(0) * I.size(1);
+    const int64_t K = I.size(2);
+    if (group_size <= 0 || K % group_size != 0) throw std::invalid_argument("embbed dim must be a multiple of group_size!");
+    if (layout == SQ_LAYOUT_L1) {
+        if (W.size(0) != N) throw std::invalid_argument("output dim mismatch!");
+        if (W.size(1) * 2 != K) throw std::invalid_argument("input dim mismatch!");
+        if (ZS.size(0) != N || ZS.size(1) != 2 * (K / group_size))
+            throw std::invalid_argument("zeros_scales shape mismatch!");
+    } else {
+        if (W.size(0) != K) throw std::invalid_argument("input dim mismatch!");
+        if (W.size(1) * 8 != N) throw std::invalid_argument("output dim mismatch!");
+        if (group_size != 128) throw std::runtime_error("unsupported group size");
+        if (ZS.size(0) != K / group_size || ZS.size(1) != 2 * (int64_t)N)
+            throw std::invalid_argument("zeros_scales shape mismatch!");
+    }
+    TORCH_CHECK(M < (1LL << 31) && K < (1LL << 31), "problem too large");
+
+    c10::DeviceGuard guard(I.device());
+    at::Tensor O = torch::empty({I.size(0), I.size(1), N}, I.options());
+    const void* w_ptr = W.data_ptr();
+    const void* zs_ptr = ZS.data_ptr();
+    std::pair<at::Tensor, at::Tensor> keep;
+    if (layout == SQ_LAYOUT_L2) {
+        keep = l1_view_of_l2(W, ZS, N, (int)K, group_size);
+        w_ptr = keep.first.data_ptr();
+        zs_ptr = keep.second.data_ptr();
+    }
+    raise_if_error(sq_w4a16_gemm_ex(I.data_ptr(), w_ptr, zs_ptr, O.data_ptr(), (int)M, N, (int)K, group_size,
+                                    SQ_LAYOUT_L1, algo, current_stream(I)),
+                   "gemm_awq_ut");
+    return O;
+}
+
+// I [bs, seq, K] fp16; W / W_zeros_scales in layout L1 or L2; returns [bs, seq, N].
+// As in the reference the M and K arguments are not used: M is bs*seq and K is
+// I.size(2).
+at::Tensor gemm_awq_ut(at::Tensor I, at::Tensor W, at::Tensor W_zeros_scales, const int M, const int N,
+                       const int K, const int group_size) {
+    (void)M;
+    (void)K;
+    return gemm_impl(I, W, W_zeros_scales, N, group_size, SQ_ALGO_AUTO);
+}
+
+// Same with an explicit kernel id (SQ_ALGO_* | tuning word << 8); for tests and benchmarks.
+at::Tensor gemm_awq_algo(at::Tensor I, at::Tensor W, at::Tensor W_zeros_scales, const int N, const int group_size,
+                         const int algo) {
+    return gemm_impl(I, W, W_zeros_scales, N, group_size, algo);
+}
+
+at::Tensor dequant(at::Tensor W, at::Tensor zeros_scales, const int N, const int K, const int group_size) {
+    SQ_CHECK_DEVICE(W);
+    SQ_CHECK_DEVICE(zeros_scales);
+    SQ_CHECK_CONTIGUOUS(W);
+    SQ_CHECK_CONTIGUOUS(zeros_scales);
+    SQ_CHECK_DTYPE(zeros_scales, at::kHalf);
+    SQ_CHECK_DIMS(W, 2);
+    const int layout = layout_of(W);
+    if (layout == SQ_LAYOUT_L1) {
+        if (W.size(0) != N || W.size(1) * 2 != K) throw std::invalid_argument("weight shape mismatch!");
+    } else {
+        if (W.size(0) != K || W.size(1) * 8 != N) throw std::invalid_argument("weight shape mismatch!");
+    }
+    if (group_size <= 0 || K % group_size != 0 || zeros_scales.numel() != 2 * (int64_t)N * (K / group_size))
+        throw std::invalid_argument("zeros_scales shape mismatch!");
+    c10::DeviceGuard guard(W.device());
+    at::Tensor out = torch::empty({N, K}, zeros_scales.options());
+    raise_if_error(sq_w4a16_dequant(W.data_ptr(), zeros_scales.data_ptr(), out.data_ptr(), N, K, group_size, layout,
+                                    current_stream(W)),
+                   "dequant");
+    return out;
+}
+
+void transpose_merge_zeros_scales(at::Tensor zeros, at::Tensor scales, at::Tensor zeros_scales, int in_features,
+                                  int out_features, int group_size) {
+    SQ_CHECK_DEVICE(zeros);
+    SQ_CHECK_DEVICE(scales);
+    SQ_CHECK_DEVICE(zeros_scales);
+    SQ_CHECK_CONTIGUOUS(zeros);
+    SQ_CHECK_CONTIGUOUS(scales);
+    SQ_CHECK_CONTIGUOUS(zeros_scales);
+    SQ_CHECK_DTYPE(zeros, at::kHalf);
+    SQ_CHECK_DTYPE(scales, at::kHalf);
+    SQ_CHECK_DTYPE(zeros_scales, at::kHalf);
+    TORCH_CHECK(group_size > 0 && in_features % group_size == 0, "in_features must be a multiple of group_size");
+    const int64_t count = (int64_t)out_features * (in_features / group_size);
+    TORCH_CHECK(zeros.numel() == count && scales.numel() == count && zeros_scales.numel() == 2 * count,
+                "zeros / scales / zeros_scales sizes do not match in_features, out_features, group_size");
+    c10::DeviceGuard guard(zeros.device());
+    raise_if_error(sq_transpose_merge_zeros_scales(zeros.data_ptr(), scales.data_ptr(), zeros_scales.data_ptr(),
+                                                   in_features, out_features, group_size, current_stream(zeros)),
+                   "transpose_merge_zeros_scales");
+}
+
+void convert_ours_to_awq(at::Tensor qweight_src, at::Tensor qweight_dst, int in_features, int out_features) {
+    SQ_CHECK_DEVICE(qweight_src);
+    SQ_CHECK_DEVICE(qweight_dst);
+    SQ_CHECK_CONTIGUOUS(qweight_src);
+    SQ_CHECK_CONTIGUOUS(qweight_dst);
+    SQ_CHECK_DTYPE(qweight_src, at::kByte);
+    TORCH_CHECK(qweight_src.numel() == (int64_t)out_features * in_features / 2, "qweight_src size mismatch");
+    TORCH_CHECK((int64_t)qweight_dst.numel() * qweight_dst.element_size() == (int64_t)in_features * out_features / 2,
+                "qweight_dst size mismatch");
+    c10::DeviceGuard guard(qweight_src.device());
+    raise_if_error(sq_convert_ours_to_awq(qweight_src.data_ptr(), qweight_dst.data_ptr(), in_features, out_features,
+                                          current_stream(qweight_src)),
+                   "convert_ours_to_awq");
+}
+
+void convert_awq_to_lmdeploy(at::Tensor qweight, at::Tensor qweight_dst, int in_features, int out_features) {
+    SQ_CHECK_DEVICE(qweight);
+    SQ_CHECK_DEVICE(qweight_dst);
+    SQ_CHECK_CONTIGUOUS(qweight);
+    SQ_CHECK_CONTIGUOUS(qweight_dst);
+    SQ_CHECK_DTYPE(qweight_dst, at::kInt);
+    TORCH_CHECK((int64_t)qweight.numel() * qweight.element_size() == (int64_t)in_features * out_features / 2,
+                "qweight size mismatch");
+    TORCH_CHECK(qweight_dst.numel() == (int64_t)in_features * out_features / 8, "qweight_dst size mismatch");
+    c10::DeviceGuard guard(qweight.device());
+    raise_if_error(sq_convert_awq_to_lmdeploy(qweight.data_ptr(), qweight_dst.data_ptr(), in_features, out_features,
+                                              current_stream(qweight)),
+                   "convert_awq_to_lmdeploy");
+}
+
+// uint8 [N, K/4] 2-bit packed -> uint8 [N, K/2] 4-bit packed (layout L1).
+at::Tensor convert_2bit_to_4bit(at::Tensor qweight_2bit) {
+    SQ_CHECK_DEVICE(qweight_2bit);
+    SQ_CHECK_CONTIGUOUS(qweight_2bit);
+    SQ_CHECK_DTYPE(qweight_2bit, at::kByte);
+    SQ_CHECK_DIMS(qweight_2bit, 2);
+    c10::DeviceGuard guard(qweight_2bit.device());
+    const int N = (int)qweight_2bit.size(0);
+    const int K = (int)qweight_2bit.size(1) * 4;
+    at::Tensor out = torch::empty({N, K / 2}, qweight_2bit.options());
+    raise_if_error(sq_convert_2bit_to_4bit(qweight_2bit.data_ptr(), out.data_ptr(), N, K, current_stream(qweight_2bit)),
+                   "convert_2bit_to_4bit");
+    return out;
+}
+
+void clear_repack_cache() {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    g_repack_cache.clear();
+}
+
+int repack_cache_size() {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    sweep_cache_locked();
+    return (int)g_repack_cache.size();
+}
+
+}  // namespace
+
+PYBIND11_MODULE(quant, m) {
+    m.doc() = "W4A16 quantized linear for MI355X (gfx950): drop-in for the reference's `quant` extension";
+    m.def("gemm_awq_ut", &gemm_awq_ut);
+    m.def("dequant", &dequant);
+    m.def("transpose_merge_zeros_scales", &transpose_merge_zeros_scales);
+    m.def("convert_ours_to_awq", &convert_ours_to_awq);
+    m.def("convert_awq_to_lmdeploy", &convert_awq_to_lmdeploy);
+    // Additions without a counterpart in the reference's module.
+    m.def("gemm_awq_algo", &gemm_awq_algo);
+    m.def("convert_2bit_to_4bit", &convert_2bit_to_4bit);
+    m.def("clear_repack_cache", &clear_repack_cache);
+    m.def("repack_cache_size", &repack_cache_size);
+    m.def("version", []() { return sq_version(); });
+}

@@ -1,0 +1,146 @@
+// C ABI of libsq_w4a16.so: argument validation and kernel dispatch.  Declarations
+// and the contract of every entry point are in include/sq_w4a16.h.
+#include "../../include/sq_w4a16.h"
+
+#include "sq_kernels.h"
+
+namespace {
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int launch_code(hipError_t e) { return e == hipSuccess ? SQ_OK : SQ_ERR_LAUNCH; }
+inline bool pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
+// Shape rules shared by gemm and dequant.
+int check_weight(int N, int K, int g, int layout) {
+    if (layout != SQ_LAYOUT_L1 && layout != SQ_LAYOUT_L2) return SQ_ERR_BAD_LAYOUT;
+    if (N <= 0 || K <= 0) return SQ_ERR_BAD_SHAPE;
+    if (layout == SQ_LAYOUT_L1) {
+        if (g != 32 && g != 64 && g != 128) return SQ_ERR_BAD_GROUP;
+        if (N % 8 != 0 || K % 32 != 0 || K % g != 0) return SQ_ERR_BAD_SHAPE;
+    } else {
+        if (g != 128) return SQ_ERR_BAD_GROUP;
+        if (N % 32 != 0 || K % 32 != 0 || K % g != 0) return SQ_ERR_BAD_SHAPE;
+    }
+    if ((long)N * (long)K > (1L << 40)) return SQ_ERR_BAD_SHAPE;
+    return SQ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int sq_version(void) { return 100; }
+
+const char* sq_strerror(int code) {
+    switch (code) {
+        case SQ_OK: return "ok";
+        case SQ_ERR_NULL_POINTER: return "null pointer argument";
+        case SQ_ERR_BAD_SHAPE: return "unsupported shape (need N % 8 == 0, K % 32 == 0, K % group_size == 0)";
+        case SQ_ERR_BAD_GROUP: return "unsupported group size";
+        case SQ_ERR_BAD_LAYOUT: return "unknown or unsupported weight layout";
+        case SQ_ERR_BAD_ALGO: return "unknown kernel id or kernel not applicable to this shape";
+        case SQ_ERR_MISALIGNED: return "pointer is not 16-byte aligned";
+        case SQ_ERR_LAUNCH: return "HIP kernel launch failed";
+        case SQ_ERR_WORKSPACE: return "workspace missing or too small";
+        default: return "unknown error code";
+    }
+}
+
+int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
+                     int layout, int algo, void* stream) {
+    if (M < 0) return SQ_ERR_BAD_SHAPE;
+    const int rc = check_weight(N, K, group_size, layout);
+    if (rc != SQ_OK) return rc;
+    // The GEMM kernels consume layout L1; an L2 weight is converted once with
+    // sq_repack_l2_to_l1 by the caller (the `quant` extension caches the result).
+    if (layout != SQ_LAYOUT_L1) return SQ_ERR_BAD_LAYOUT;
+    if (M == 0) return SQ_OK;
+    if (!x || !w || !zs || !y) return SQ_ERR_NULL_POINTER;
+    if (!aligned16(x) || !aligned16(w) || !aligned16(zs) || !aligned16(y)) return SQ_ERR_MISALIGNED;
+    if ((long)M * (long)K > (1L << 40) || (long)M * (long)N > (1L << 40)) return SQ_ERR_BAD_SHAPE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    int kernel = algo & 0xFF;
+    const int tune = (algo >> 8) & 0xFFFF;
+    if (kernel == SQ_ALGO_AUTO) {
+        if (M <= 8)
+            kernel = SQ_ALGO_GEMV_FIXUP;
+        else if (M <= 32)
+            kernel = SQ_ALGO_SKINNY;
+        else
+            kernel = SQ_ALGO_GEMM;
+    }
+    switch (kernel) {
+        case SQ_ALGO_GEMV:
+        case SQ_ALGO_GEMV_FIXUP:
+            if (M > 8) return SQ_ERR_BAD_ALGO;
+            return launch_code(sq::launch_gemv_tuned(x, w, zs, y, M, N, K, group_size,
+                                                     kernel == SQ_ALGO_GEMV_FIXUP, tune, st));
+        case SQ_ALGO_SKINNY:
+            if (M > 64) return SQ_ERR_BAD_ALGO;
+            return launch_code(sq::launch_skinny_tuned(x, w, zs, y, M, N, K, group_size, tune, st));
+        case SQ_ALGO_GEMM:
+            return launch_code(sq::launch_gemm_tuned(x, w, zs, y, M, N, K, group_size, tune, st));
+        default:
+            return SQ_ERR_BAD_ALGO;
+    }
+}
+
+int sq_w4a16_gemm(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
+                  int layout, void* stream) {
+    return sq_w4a16_gemm_ex(x, w, zs, y, M, N, K, group_size, layout, SQ_ALGO_AUTO, stream);
+}
+
+int sq_w4a16_dequant(const void* w, const void* zs, void* out, int N, int K, int group_size, int layout,
+                     void* stream) {
+    const int rc = check_weight(N, K, group_size, layout);
+    if (rc != SQ_OK) return rc;
+    if (!w || !zs || !out) return SQ_ERR_NULL_POINTER;
+    if (!aligned16(w) || !aligned16(zs) || !aligned16(out)) return SQ_ERR_MISALIGNED;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (layout == SQ_LAYOUT_L1) return launch_code(sq::launch_dequant_l1(w, zs, out, N, K, group_size, st));
+    return launch_code(sq::launch_dequant_l2(w, zs, out, N, K, group_size, st));
+}
+
+int sq_transpose_merge_zeros_scales(const void* zeros, const void* scales, void* zs, int in_features,
+                                    int out_features, int group_size, void* stream) {
+    if (in_features <= 0 || out_features <= 0) return SQ_ERR_BAD_SHAPE;
+    if (group_size <= 0 || in_features % group_size != 0) return SQ_ERR_BAD_GROUP;
+    if (!zeros || !scales || !zs) return SQ_ERR_NULL_POINTER;
+    return launch_code(sq::launch_transpose_merge_zeros_scales(zeros, scales, zs, in_features, out_features,
+                                                               group_size, static_cast<hipStream_t>(stream)));
+}
+
+int sq_convert_ours_to_awq(const void* src, void* dst, int in_features, int out_features, void* stream) {
+    if (in_features <= 0 || out_features <= 0 || in_features % 2 != 0 || out_features % 8 != 0)
+        return SQ_ERR_BAD_SHAPE;
+    if (!src || !dst) return SQ_ERR_NULL_POINTER;
+    return launch_code(
+        sq::launch_ours_to_awq(src, dst, in_features, out_features, static_cast<hipStream_t>(stream)));
+}
+
+int sq_convert_awq_to_lmdeploy(const void* src, void* dst, int in_features, int out_features, void* stream) {
+    if (in_features <= 0 || out_features <= 0 || in_features % 32 != 0 || out_features % 32 != 0)
+        return SQ_ERR_BAD_SHAPE;
+    if (!src || !dst) return SQ_ERR_NULL_POINTER;
+    if (src == dst) return SQ_ERR_BAD_SHAPE;
+    return launch_code(
+        sq::launch_awq_to_lmdeploy(src, dst, in_features, out_features, static_cast<hipStream_t>(stream)));
+}
+
+int sq_repack_l2_to_l1(const void* w_l2, const void* zs_l2, void* w_l1, void* zs_l1, int N, int K, int group_size,
+                       void* stream) {
+    const int rc = check_weight(N, K, group_size, SQ_LAYOUT_L2);
+    if (rc != SQ_OK) return rc;
+    if (!w_l2 || !zs_l2 || !w_l1 || !zs_l1) return SQ_ERR_NULL_POINTER;
+    return launch_code(
+        sq::launch_l2_to_l1(w_l2, zs_l2, w_l1, zs_l1, N, K, group_size, static_cast<hipStream_t>(stream)));
+}
+
+int sq_convert_2bit_to_4bit(const void* src, void* dst, int N, int K, void* stream) {
+    if (N <= 0 || K <= 0 || K % 4 != 0) return SQ_ERR_BAD_SHAPE;
+    if (!src || !dst) return SQ_ERR_NULL_POINTER;
+    return launch_code(sq::launch_2bit_to_4bit(src, dst, N, K, static_cast<hipStream_t>(stream)));
+}
+
+}  // extern "C"

@@ -1,0 +1,77 @@
+// Shared device helpers for the W4A16 kernels (gfx950 / CDNA4, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sq {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+template <typename To, typename From>
+__device__ __forceinline__ To bit_cast(const From& v) {
+    static_assert(sizeof(To) == sizeof(From), "size mismatch");
+    return __builtin_bit_cast(To, v);
+}
+
+// One packed word (layout L1: nibbles k0,k2,k4,k6,k1,k3,k5,k7 from the least
+// significant) -> four half2 bit patterns holding 64 + q for (k0,k1), (k2,k3),
+// (k4,k5), (k6,k7).  0x5400 is fp16 64.0 and ulp(64) = 1/16, so a nibble placed
+// in mantissa bits 4..7 adds exactly its value.
+// (reference: quantization/muxi/backend/utils.cuh:81-134)
+__device__ __forceinline__ void unpack8_bias64(uint32_t w, uint32_t h[4]) {
+    const uint32_t t = w >> 8;
+    h[0] = ((w & 0x000F000Fu) | 0x05400540u) << 4;
+    h[1] = (w & 0x00F000F0u) | 0x54005400u;
+    h[2] = ((t & 0x000F000Fu) | 0x05400540u) << 4;
+    h[3] = (t & 0x00F000F0u) | 0x54005400u;
+}
+
+// (h - z64) * s on a half2, each operation rounded once in fp16: the difference
+// of two values in [64,79] is exact, so the result is the correctly rounded
+// (q - z) * s.  (reference: quantization/muxi/backend/w4a16_gemm.cuh:58-81)
+__device__ __forceinline__ uint32_t dequant_pair(uint32_t h, half2_t z64, half2_t s) {
+    half2_t v = bit_cast<half2_t>(h);
+    v = (v - z64) * s;
+    return bit_cast<uint32_t>(v);
+}
+
+// Word -> 8 dequantised fp16 (natural k order) as one 128-bit value.
+__device__ __forceinline__ half8_t dequant8(uint32_t w, half2_t z64, half2_t s) {
+    uint32_t h[4];
+    unpack8_bias64(w, h);
+    u32x4_t r;
+    r.x = dequant_pair(h[0], z64, s);
+    r.y = dequant_pair(h[1], z64, s);
+    r.z = dequant_pair(h[2], z64, s);
+    r.w = dequant_pair(h[3], z64, s);
+    return bit_cast<half8_t>(r);
+}
+
+// Word -> 8 fp16 holding 64 + q (no zero / scale applied).
+__device__ __forceinline__ half8_t unpack8_raw(uint32_t w) {
+    uint32_t h[4];
+    unpack8_bias64(w, h);
+    u32x4_t r = {h[0], h[1], h[2], h[3]};
+    return bit_cast<half8_t>(r);
+}
+
+// Sum over the four lanes {l, l^4, l^8, l^12} of a 16-lane row using DPP row
+// rotations (no LDS traffic).
+__device__ __forceinline__ float row_sum_stride4(float v) {
+    int i = bit_cast<int>(v);
+    v += bit_cast<float>(__builtin_amdgcn_update_dpp(0, i, 0x124, 0xF, 0xF, false));  // row_ror:4
+    i = bit_cast<int>(v);
+    v += bit_cast<float>(__builtin_amdgcn_update_dpp(0, i, 0x128, 0xF, 0xF, false));  // row_ror:8
+    return v;
+}
+
+__device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
+
+}  // namespace sq

@@ -1,0 +1,34 @@
+// Internal launch interface between the C ABI (sq_api.hip) and the kernel files.
+// Every launcher assumes its arguments were validated by the caller, enqueues on
+// `st` and returns the hipError_t of the launch.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sq {
+
+// sq_dequant.hip
+hipError_t launch_dequant_l1(const void* w, const void* zs, void* out, int N, int K, int g, hipStream_t st);
+hipError_t launch_dequant_l2(const void* w, const void* zs, void* out, int N, int K, int g, hipStream_t st);
+
+// sq_repack.hip
+hipError_t launch_transpose_merge_zeros_scales(const void* zeros, const void* scales, void* zs, int K, int N,
+                                               int g, hipStream_t st);
+hipError_t launch_ours_to_awq(const void* src, void* dst, int K, int N, hipStream_t st);
+hipError_t launch_awq_to_lmdeploy(const void* src, void* dst, int K, int N, hipStream_t st);
+hipError_t launch_l2_to_l1(const void* w_l2, const void* zs_l2, void* w_l1, void* zs_l1, int N, int K, int g,
+                           hipStream_t st);
+hipError_t launch_2bit_to_4bit(const void* src, void* dst, int N, int K, hipStream_t st);
+
+// The *_tuned launchers take a kernel-specific tuning word (0 = built-in heuristic).
+// sq_gemv.hip: M <= 8.  tune = row steps per workgroup (1,2,4) | waves << 8.
+hipError_t launch_gemv_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
+                             bool fixup, int tune, hipStream_t st);
+// sq_skinny.hip: M <= 64.  tune = waves | mode << 8 (mode 1 = exact, 2 = fixup).
+hipError_t launch_skinny_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
+                               int tune, hipStream_t st);
+// sq_gemm.hip: any M.  tune = 32-row tiles per workgroup (1,2,4).
+hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
+                             int tune, hipStream_t st);
+
+}  // namespace sq

@@ -1,0 +1,102 @@
+"""Build recipe: libsq_w4a16.so (HIP kernels + C ABI) and the `quant` torch extension.
+
+Both are built in-tree, next to the `sqamd` package (the directory that is put on
+sys.path so that `import quant` finds the extension):
+
+    sparse-quant_amd/libsq_w4a16.so
+    sparse-quant_amd/quant.cpython-<abi>.so
+
+hipcc cross-compiles for gfx950 without a GPU.  Run as `python -m sqamd.build`
+from sparse-quant_amd/, or call build_all().
+"""
+import os
+import subprocess
+import sys
+import sysconfig
+from concurrent.futures import ThreadPoolExecutor
+
+PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))  # sparse-quant_amd/
+REPO_ROOT = os.path.dirname(PKG_ROOT)
+CSRC = os.path.join(PKG_ROOT, "csrc")
+OBJ_DIR = os.path.join(PKG_ROOT, "build")
+LIB_PATH = os.path.join(PKG_ROOT, "libsq_w4a16.so")
+EXT_PATH = os.path.join(PKG_ROOT, "quant" + sysconfig.get_config_var("EXT_SUFFIX"))
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+
+HIP_SOURCES = ["sq_api.hip", "sq_dequant.hip", "sq_repack.hip", "sq_gemv.hip", "sq_skinny.hip", "sq_gemm.hip",
+               "sq_attn.hip"]
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+             # keep the compiler from forming packed-fp32 instructions
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops' is not a recognized feature" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    if out.strip():
+        print(out)
+
+
+def build_lib(verbose=True):
+    """Compile every HIP source for gfx950 and link libsq_w4a16.so."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    hipcc = os.path.join(ROCM, "bin", "hipcc")
+    sources = [s for s in HIP_SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    objs = [os.path.join(OBJ_DIR, s.replace(".hip", ".o")) for s in sources]
+
+    def compile_one(pair):
+        src, obj = pair
+        _run([hipcc] + HIP_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
+        list(pool.map(compile_one, zip(sources, objs)))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs +
+         ["-Wl,-rpath," + os.path.join(ROCM, "lib")])
+    if verbose:
+        print("built", LIB_PATH)
+    return LIB_PATH
+
+
+def build_ext(verbose=True):
+    """Compile the `quant` torch extension (host C++ only) against libsq_w4a16.so."""
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    inc = ce.include_paths() + [sysconfig.get_paths()["include"], os.path.join(ROCM, "include"),
+                                os.path.join(REPO_ROOT, "include")]
+    try:
+        import pybind11
+        inc.append(pybind11.get_include())
+    except ImportError:
+        pass
+    libdirs = ce.library_paths()
+    cmd = ["g++", "-O2", "-std=c++17", "-shared", "-fPIC", "-fvisibility=hidden",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=quant",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           os.path.join(CSRC, "quant_ext.cpp"), "-o", EXT_PATH]
+    cmd += ["-I" + p for p in inc]
+    cmd += ["-L" + p for p in libdirs] + ["-L" + PKG_ROOT]
+    cmd += ["-lsq_w4a16", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python"]
+    cmd += ["-Wl,-rpath,$ORIGIN"] + ["-Wl,-rpath," + p for p in libdirs]
+    _run(cmd)
+    if verbose:
+        print("built", EXT_PATH)
+    return EXT_PATH
+
+
+def build_all():
+    build_lib()
+    build_ext()
+
+
+if __name__ == "__main__":
+    what = sys.argv[1] if len(sys.argv) > 1 else "all"
+    if what == "lib":
+        build_lib()
+    elif what == "ext":
+        build_ext()
+    else:
+        build_all()

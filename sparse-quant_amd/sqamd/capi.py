@@ -1,0 +1,132 @@
+"""ctypes binding of the C ABI in include/sq_w4a16.h (libsq_w4a16.so).
+
+This is the thinnest possible host side: torch tensors are used only for device
+memory and streams; every call forwards raw pointers.  The library must already
+be built (python -m sqamd.build); loading fails loudly otherwise.
+"""
+import ctypes
+import os
+
+import torch  # noqa: F401  (loads torch's HIP runtime first so that one runtime is shared)
+
+PKG_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(PKG_ROOT, "libsq_w4a16.so")
+
+SQ_OK = 0
+SQ_ERR_NULL_POINTER, SQ_ERR_BAD_SHAPE, SQ_ERR_BAD_GROUP, SQ_ERR_BAD_LAYOUT = 1, 2, 3, 4
+SQ_ERR_BAD_ALGO, SQ_ERR_MISALIGNED, SQ_ERR_LAUNCH, SQ_ERR_WORKSPACE = 5, 6, 7, 8
+SQ_LAYOUT_L1, SQ_LAYOUT_L2 = 1, 2
+SQ_ALGO_AUTO, SQ_ALGO_GEMV, SQ_ALGO_GEMV_FIXUP, SQ_ALGO_SKINNY, SQ_ALGO_GEMM = 0, 1, 2, 3, 4
+
+_vp, _i = ctypes.c_void_p, ctypes.c_int
+
+# name -> (restype, argtypes); mirrors include/sq_w4a16.h one to one.
+SIGNATURES = {
+    "sq_version": (_i, []),
+    "sq_strerror": (ctypes.c_char_p, [_i]),
+    "sq_w4a16_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "sq_w4a16_gemm_ex": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "sq_w4a16_dequant": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "sq_transpose_merge_zeros_scales": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sq_convert_ours_to_awq": (_i, [_vp, _vp, _i, _i, _vp]),
+    "sq_convert_awq_to_lmdeploy": (_i, [_vp, _vp, _i, _i, _vp]),
+    "sq_repack_l2_to_l1": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sq_convert_2bit_to_4bit": (_i, [_vp, _vp, _i, _i, _vp]),
+}
+
+_lib = None
+
+
+class SqError(RuntimeError):
+    def __init__(self, code, what):
+        self.code = code
+        super().__init__("%s: %s (code %d)" % (what, strerror(code), code))
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libsq_w4a16.so is missing at %s: run `python -m sqamd.build` first; there is no "
+                               "fallback path" % LIB_PATH)
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def strerror(code):
+    return lib().sq_strerror(int(code)).decode()
+
+
+def _ptr(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def _stream(stream=None):
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return ctypes.c_void_p(stream.cuda_stream)
+
+
+def _check(code, what):
+    if code != SQ_OK:
+        raise SqError(code, what)
+
+
+def gemm(x, w, zs, n, k, group_size, layout=SQ_LAYOUT_L1, algo=SQ_ALGO_AUTO, out=None, stream=None):
+    """x fp16 [M,K] -> y fp16 [M,N] through sq_w4a16_gemm_ex."""
+    m = x.numel() // k
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
+    _check(lib().sq_w4a16_gemm_ex(_ptr(x), _ptr(w), _ptr(zs), _ptr(out), m, n, k, group_size, layout, algo,
+                                  _stream(stream)), "sq_w4a16_gemm_ex")
+    return out
+
+
+def dequant(w, zs, n, k, group_size, layout=SQ_LAYOUT_L1, stream=None):
+    out = torch.empty((n, k), dtype=torch.float16, device=w.device)
+    _check(lib().sq_w4a16_dequant(_ptr(w), _ptr(zs), _ptr(out), n, k, group_size, layout, _stream(stream)),
+           "sq_w4a16_dequant")
+    return out
+
+
+def transpose_merge_zeros_scales(zeros, scales, in_features, out_features, group_size, stream=None):
+    zs = torch.empty((in_features // group_size, 2 * out_features), dtype=torch.float16, device=zeros.device)
+    _check(lib().sq_transpose_merge_zeros_scales(_ptr(zeros), _ptr(scales), _ptr(zs), in_features, out_features,
+                                                 group_size, _stream(stream)), "sq_transpose_merge_zeros_scales")
+    return zs
+
+
+def convert_ours_to_awq(src, in_features, out_features, stream=None):
+    dst = torch.empty((in_features, out_features // 2), dtype=torch.uint8, device=src.device)
+    _check(lib().sq_convert_ours_to_awq(_ptr(src), _ptr(dst), in_features, out_features, _stream(stream)),
+           "sq_convert_ours_to_awq")
+    return dst
+
+
+def convert_awq_to_lmdeploy(src, in_features, out_features, stream=None):
+    dst = torch.empty((in_features, out_features // 8), dtype=torch.int32, device=src.device)
+    _check(lib().sq_convert_awq_to_lmdeploy(_ptr(src), _ptr(dst), in_features, out_features, _stream(stream)),
+           "sq_convert_awq_to_lmdeploy")
+    return dst
+
+
+def repack_l2_to_l1(w_l2, zs_l2, n, k, group_size, stream=None):
+    w1 = torch.empty((n, k // 2), dtype=torch.uint8, device=w_l2.device)
+    zs1 = torch.empty((n, 2 * (k // group_size)), dtype=torch.float16, device=w_l2.device)
+    _check(lib().sq_repack_l2_to_l1(_ptr(w_l2), _ptr(zs_l2), _ptr(w1), _ptr(zs1), n, k, group_size,
+                                    _stream(stream)), "sq_repack_l2_to_l1")
+    return w1, zs1
+
+
+def convert_2bit_to_4bit(w2, stream=None):
+    n, k4 = w2.shape
+    out = torch.empty((n, k4 * 2), dtype=torch.uint8, device=w2.device)
+    _check(lib().sq_convert_2bit_to_4bit(_ptr(w2), _ptr(out), n, k4 * 4, _stream(stream)),
+           "sq_convert_2bit_to_4bit")
+    return out

@@ -1,0 +1,84 @@
+"""WALinear: the quantized linear module the model files instantiate.
+
+Mirror of the reference's module (test/muxi/module/qlinear/qlinear.py:8-106 and
+test/nvidia/module/qlinear/qlinear.py:10-92): same constructor arguments, the same
+buffer names, shapes and dtypes (so a state_dict saved by the reference loads
+unchanged), the same forward contract `gemm_awq_ut(x, weight, zeros_scales, ...) +
+bias`.  `layout` selects which of the reference's two buffer conventions is used:
+
+    "l1" (default)  weight uint8 [N, K*w_bit/8], zeros_scales fp16 [N, 2K/g], g default 64
+    "l2"            weight int32 [K, N*w_bit/32], zeros_scales fp16 [K/g, 2N], g default 128
+"""
+import torch
+from torch import nn
+
+import quant
+from . import quant_funcs
+
+
+class WALinear(nn.Module):
+    def __init__(self, in_features, out_features, w_config=None, a_config=None, w_bit=4, a_bit=16,
+                 group_size=None, bias=True, quantize_output=False, dev="cuda", dtype=None, layout="l1"):
+        super().__init__()
+        if layout not in ("l1", "l2"):
+            raise ValueError("layout must be 'l1' or 'l2'")
+        self.in_features = in_features
+        self.out_features = out_features
+        self.w_config = w_config
+        self.a_config = a_config
+        self.w_bit = w_bit
+        self.a_bit = a_bit
+        self.layout = layout
+        self.group_size = group_size if group_size is not None else (64 if layout == "l1" else 128)
+        self.quantize_output = quantize_output
+        g = self.group_size
+        if layout == "l1":
+            self.register_buffer("zeros_scales", torch.zeros(out_features, in_features * 2 // g,
+                                                             dtype=torch.float16, device=dev))
+            self.register_buffer("weight", torch.zeros(out_features, in_features * w_bit // 8,
+                                                       dtype=dtype or torch.uint8, device=dev))
+        else:
+            self.register_buffer("zeros_scales", torch.zeros(in_features // g, out_features * 2,
+                                                             dtype=torch.float16, device=dev))
+            self.register_buffer("weight", torch.zeros(in_features, out_features * w_bit // 32,
+                                                       dtype=dtype or torch.int32, device=dev))
+        if bias:
+            self.register_buffer("bias", torch.zeros((1, out_features), dtype=torch.float16, device=dev))
+        else:
+            self.register_buffer("bias", None)
+
+    @torch.no_grad()
+    def forward(self, x):
+        weight = self.weight
+        if self.w_bit == 2:
+            if self.layout != "l1":
+                raise NotImplementedError("2-bit weights are supported in layout 'l1' only")
+            weight = quant.convert_2bit_to_4bit(weight)
+        lead = x.shape[:-1]
+        x3 = x.reshape(1, -1, x.shape[-1]) if x.dim() != 3 else x
+        y = quant.gemm_awq_ut(x3.contiguous(), weight, self.zeros_scales, x3.shape[-2], self.out_features,
+                              self.in_features, self.group_size)
+        y = y.reshape(*lead, self.out_features)
+        if self.bias is not None:
+            y = y + self.bias
+        return y
+
+    @staticmethod
+    def from_float(module, w_config, a_config=None, quantize_output=False, layout="l1"):
+        assert isinstance(module, nn.Linear)
+        n_bit, g = w_config["n_bit"], w_config["group_size"]
+        new = WALinear(module.in_features, module.out_features, w_config, a_config, w_bit=n_bit, group_size=g,
+                       bias=module.bias is not None, quantize_output=quantize_output, dev=module.weight.device,
+                       layout=layout)
+        if layout == "l1":
+            new.weight, new.zeros_scales = quant_funcs.quant_muxi(module.weight.data, module.in_features,
+                                                                  module.out_features, n_bit=n_bit, group_size=g)
+        else:
+            new.weight, new.zeros_scales = quant_funcs.quant_lmdeploy(module.weight.data, module.in_features,
+                                                                      module.out_features, group_size=g, n_bit=n_bit)
+        if module.bias is not None:
+            new.bias = module.bias.data.half().unsqueeze(0)
+        return new
+
+    def __repr__(self):
+        return "W{}A{}Linear({}, {})".format(self.w_bit, self.a_bit, self.in_features, self.out_features)
