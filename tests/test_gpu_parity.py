@@ -81,7 +81,7 @@ def test_dequant_handmade_word(capi):
 
 
 # ------------------------------------------------------------------ GEMM parity
-SMALL_SHAPES = [(64, 512, 64), (256, 1024, 128), (136, 640, 32), (48, 11008 // 4, 128)]
+SMALL_SHAPES = [(64, 512, 64), (256, 1024, 128), (136, 640, 32), (48, 2816, 128)]
 
 
 @pytest.mark.parametrize("n,k,g", SMALL_SHAPES)
@@ -145,7 +145,9 @@ def test_properties_full_size(capi, algo_name, m):
     assert torch.equal(y1, y1b)
     # scaling the activations by 2 is exact in fp16 and fp32, so the output doubles bit for bit
     y2 = capi.gemm(x * 2, d["w_dev"], d["zs_dev"], n, k, g, algo=algo)
-    assert torch.equal(y2, y1 * 2)
+    # (outputs in the fp16 subnormal range are excluded: there 2*round(a) != round(2a))
+    normal = y1.abs() >= 2.0 ** -13
+    assert torch.equal(y2[normal], (y1 * 2)[normal])
     # a one-hot activation row returns a column of W_hat, exactly
     e = torch.zeros((m, k), dtype=torch.float16, device=DEV)
     cols = [(37 * i + 5) % k for i in range(m)]
