@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""Benchmark of the W4A16 linear hot path on one MI355X.
+
+Workload (BASELINE.json configs[1], decode regime): the six W4A16 linears of one
+OPT-6.7B decoder layer -- q/k/v/out 4096x4096, fc1 4096->16384, fc2 16384->4096 --
+int4 weights in layout L1, group size 128, fp16 activations, M = 1 token.  One
+"step" is one pass over the six linears of one layer, launched back to back on one
+HIP stream through the C ABI (sq_w4a16_gemm).  Successive steps walk a pool of
+distinct layers (> 256 MB in total), so every launch streams its weights from HBM
+rather than from the Infinity Cache.
+
+The metric is achieved GB/s: algorithmic bytes of a step
+    sum over linears of  N*K/2 + (K/g)*N*4 + M*K*2 + M*N*2   (= 107 102 208 B at M = 1)
+divided by the time of a step, inputs already resident in HBM.
+
+Also printed on the same JSON line:
+  roofline      algorithmic bytes per launch / average launch duration of the decode
+                kernel (HIP events on the launch stream over the timed region) against
+                the 8 TB/s HBM peak
+  cpu_baseline  the CPU restatement of the same path (oracle/) timed on this box's
+                host cores on one step
+  prefill       TFLOP/s of the M = 2048 linears (second half of the metric)
+
+`--m`, `--group` and `--shapes` select other points of the same workload family.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+for _p in (os.path.join(REPO, "sparse-quant_amd"), os.path.join(REPO, "oracle")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_FP16_PEAK_TFLOPS = 2500.0
+OPT67_LAYER = [("q_proj", 4096, 4096), ("k_proj", 4096, 4096), ("v_proj", 4096, 4096), ("out_proj", 4096, 4096),
+               ("fc1", 16384, 4096), ("fc2", 4096, 16384)]  # (name, N, K)
+
+
+def algorithmic_bytes(m, n, k, g):
+    return n * k // 2 + (k // g) * n * 4 + m * k * 2 + m * n * 2
+
+
+def make_linear(n, k, g, dev, gen):
+    import torch
+    w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=dev, generator=gen)
+    z = torch.randint(0, 16, (n, k // g), device=dev, generator=gen).half() + 64
+    s = (torch.randn((n, k // g), device=dev, generator=gen).abs() * 0.02 + 1e-3).half()
+    zs = torch.stack([z, s], dim=-1).reshape(n, 2 * (k // g)).contiguous()
+    return w, zs
+
+
+def cpu_baseline(m, g, shapes):
+    """One step of the same workload through the oracle's C restatement (all host cores)."""
+    import numpy as np
+    import w4a16_oracle as orc
+    so = os.path.join(REPO, "oracle", "build", "libw4a16_oracle.so")
+    total_bytes = sum(algorithmic_bytes(m, n, k, g) for _, n, k in shapes)
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+    data = []
+    for idx, (_, n, k) in enumerate(shapes):
+        d = orc.synth_linear(n, k, g, seed=idx)
+        data.append((n, k, d["w_l1"], d["zs_l1"], orc.synth_x(m, k, seed=100 + idx)))
+    if os.path.exists(so):
+        lib = ctypes.CDLL(so)
+        vp = ctypes.c_void_p
+
+        def step():
+            for n, k, w, zs, x in data:
+                y = np.empty((m, n), dtype=np.float32)
+                lib.sq_oracle_gemm_l1(vp(x.ctypes.data), vp(w.ctypes.data), vp(zs.ctypes.data), vp(y.ctypes.data),
+                                      m, n, k, g)
+        kind_note = "C restatement (oracle/w4a16_oracle.c, OpenMP)"
+    else:
+        threads = 1
+
+        def step():
+            for n, k, w, zs, x in data:
+                orc.gemm_l1(x, w, zs, g)
+        kind_note = "numpy restatement (oracle/w4a16_oracle.py)"
+    step()
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[1]
+    return {"value": round(total_bytes / t / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "one step (six linears of one OPT-6.7B layer, M=%d, g=%d), median of 3, %s, %.1f ms per step"
+                      % (m, g, kind_note, t * 1e3)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--m", type=int, default=1, help="tokens per launch (decode batch)")
+    ap.add_argument("--group", type=int, default=128)
+    ap.add_argument("--layers", type=int, default=8, help="distinct layers in the rotating weight pool")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 TFLOP/s leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    from sqamd import capi
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    lib = capi.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0)
+    m, g = args.m, args.group
+    shapes = OPT67_LAYER
+
+    pool = [[make_linear(n, k, g, dev, gen) for _, n, k in shapes] for _ in range(args.layers)]
+    xs = {k: torch.randn((m, k), device=dev, generator=gen).half() for k in {k for _, _, k in shapes}}
+    ys = {n: torch.empty((m, n), dtype=torch.float16, device=dev) for n in {n for _, n, _ in shapes}}
+    bytes_per_step = sum(algorithmic_bytes(m, n, k, g) for _, n, k in shapes)
+    launches_per_step = len(shapes)
+
+    stream = torch.cuda.Stream(device=dev)
+    vp = ctypes.c_void_p
+    st = vp(stream.cuda_stream)
+    calls = []
+    for layer in pool:
+        row = []
+        for (w, zs), (_, n, k) in zip(layer, shapes):
+            row.append((vp(xs[k].data_ptr()), vp(w.data_ptr()), vp(zs.data_ptr()), vp(ys[n].data_ptr()), m, n, k, g,
+                        capi.SQ_LAYOUT_L1, st))
+        calls.append(row)
+    gemm = lib.sq_w4a16_gemm
+
+    def run_layer(i):
+        for a in calls[i % len(calls)]:
+            rc = gemm(*a)
+            if rc != 0:
+                raise RuntimeError("sq_w4a16_gemm failed: " + capi.strerror(rc))
+
+    with torch.cuda.stream(stream):
+        for i in range(len(calls)):
+            run_layer(i)
+        stream.synchronize()
+        graph = None
+        if not args.no_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(len(calls)):
+                    run_layer(i)
+        per_replay = len(calls)
+
+        def run_steps(count):
+            if graph is None:
+                for i in range(count):
+                    run_layer(i)
+                return count
+            reps = (count + per_replay - 1) // per_replay
+            for _ in range(reps):
+                graph.replay()
+            return reps * per_replay
+
+        run_steps(args.warmup)
+        stream.synchronize()
+        steps = args.steps if graph is None else ((args.steps + per_replay - 1) // per_replay) * per_replay
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        done = run_steps(steps)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        assert done == steps
+    wall_ms = (t1 - t0) * 1e3
+    gpu_ms = e0.elapsed_time(e1)
+    ms_per_step = wall_ms / steps
+    value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
+    launch_us = gpu_ms * 1e3 / (steps * launches_per_step)
+    achieved = (bytes_per_step / launches_per_step) / (launch_us * 1e-6) / 1e9
+
+    traffic = None
+    tfile = os.path.join(REPO, "profiles", "gemv_decode_traffic.json")
+    if os.path.exists(tfile) and m == 1 and g == 128:
+        try:
+            traffic = json.load(open(tfile)).get("hbm_bytes_per_launch")
+        except Exception:
+            traffic = None
+
+    out = {
+        "metric": "W4A16 linear GB/s at M=1 (OPT-6.7B decoder-layer linears, cold weights)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int4 weights x fp16 activations, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "OPT-6.7B decoder-layer linears (q,k,v,out 4096x4096; fc1 4096->16384; fc2 "
+                               "16384->4096), W4A16 group %d, M=%d, one step = six launches, %d-layer rotating "
+                               "weight pool (%.0f MB)" % (g, m, args.layers, args.layers * bytes_per_step / 1e6),
+                   "launch": "hip-graph replay" if graph is not None else "eager", "bytes_per_step": bytes_per_step},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "kernel": "sq::gemv2_kernel (decode GEMV)", "avg_launch_us": round(launch_us, 3),
+                     "bytes_per_launch": bytes_per_step // launches_per_step},
+    }
+
+    if not args.no_prefill:
+        out["prefill"] = prefill_leg(torch, capi, pool[0], shapes, g, dev, gen, stream)
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(m, g, shapes)
+    print(json.dumps(out))
+
+
+def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10):
+    """TFLOP/s of the M=2048 linears of the same layer (BASELINE.json configs[2])."""
+    res = {}
+    flops_total, time_total = 0.0, 0.0
+    with torch.cuda.stream(stream):
+        for (w, zs), (name, n, k) in list(zip(layer, shapes))[3:]:
+            x = torch.randn((m, k), device=dev, generator=gen).half()
+            y = torch.empty((m, n), dtype=torch.float16, device=dev)
+            for _ in range(3):
+                capi.gemm(x, w, zs, n, k, g, out=y, stream=stream)
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(reps):
+                capi.gemm(x, w, zs, n, k, g, out=y, stream=stream)
+            e1.record(stream)
+            stream.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / reps
+            fl = 2.0 * m * n * k
+            res[name] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 1)}
+            flops_total += fl
+            time_total += us
+    tf = flops_total / time_total / 1e6
+    return {"m": m, "tflops": round(tf, 1), "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
+            "per_linear": res}
+
+
+if __name__ == "__main__":
+    main()

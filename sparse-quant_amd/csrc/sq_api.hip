@@ -74,8 +74,11 @@ int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y, int 
         case SQ_ALGO_GEMV:
         case SQ_ALGO_GEMV_FIXUP:
             if (M > 8) return SQ_ERR_BAD_ALGO;
-            return launch_code(sq::launch_gemv_tuned(x, w, zs, y, M, N, K, group_size,
-                                                     kernel == SQ_ALGO_GEMV_FIXUP, tune, st));
+            if (tune & 0x8000)
+                return launch_code(sq::launch_gemv_tuned(x, w, zs, y, M, N, K, group_size,
+                                                         kernel == SQ_ALGO_GEMV_FIXUP, tune & 0x7FFF, st));
+            return launch_code(sq::launch_gemv2_tuned(x, w, zs, y, M, N, K, group_size,
+                                                      kernel == SQ_ALGO_GEMV_FIXUP, tune, st));
         case SQ_ALGO_SKINNY:
             if (M > 64) return SQ_ERR_BAD_ALGO;
             return launch_code(sq::launch_skinny_tuned(x, w, zs, y, M, N, K, group_size, tune, st));

@@ -72,6 +72,25 @@ __device__ __forceinline__ float row_sum_stride4(float v) {
     return v;
 }
 
+// Sum over the four lanes of a quad (lanes 4q .. 4q+3), result in every lane.
+__device__ __forceinline__ float quad_sum(float v) {
+    v += bit_cast<float>(__builtin_amdgcn_update_dpp(0, bit_cast<int>(v), 0xB1, 0xF, 0xF, false));  // quad_perm 1,0,3,2
+    v += bit_cast<float>(__builtin_amdgcn_update_dpp(0, bit_cast<int>(v), 0x4E, 0xF, 0xF, false));  // quad_perm 2,3,0,1
+    return v;
+}
+
+// Broadcast lane T of every quad to the four lanes of that quad (128-bit value).
+template <int T>
+__device__ __forceinline__ u32x4_t quad_bcast(u32x4_t v) {
+    constexpr int ctrl = T * 0x55;  // quad_perm T,T,T,T
+    u32x4_t r;
+    r.x = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v.x, ctrl, 0xF, 0xF, false);
+    r.y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v.y, ctrl, 0xF, 0xF, false);
+    r.z = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v.z, ctrl, 0xF, 0xF, false);
+    r.w = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v.w, ctrl, 0xF, 0xF, false);
+    return r;
+}
+
 __device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
 
 }  // namespace sq

@@ -64,29 +64,49 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const uint8_t* __restrict__ 
             wq[rs] = __builtin_nontemporal_load((const u32x4_t*)(W + (long)row * (K >> 1) + (kc >> 1)));
             zsv[rs] = ZS[(long)row * groups + (kc >> gshift)];
         }
-        // Activations of the 32 k of this block for token min(4*mt+i, M-1).
+        // Activations of the 32 k of this block.
         u32x4_t xa[MT][4];
-#pragma unroll
-        for (int mt = 0; mt < MT; mt++) {
-            const int m = imin(4 * mt + i, M - 1);
-            const u32x4_t* xp = (const u32x4_t*)(X + (long)m * K + kc);
-#pragma unroll
-            for (int t = 0; t < 4; t++) {
-                u32x4_t v = xp[t];
-                xa[mt][t] = kvalid ? v : (u32x4_t){0u, 0u, 0u, 0u};
-            }
-        }
-
         float4_t xs[MT];
-        if (FIXUP) {
+        if (MROWS == 1) {
+            // One token: the four lanes of a block need the same 64 bytes.  Each
+            // loads a different quarter (so the wave reads the slice's 1 KiB once,
+            // fully coalesced) and the quarters are exchanged with DPP quad
+            // broadcasts; every row of A then holds token 0.
+            const u32x4_t own = *(const u32x4_t*)(X + kc + 8 * i);
+            const u32x4_t xv = kvalid ? own : (u32x4_t){0u, 0u, 0u, 0u};
+            xa[0][0] = quad_bcast<0>(xv);
+            xa[0][1] = quad_bcast<1>(xv);
+            xa[0][2] = quad_bcast<2>(xv);
+            xa[0][3] = quad_bcast<3>(xv);
+            if (FIXUP) {
+                const half8_t h = bit_cast<half8_t>(xv);
+                float sum = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) sum += (float)h[e];
+                sum = quad_sum(sum);
+                xs[0] = (float4_t){sum, sum, sum, sum};
+            }
+        } else {
 #pragma unroll
             for (int mt = 0; mt < MT; mt++) {
-                xs[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                const int m = imin(4 * mt + i, M - 1);
+                const u32x4_t* xp = (const u32x4_t*)(X + (long)m * K + kc);
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    const half8_t xv = bit_cast<half8_t>(xa[mt][t]);
-                    xs[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xv.lo, ones, xs[mt], 0, 0, 0);
-                    xs[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xv.hi, ones, xs[mt], 0, 0, 0);
+                    u32x4_t v = xp[t];
+                    xa[mt][t] = kvalid ? v : (u32x4_t){0u, 0u, 0u, 0u};
+                }
+            }
+            if (FIXUP) {
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    xs[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const half8_t xv = bit_cast<half8_t>(xa[mt][t]);
+                        xs[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xv.lo, ones, xs[mt], 0, 0, 0);
+                        xs[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xv.hi, ones, xs[mt], 0, 0, 0);
+                    }
                 }
             }
         }

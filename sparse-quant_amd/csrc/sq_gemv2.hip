@@ -1,0 +1,254 @@
+// Decode GEMV / very skinny GEMM (M <= 8) for layout L1, streaming formulation.
+// HBM-bandwidth bound: algorithmic bytes = N*K/2 + (K/g)*N*4 + M*K*2 + M*N*2.
+//
+// Mapping.  v_mfma_f32_4x4x4_16B_f16 multiplies 16 independent 4x4x4 blocks; in
+// block b lane 4b+i supplies row i of A (4 k) and column i of B (4 k) and receives
+// D[0..3][i].  With A = activations (row = token) and B = weights (column = output
+// row) every lane accumulates its own output row over its own k for up to 4
+// tokens, and the matrix core does every multiply-add; the VALU only unpacks.
+//
+// A workgroup is NR x KS waves: wave (r, q) owns the 4 output rows r0 + 4r .. +3
+// and the q-th of KS contiguous ranges of 512-wide k-steps.  In k-step s lane
+// 4b+i loads the 128-bit word with k = 512*s + 32*b .. +31 of its row, so one
+// wave-wide load covers 4 rows x 256 contiguous bytes, and all (up to S) loads of
+// a round are issued back to back before anything is consumed.  The activations
+// of the round (and, for the fixup mode, their sums over each run of 32 k) are
+// staged once per workgroup in LDS with row pitch 1 KiB * S + 16 bytes, which
+// puts the 64 lanes of a 128-bit read on 64 distinct 16-byte slots.  A lane's sum
+// over its 16 blocks is folded with DPP row rotations and two cross-row shuffles;
+// the KS partial sums of a row meet in LDS once, at the end.
+//
+// Arithmetic modes (both accumulate in fp32):
+//   exact : B = fp16((q - z) * s), bit-identical to the reference's W_hat.
+//   fixup : B = 64 + q (bit pattern only); per run of 32 k the lane adds
+//           s * (sum x*(64+q) - (64+z) * sum x): zero and scale are applied once per
+//           run in fp32 instead of once per weight in fp16.
+// (replaces w4a16_bs1_kernel / w4a16_bs2_kernel, reference:
+// quantization/muxi/backend/w4a16_gemm.cuh:14-151,153-326)
+#include "sq_common.h"
+#include "sq_kernels.h"
+
+namespace sq {
+
+template <int MROWS, int NR, int KS, int S, bool FIXUP>
+__global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __restrict__ W,
+                                                             const half2_t* __restrict__ ZS,
+                                                             const half_t* __restrict__ X,
+                                                             half_t* __restrict__ Y, int M, int N, int K,
+                                                             int gshift) {
+    constexpr int MT = (MROWS + 3) / 4;
+    constexpr int PITCH = 1024 * S + 16;                 // bytes per staged activation row
+    constexpr int NT = 64 * NR * KS;
+    constexpr int STAGE_TOTAL = KS * MROWS * S * 64;     // 128-bit words staged per round
+    constexpr int STAGE_PER_THREAD = (STAGE_TOTAL + NT - 1) / NT;
+
+    __shared__ __attribute__((aligned(16))) uint8_t xbuf[KS][MROWS * PITCH];
+    __shared__ __attribute__((aligned(16))) float xsum[KS][S * 16][MROWS];
+    __shared__ float red[KS][NR][MROWS][4];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wr = wave % NR;   // row group of this wave
+    const int wq_ = wave / NR;  // k range of this wave
+    const int i = lane & 3;
+    const int b = lane >> 2;
+    const int out_row = blockIdx.x * (4 * NR) + 4 * wr + i;
+    const int row = imin(out_row, N - 1);
+    const int groups = K >> gshift;
+    const int nsteps = (K + 511) >> 9;
+    const int spw = (nsteps + KS - 1) / KS;  // k-steps per wave
+    const int rounds = (spw + S - 1) / S;
+    const uint8_t* wrow = W + (long)row * (K >> 1);
+    const half2_t* zrow = ZS + (long)row * groups;
+
+    float4_t acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; mt++) acc[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+    for (int rnd = 0; rnd < rounds; rnd++) {
+        // Stage the activations of this round for all KS ranges: word idx covers
+        // range q = idx / (MROWS*S*64), token m, k-step j = (idx / 64) % S.
+        u32x4_t xr[STAGE_PER_THREAD];
+#pragma unroll
+        for (int p = 0; p < STAGE_PER_THREAD; p++) {
+            const int idx = tid + p * NT;
+            const int q = idx / (MROWS * S * 64);
+            const int m = (idx / (S * 64)) % MROWS;
+            const int w8 = idx % (S * 64);  // 128-bit word inside the staged row
+            const int j = rnd * S + (w8 >> 6);
+            const int k = (q * spw + j) * 512 + (w8 & 63) * 8;
+            const bool ok = (idx < STAGE_TOTAL) && (m < M) && (j < spw) && (k < K);
+            const u32x4_t v = *(const u32x4_t*)(X + (ok ? (long)m * K + k : 0));
+            xr[p] = ok ? v : (u32x4_t){0u, 0u, 0u, 0u};
+        }
+        // The weight stream of this round; a k-step outside the wave's range or
+        // past K reads a valid address and meets zero activations (the host picks S and
+        // KS so that this is rare).
+        u32x4_t wq[S];
+        half2_t zq[S];
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+            const int j = rnd * S + s;
+            const int kk = (wq_ * spw + j) * 512 + 32 * b;
+            const int kc = (j < spw && kk < K) ? kk : 0;
+            wq[s] = __builtin_nontemporal_load((const u32x4_t*)(wrow + (kc >> 1)));
+            zq[s] = zrow[kc >> gshift];
+        }
+        if (rnd > 0) __syncthreads();  // everyone is done reading the previous round
+#pragma unroll
+        for (int p = 0; p < STAGE_PER_THREAD; p++) {
+            const int idx = tid + p * NT;
+            const int q = idx / (MROWS * S * 64);
+            const int m = (idx / (S * 64)) % MROWS;
+            const int w8 = idx % (S * 64);
+            if (idx < STAGE_TOTAL) *(u32x4_t*)(&xbuf[q][m * PITCH + w8 * 16]) = xr[p];
+            if (FIXUP) {
+                const half8_t h = bit_cast<half8_t>(xr[p]);
+                float sum = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) sum += (float)h[e];
+                sum = quad_sum(sum);
+                if ((tid & 3) == 0 && idx < STAGE_TOTAL) xsum[q][w8 >> 2][m] = sum;
+            }
+        }
+        __syncthreads();
+
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+            half8_t xa[MT][4];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) {
+                const int m = (4 * mt + i) & (MROWS - 1);
+                const uint8_t* xp = &xbuf[wq_][m * PITCH + (512 * s + 32 * b) * 2];
+#pragma unroll
+                for (int t = 0; t < 4; t++) xa[mt][t] = *(const half8_t*)(xp + 16 * t);
+            }
+            const half2_t p = zq[s];
+            if (!FIXUP) {
+                const half2_t z64 = {p.x, p.x};
+                const half2_t sc = {p.y, p.y};
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const half8_t wv = dequant8(wq[s][t], z64, sc);
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        acc[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, wv.lo, acc[mt], 0, 0, 0);
+                        acc[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].hi, wv.hi, acc[mt], 0, 0, 0);
+                    }
+                }
+            } else {
+                float4_t tmp[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) tmp[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const half8_t wv = unpack8_raw(wq[s][t]);
+#pragma unroll
+                    for (int mt = 0; mt < MT; mt++) {
+                        tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, wv.lo, tmp[mt], 0, 0, 0);
+                        tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].hi, wv.hi, tmp[mt], 0, 0, 0);
+                    }
+                }
+                const float zf = (float)p.x;
+                const float sf = (float)p.y;
+                const float* xs = &xsum[wq_][16 * s + b][0];
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (4 * mt + j < MROWS) acc[mt][j] += sf * (tmp[mt][j] - zf * xs[4 * mt + j]);
+            }
+        }
+    }
+
+    // Fold the 16 blocks of the wave: DPP inside each 16-lane row, shuffles across
+    // rows; then the KS ranges of a row through LDS.
+#pragma unroll
+    for (int m = 0; m < MROWS; m++) {
+        float v = row_sum_stride4(acc[m >> 2][m & 3]);
+        v += __shfl_xor(v, 16);
+        v += __shfl_xor(v, 32);
+        if (KS == 1) {
+            if (lane < 4 && out_row < N && m < M) Y[(long)m * N + out_row] = (half_t)v;
+        } else if (lane < 4) {
+            red[wq_][wr][m][i] = v;
+        }
+    }
+    if (KS > 1) {
+        __syncthreads();
+        if (tid < NR * MROWS * 4) {
+            const int ri = tid & 3;
+            const int m = (tid >> 2) % MROWS;
+            const int r = (tid >> 2) / MROWS;
+            float sum = 0.f;
+#pragma unroll
+            for (int q = 0; q < KS; q++) sum += red[q][r][m][ri];
+            const int orow = blockIdx.x * (4 * NR) + 4 * r + ri;
+            if (orow < N && m < M) Y[(long)m * N + orow] = (half_t)sum;
+        }
+    }
+}
+
+template <int MROWS, int NR, int KS, int S>
+static hipError_t launch_cfg(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int gshift,
+                             bool fixup, hipStream_t st) {
+    const dim3 grid((N + 4 * NR - 1) / (4 * NR));
+    if (fixup)
+        hipLaunchKernelGGL((gemv2_kernel<MROWS, NR, KS, S, true>), grid, dim3(64 * NR * KS), 0, st, (const uint8_t*)w,
+                           (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift);
+    else
+        hipLaunchKernelGGL((gemv2_kernel<MROWS, NR, KS, S, false>), grid, dim3(64 * NR * KS), 0, st,
+                           (const uint8_t*)w, (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift);
+    return hipGetLastError();
+}
+
+// Staged activations are kept under 48 KiB of LDS: KS * MROWS * S KiB.
+template <int MROWS, int S>
+static hipError_t launch_steps(int nr, int ks, const void* x, const void* w, const void* zs, void* y, int M, int N,
+                               int K, int gshift, bool fixup, hipStream_t st) {
+    constexpr int KS_MAX = 48 / (MROWS * S) >= 4 ? 4 : (48 / (MROWS * S) >= 2 ? 2 : 1);
+    if (ks > KS_MAX) ks = KS_MAX;
+    while (nr * ks > 16) nr >>= 1;
+#define SQ_CASE(NR_, KS_)                                                                    \
+    if (nr == NR_ && ks == KS_) {                                                           \
+        if constexpr (KS_ <= KS_MAX)                                                        \
+            return launch_cfg<MROWS, NR_, KS_, S>(x, w, zs, y, M, N, K, gshift, fixup, st); \
+    }
+    SQ_CASE(2, 1) SQ_CASE(4, 1) SQ_CASE(8, 1)
+    SQ_CASE(2, 2) SQ_CASE(4, 2) SQ_CASE(8, 2)
+    SQ_CASE(2, 4) SQ_CASE(4, 4)
+#undef SQ_CASE
+    return launch_cfg<MROWS, 4, 1, S>(x, w, zs, y, M, N, K, gshift, fixup, st);
+}
+
+template <int MROWS>
+static hipError_t launch_rows(int nr, int ks, int steps, const void* x, const void* w, const void* zs, void* y,
+                              int M, int N, int K, int gshift, bool fixup, hipStream_t st) {
+    constexpr int S_MAX = (MROWS >= 4) ? 4 : 8;
+    if (steps >= 8 && S_MAX >= 8) return launch_steps<MROWS, S_MAX>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, st);
+    if (steps >= 4) return launch_steps<MROWS, 4>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, st);
+    return launch_steps<MROWS, 2>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, st);
+}
+
+// tune = 0 for the built-in heuristic, else (row groups per workgroup: 2,4,8) |
+// (k ranges per workgroup: 1,2,4) << 4.  A workgroup covers 4 * row groups rows; the
+// number of k-steps a wave issues per round (2, 4 or 8) follows from K and the k ranges.
+hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
+                              bool fixup, int tune, hipStream_t st) {
+    int gshift = 0;
+    while ((1 << gshift) < g) gshift++;
+    int nr = tune & 0xF, ks = (tune >> 4) & 0xF;
+    const int nsteps = (K + 511) / 512;
+    // Measured on MI355X (cold weights, M = 1): K = 16384 wants 4 k ranges x 2 row groups,
+    // 16384 x 4096 wants 2 x 4, 4096 x 4096 wants 1 x 4.
+    if (ks != 1 && ks != 2 && ks != 4) ks = nsteps > 16 ? 4 : (((long)N * K >= (1L << 25) && nsteps >= 8) ? 2 : 1);
+    if (nr != 2 && nr != 4 && nr != 8) nr = ks == 4 ? 2 : 4;
+    const int spw = (nsteps + ks - 1) / ks;
+    if (M <= 1) return launch_rows<1>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, st);
+    if (M <= 2) return launch_rows<2>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, st);
+    if (M <= 4) return launch_rows<4>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, st);
+    return launch_rows<8>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, st);
+}
+
+}  // namespace sq

@@ -24,6 +24,9 @@ hipError_t launch_2bit_to_4bit(const void* src, void* dst, int N, int K, hipStre
 // sq_gemv.hip: M <= 8.  tune = row steps per workgroup (1,2,4) | waves << 8.
 hipError_t launch_gemv_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
                              bool fixup, int tune, hipStream_t st);
+// sq_gemv2.hip: M <= 8, streaming formulation.  tune = waves per workgroup (1,2,4,8).
+hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
+                              bool fixup, int tune, hipStream_t st);
 // sq_skinny.hip: M <= 64.  tune = waves | mode << 8 (mode 1 = exact, 2 = fixup).
 hipError_t launch_skinny_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
                                int tune, hipStream_t st);
