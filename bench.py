@@ -106,6 +106,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 TFLOP/s leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch plain device copies of 256 MiB (reads 256 MiB, writes 256 MiB): the known-size "
+                         "kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -211,6 +214,14 @@ def main():
                      "bytes_per_launch": bytes_per_step // launches_per_step},
     }
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        out["calibration"] = {"kernel": "torch elementwise copy", "bytes_read": 256 << 20, "bytes_written": 256 << 20,
+                              "launches": 5}
     if not args.no_prefill:
         out["prefill"] = prefill_leg(torch, capi, pool[0], shapes, g, dev, gen, stream)
     if not args.no_cpu:

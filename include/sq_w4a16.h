@@ -55,9 +55,11 @@ const char* sq_strerror(int code);
  * accumulation.  Replaces the body of gemm_awq_ut / Gemm_awq_pure
  * (reference: quantization/muxi/backend/gemm_quant.cu:12-59,84-109;
  * quantization/nvidia/kernel/gemm_quant.cu:13-40,98-123).
- * Requirements: M >= 1; N % 8 == 0; K % 32 == 0; K % g == 0; g in {32,64,128}
- * for L1 (g == 128 for L2, plus K % 32 == 0 and N % 32 == 0); x, w, zs, y
- * 16-byte aligned.  M == 0 is accepted and launches nothing. */
+ * Requirements: N % 8 == 0; K % 32 == 0; K % g == 0; g in {32,64,128}; x, w, zs,
+ * y 16-byte aligned.  M == 0 is accepted and launches nothing.  The kernels
+ * consume layout L1; for SQ_LAYOUT_L2 the call returns SQ_ERR_BAD_LAYOUT: convert
+ * the weight once with sq_repack_l2_to_l1 (the `quant` extension does this behind
+ * gemm_awq_ut and caches the result for the life of the source tensor). */
 int sq_w4a16_gemm(const void* x, const void* w, const void* zs, void* y,
                   int M, int N, int K, int group_size, int layout, void* stream);
 
