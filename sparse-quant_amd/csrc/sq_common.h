@@ -20,44 +20,62 @@ __device__ __forceinline__ To bit_cast(const From& v) {
     return __builtin_bit_cast(To, v);
 }
 
+// The two nibble masks, pinned in VGPRs: on gfx9-family encodings a VOP3
+// instruction takes no literal and at most one scalar operand, so
+// (w & mask) | magic becomes a single v_and_or_b32 only with the mask in a VGPR
+// and the magic number in an SGPR.
+struct NibbleMasks {
+    uint32_t lo, hi;
+};
+__device__ __forceinline__ NibbleMasks nibble_masks() {
+    NibbleMasks m = {0x000F000Fu, 0x00F000F0u};
+    asm("" : "+v"(m.lo));
+    asm("" : "+v"(m.hi));
+    return m;
+}
+
 // One packed word (layout L1: nibbles k0,k2,k4,k6,k1,k3,k5,k7 from the least
 // significant) -> four half2 bit patterns holding 64 + q for (k0,k1), (k2,k3),
 // (k4,k5), (k6,k7).  0x5400 is fp16 64.0 and ulp(64) = 1/16, so a nibble placed
 // in mantissa bits 4..7 adds exactly its value.
 // (reference: quantization/muxi/backend/utils.cuh:81-134)
-__device__ __forceinline__ void unpack8_bias64(uint32_t w, uint32_t h[4]) {
+__device__ __forceinline__ void unpack8_bias64(uint32_t w, uint32_t h[4], const NibbleMasks& nm) {
     const uint32_t t = w >> 8;
-    h[0] = ((w & 0x000F000Fu) | 0x05400540u) << 4;
-    h[1] = (w & 0x00F000F0u) | 0x54005400u;
-    h[2] = ((t & 0x000F000Fu) | 0x05400540u) << 4;
-    h[3] = (t & 0x00F000F0u) | 0x54005400u;
+    h[0] = ((w & nm.lo) | 0x05400540u) << 4;
+    h[1] = (w & nm.hi) | 0x54005400u;
+    h[2] = ((t & nm.lo) | 0x05400540u) << 4;
+    h[3] = (t & nm.hi) | 0x54005400u;
 }
 
 // (h - z64) * s on a half2, each operation rounded once in fp16: the difference
 // of two values in [64,79] is exact, so the result is the correctly rounded
 // (q - z) * s.  (reference: quantization/muxi/backend/w4a16_gemm.cuh:58-81)
-__device__ __forceinline__ uint32_t dequant_pair(uint32_t h, half2_t z64, half2_t s) {
+__device__ __forceinline__ uint32_t dequant_pair(uint32_t h, half2_t zb, half2_t s) {
     half2_t v = bit_cast<half2_t>(h);
-    v = (v - z64) * s;
+    v = (v - zb) * s;
     return bit_cast<uint32_t>(v);
 }
 
-// Word -> 8 dequantised fp16 (natural k order) as one 128-bit value.
-__device__ __forceinline__ half8_t dequant8(uint32_t w, half2_t z64, half2_t s) {
-    uint32_t h[4];
-    unpack8_bias64(w, h);
+// Word -> 8 dequantised fp16 (natural k order) as one 128-bit value, bit-identical
+// to fp16 (q - z) * s.  Low nibbles are unpacked without a shift as 1024 + q
+// (magic 0x6400), high nibbles as 64 + q (magic 0x5400); the stored zero 64 + z is
+// used as is for the high ones and as 1024 + z (= stored zero + 960, exact in fp16)
+// for the low ones, so both differences are the exact integer q - z.
+__device__ __forceinline__ half8_t dequant8(uint32_t w, half2_t z64, half2_t s, const NibbleMasks& nm) {
+    const half2_t z1024 = z64 + (half2_t){(half_t)960.f, (half_t)960.f};
+    const uint32_t t = w >> 8;
     u32x4_t r;
-    r.x = dequant_pair(h[0], z64, s);
-    r.y = dequant_pair(h[1], z64, s);
-    r.z = dequant_pair(h[2], z64, s);
-    r.w = dequant_pair(h[3], z64, s);
+    r.x = dequant_pair((w & nm.lo) | 0x64006400u, z1024, s);
+    r.y = dequant_pair((w & nm.hi) | 0x54005400u, z64, s);
+    r.z = dequant_pair((t & nm.lo) | 0x64006400u, z1024, s);
+    r.w = dequant_pair((t & nm.hi) | 0x54005400u, z64, s);
     return bit_cast<half8_t>(r);
 }
 
 // Word -> 8 fp16 holding 64 + q (no zero / scale applied).
-__device__ __forceinline__ half8_t unpack8_raw(uint32_t w) {
+__device__ __forceinline__ half8_t unpack8_raw(uint32_t w, const NibbleMasks& nm) {
     uint32_t h[4];
-    unpack8_bias64(w, h);
+    unpack8_bias64(w, h, nm);
     u32x4_t r = {h[0], h[1], h[2], h[3]};
     return bit_cast<half8_t>(r);
 }

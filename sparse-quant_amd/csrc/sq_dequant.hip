@@ -13,6 +13,7 @@ __global__ __launch_bounds__(256) void dequant_l1_kernel(const uint32_t* __restr
                                                          const half2_t* __restrict__ zs,
                                                          half8_t* __restrict__ out, int K8, int gshift8,
                                                          int groups, long total_words) {
+    const NibbleMasks nm = nibble_masks();
     const long stride = (long)gridDim.x * blockDim.x;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total_words; i += stride) {
         const int n = (int)(i / K8);
@@ -21,7 +22,7 @@ __global__ __launch_bounds__(256) void dequant_l1_kernel(const uint32_t* __restr
         const half2_t p = zs[(long)n * groups + (k8 >> gshift8)];
         const half2_t z64 = {p.x, p.x};
         const half2_t s = {p.y, p.y};
-        __builtin_nontemporal_store(dequant8(word, z64, s), out + i);
+        __builtin_nontemporal_store(dequant8(word, z64, s, nm), out + i);
     }
 }
 

@@ -10,9 +10,9 @@
 //     reference's W_hat).  Its four 32-bit words are exactly the B operands of the
 //     four MFMA k-steps, so the weights never pass through LDS and no wave repeats
 //     another wave's dequantisation;
-//   * activations: the BM x 64 tile goes global -> registers -> LDS (double
-//     buffered, row pitch 144 B so that 128-bit reads are bank-conflict free) and
-//     every wave reads its A operands with ds_read_b128; lane (l%32, l/32) reads
+//   * activations: the BM x 64 tile goes global -> registers (three K steps ahead) ->
+//     LDS (double buffered, XOR-swizzled 16-byte chunks so that 128-bit reads are
+//     bank-conflict free) and every wave reads its A operands with ds_read_b128; lane (l%32, l/32) reads
 //     x[m0 + 32*mi + l%32][k0 + 32*(l/32) + 8*t .. +7], the same k the weight
 //     operand of that lane holds.
 // One barrier per K step.  D[m][n]: lane = n%32 + 32*((m/4)%2), register =
@@ -23,19 +23,30 @@
 #include "sq_common.h"
 #include "sq_kernels.h"
 
+#include <type_traits>
+
 namespace sq {
 
 constexpr int GEMM_BN = 256;
 constexpr int GEMM_BK = 64;
-constexpr int GEMM_PITCH = 72;  // halves per LDS row (64 + 8 padding)
+constexpr int GEMM_STAGES = 3;  // register stages; loads run GEMM_STAGES - 1 steps ahead
 
+__device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+// Two waves per SIMD (two workgroups per CU): one wave alone cannot both issue the
+// unpack / LDS / load instructions of a step and keep the matrix pipe full.
 template <int MI>
-__global__ __launch_bounds__(256) void gemm_kernel(const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS,
                                                    const half_t* __restrict__ X, half_t* __restrict__ Y, int M,
                                                    int N, int K, int gshift) {
     constexpr int BM = 32 * MI;
-    __shared__ __attribute__((aligned(16))) half_t xs[2][BM * GEMM_PITCH];
+    // Activation tile, two stages, row pitch 128 B (64 halves, no padding); the eight
+    // 16-byte chunks of row R are stored at chunk position c ^ swz(R); 8 consecutive
+    // rows then use 8 distinct positions and 16 consecutive rows 16 distinct 16-byte
+    // slots of a 256-byte bank period, so the 128-bit operand reads are conflict free.
+    __shared__ __attribute__((aligned(1024))) uint8_t xs[2][BM * 128];
 
+    const NibbleMasks nm = nibble_masks();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -46,17 +57,18 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint8_t* __restrict__ W
     const int groups = K >> gshift;
     const int nit = (K + GEMM_BK - 1) / GEMM_BK;
 
-    // Global -> LDS staging of the activation tile: thread t moves, per pass p, the
-    // 16 bytes at row 32*p + t/8, halves (t%8)*8 .. +7.
-    const int xr = tid >> 3;
-    const int xc = (tid & 7) * 8;
+    // Global -> registers -> LDS staging of the activation tile.  Pass p of wave w moves
+    // rows 32*p + 8*w .. +7; lane l = 8*r + c' fetches the chunk that belongs at
+    // position c' of row R = 32*p + 8*w + r, so a wave writes 1 KiB of contiguous LDS.
+    // Rows past M are clamped to row M-1: they only feed output rows that are never
+    // stored.
     const half_t* xsrc[MI];
-    bool xrow_ok[MI];
+    int xchunk[MI];
 #pragma unroll
     for (int p = 0; p < MI; p++) {
-        const int m = m0 + 32 * p + xr;
-        xrow_ok[p] = m < M;
-        xsrc[p] = X + (long)imin(m, M - 1) * K + xc;
+        const int R = 32 * p + 8 * wave + (lane >> 3);
+        xchunk[p] = ((lane & 7) ^ swz(R)) * 8;
+        xsrc[p] = X + (long)imin(m0 + R, M - 1) * K;
     }
 
     const uint8_t* wsrc[2];
@@ -76,62 +88,102 @@ __global__ __launch_bounds__(256) void gemm_kernel(const uint8_t* __restrict__ W
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[mi][ni][v] = 0.f;
 
-    u32x4_t xreg[MI];
-    u32x4_t wq[2];
-    half2_t zq[2];
+    // All loads are unconditional: a k past the end is clamped to the last valid 8
+    // halves / 32 nibbles and the scale of those lanes is replaced by 0, which zeroes
+    // their weight operand.
+    struct WStage {
+        u32x4_t q[2];
+        half2_t zs[2];
+    };
+    WStage w[GEMM_STAGES];
+    u32x4_t xr[GEMM_STAGES][MI];
 
-    auto load_tile = [&](int it) {
-        const int k0 = it * GEMM_BK;
+    auto load_x = [&](int it, u32x4_t (&dst)[MI]) {
 #pragma unroll
         for (int p = 0; p < MI; p++) {
-            const bool ok = xrow_ok[p] && (k0 + xc < K);
-            const u32x4_t v = *(const u32x4_t*)(xsrc[p] + (ok ? k0 : 0));
-            xreg[p] = ok ? v : (u32x4_t){0u, 0u, 0u, 0u};
+            const int kx = imin(it * GEMM_BK + xchunk[p], K - 8);
+            dst[p] = *(const u32x4_t*)(xsrc[p] + kx);
         }
-        const int kw = k0 + 32 * lc;
-        const int kc = kw < K ? kw : 0;  // past-the-end k meets zero activations
+    };
+    auto store_x = [&](int buf, const u32x4_t (&src)[MI]) {
+#pragma unroll
+        for (int p = 0; p < MI; p++) *(u32x4_t*)(&xs[buf][(32 * p + 8 * wave) * 128 + lane * 16]) = src[p];
+    };
+    auto load_w = [&](int it, WStage& ws) {
+        const int kc = imin(it * GEMM_BK + 32 * lc, K - 32);
 #pragma unroll
         for (int ni = 0; ni < 2; ni++) {
-            wq[ni] = *(const u32x4_t*)(wsrc[ni] + (kc >> 1));
-            zq[ni] = zsrc[ni][kc >> gshift];
+            ws.q[ni] = *(const u32x4_t*)(wsrc[ni] + (kc >> 1));
+            ws.zs[ni] = zsrc[ni][kc >> gshift];
         }
     };
-    auto store_tile = [&](int buf) {
+
+    // Operand read offsets: lane (ln, lc) reads row 32*mi + ln, chunk 4*lc + t.
+    int xoff[4];
 #pragma unroll
-        for (int p = 0; p < MI; p++) *(u32x4_t*)(&xs[buf][(32 * p + xr) * GEMM_PITCH + xc]) = xreg[p];
-    };
+    for (int t = 0; t < 4; t++) xoff[t] = ln * 128 + (((4 * lc + t) ^ swz(ln)) * 16);
 
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-
-    for (int it = 0; it < nit; it++) {
-        const int cur = it & 1;
-        // Dequantise this step's weights into the four B operands per column tile.
+    // One K step; C = it % GEMM_STAGES selects the register stage.  The loads of step
+    // it + 2 are issued first and fenced off (the scheduler would otherwise sink them
+    // below the matrix instructions); behind the fence the dequantisation of this
+    // step's weight registers and the matrix instructions interleave freely.  At the
+    // end the activations of step it + 1, fetched a step ago, go to the other LDS
+    // buffer: loads complete in order, so that store waits for nothing recent.
+    auto step = [&](int it, auto C, auto P) {
+        constexpr int c = decltype(C)::value;
+        constexpr int par = decltype(P)::value;  // LDS buffer of this step
+        constexpr int cf = (c + GEMM_STAGES - 1) % GEMM_STAGES;  // stage receiving step it + 2
+        constexpr int c1 = (c + 1) % GEMM_STAGES;                // stage holding step it + 1
+        load_x(it + GEMM_STAGES - 1, xr[cf]);
+        load_w(it + GEMM_STAGES - 1, w[cf]);
+        __builtin_amdgcn_sched_barrier(0);
         half8_t bf[2][4];
+        const bool kin = it * GEMM_BK + 32 * lc < K;  // false only past K: scale 0 -> W_hat 0
 #pragma unroll
         for (int ni = 0; ni < 2; ni++) {
-            const half2_t z64 = {zq[ni].x, zq[ni].x};
-            const half2_t sc = {zq[ni].y, zq[ni].y};
+            const half_t sv = kin ? w[c].zs[ni].y : (half_t)0.f;
+            const half2_t z64 = {w[c].zs[ni].x, w[c].zs[ni].x};
+            const half2_t sc = {sv, sv};
 #pragma unroll
-            for (int t = 0; t < 4; t++) bf[ni][t] = dequant8(wq[ni][t], z64, sc);
+            for (int t = 0; t < 4; t++) bf[ni][t] = dequant8(w[c].q[ni][t], z64, sc, nm);
         }
-        // Prefetch the next step (registers only; LDS is written after the MFMAs).
-        if (it + 1 < nit) load_tile(it + 1);
-
-        const half_t* xb = &xs[cur][ln * GEMM_PITCH + 32 * lc];
+        const uint8_t* xp = &xs[par][0];
 #pragma unroll
         for (int t = 0; t < 4; t++) {
 #pragma unroll
             for (int mi = 0; mi < MI; mi++) {
-                const half8_t a = *(const half8_t*)(xb + (32 * mi) * GEMM_PITCH + 8 * t);
+                const half8_t a = *(const half8_t*)(xp + (32 * mi) * 128 + xoff[t]);
 #pragma unroll
                 for (int ni = 0; ni < 2; ni++)
                     acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bf[ni][t], acc[mi][ni], 0, 0, 0);
             }
         }
-        if (it + 1 < nit) store_tile(cur ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        store_x(par ^ 1, xr[c1]);
         __syncthreads();
+    };
+
+#pragma unroll
+    for (int s0 = 0; s0 < GEMM_STAGES - 1; s0++) {
+        load_x(s0, xr[s0]);
+        load_w(s0, w[s0]);
+    }
+    store_x(0, xr[0]);
+    __syncthreads();
+    // Six steps per trip (stage indices are compile-time); the step count is padded
+    // with steps whose scale is 0 everywhere and whose loads are clamped.
+    constexpr int TRIP = 2 * GEMM_STAGES;
+    static_assert(GEMM_STAGES == 3, "the trip below is written for three register stages");
+    const int nitp = (nit + TRIP - 1) / TRIP * TRIP;
+    for (int it = 0; it < nitp; it += TRIP) {
+        // LDS buffer = step parity, register stage = step % GEMM_STAGES: unroll over
+        // their common period.
+        step(it, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+        step(it + 1, std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{});
+        step(it + 2, std::integral_constant<int, 2>{}, std::integral_constant<int, 0>{});
+        step(it + 3, std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
+        step(it + 4, std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+        step(it + 5, std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
     }
 
     // Epilogue: fp32 -> fp16, 32 consecutive columns per half-wave.

@@ -33,6 +33,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const uint8_t* __restrict__ 
     constexpr int MT = (MROWS + 3) / 4;
     extern __shared__ float red[];
 
+    const NibbleMasks nm = nibble_masks();
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int nwaves = blockDim.x >> 6;
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const uint8_t* __restrict__ 
             if (!FIXUP) {
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    const half8_t wv = dequant8(wq[rs][t], z64, sc);
+                    const half8_t wv = dequant8(wq[rs][t], z64, sc, nm);
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
                         const half8_t xv = bit_cast<half8_t>(xa[mt][t]);
@@ -132,7 +133,7 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const uint8_t* __restrict__ 
                 for (int mt = 0; mt < MT; mt++) tmp[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    const half8_t wv = unpack8_raw(wq[rs][t]);
+                    const half8_t wv = unpack8_raw(wq[rs][t], nm);
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
                         const half8_t xv = bit_cast<half8_t>(xa[mt][t]);

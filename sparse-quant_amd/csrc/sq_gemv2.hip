@@ -46,6 +46,7 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
     __shared__ __attribute__((aligned(16))) float xsum[KS][S * 16][MROWS];
     __shared__ float red[KS][NR][MROWS][4];
 
+    const NibbleMasks nm = nibble_masks();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
                 const half2_t sc = {p.y, p.y};
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    const half8_t wv = dequant8(wq[s][t], z64, sc);
+                    const half8_t wv = dequant8(wq[s][t], z64, sc, nm);
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
                         acc[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, wv.lo, acc[mt], 0, 0, 0);
@@ -143,7 +144,7 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
                 for (int mt = 0; mt < MT; mt++) tmp[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    const half8_t wv = unpack8_raw(wq[s][t]);
+                    const half8_t wv = unpack8_raw(wq[s][t], nm);
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
                         tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, wv.lo, tmp[mt], 0, 0, 0);

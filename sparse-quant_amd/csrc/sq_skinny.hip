@@ -25,6 +25,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(const uint8_t* __restrict__
                                                      const half_t* __restrict__ X, half_t* __restrict__ Y, int M,
                                                      int N, int K, int gshift) {
     extern __shared__ float red[];
+    const NibbleMasks nm = nibble_masks();
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int nwaves = blockDim.x >> 6;
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(const uint8_t* __restrict__
             const half2_t sc = {zsv.y, zsv.y};
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                const half8_t wv = dequant8(wq[t], z64, sc);
+                const half8_t wv = dequant8(wq[t], z64, sc, nm);
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++)
                     acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<half8_t>(xa[mt][t]), wv, acc[mt], 0,
@@ -81,7 +82,7 @@ __global__ __launch_bounds__(512) void skinny_kernel(const uint8_t* __restrict__
             }
 #pragma unroll
             for (int t = 0; t < 4; t++) {
-                const half8_t wv = unpack8_raw(wq[t]);
+                const half8_t wv = unpack8_raw(wq[t], nm);
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++) {
                     const half8_t xv = bit_cast<half8_t>(xa[mt][t]);
