@@ -106,6 +106,18 @@ int sq_repack_l2_to_l1(const void* w_l2, const void* zs_l2, void* w_l1, void* zs
  * (reference: test/muxi/module/qlinear/qlinear.py:93-103). */
 int sq_convert_2bit_to_4bit(const void* src, void* dst, int N, int K, void* stream);
 
+/* LUT block-sparse attention, prefill: out[z,h,m,:] = softmax over the keys of the
+ * blocks lut[h][m/64][0..nnz) of (q k^T * sm_scale) (optionally causal) times v.
+ * q, k, v, out fp16 [Z, H, S, D] contiguous, D in {64, 128}; lut int32 or int64
+ * (lut_elem_bytes 4 or 8) [H, ceil(S/64), nnz], key-block indices of 64 keys; an
+ * entry equal to its predecessor in the row is padding; at most ceil(S/64) entries
+ * of a row are visited.  Replaces sparse_attention_prefill (reference:
+ * sparse-attention/nvidia/playground/kernels/block_sparse_attention_lut.py:22-243;
+ * sparse-attention/muxi/playground/kernels/csrc/src/block_sparse_attention_lut.cu:49-55). */
+int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out, const void* lut,
+                         int lut_elem_bytes, int Z, int H, int S, int D, int nnz, float sm_scale, int causal,
+                         void* stream);
+
 #ifdef __cplusplus
 }
 #endif

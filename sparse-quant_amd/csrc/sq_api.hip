@@ -146,4 +146,15 @@ int sq_convert_2bit_to_4bit(const void* src, void* dst, int N, int K, void* stre
     return launch_code(sq::launch_2bit_to_4bit(src, dst, N, K, static_cast<hipStream_t>(stream)));
 }
 
+int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out, const void* lut, int lut_elem_bytes,
+                         int Z, int H, int S, int D, int nnz, float sm_scale, int causal, void* stream) {
+    if (Z <= 0 || H <= 0 || S <= 0 || nnz <= 0 || (D != 64 && D != 128)) return SQ_ERR_BAD_SHAPE;
+    if ((long)Z * H > 65535) return SQ_ERR_BAD_SHAPE;
+    if (lut_elem_bytes != 4 && lut_elem_bytes != 8) return SQ_ERR_BAD_LAYOUT;
+    if (!q || !k || !v || !out || !lut) return SQ_ERR_NULL_POINTER;
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return SQ_ERR_MISALIGNED;
+    return launch_code(sq::launch_lut_attention(q, k, v, out, lut, lut_elem_bytes, Z, H, S, D, nnz, sm_scale, causal,
+                                                static_cast<hipStream_t>(stream)));
+}
+
 }  // extern "C"

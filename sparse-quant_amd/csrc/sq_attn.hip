@@ -1,0 +1,192 @@
+// LUT block-sparse attention, prefill (fp16 in/out, fp32 softmax and accumulation).
+// For query block i of head h only the key blocks lut[h][i][0..nnz) are visited
+// (64 x 64 blocks; a LUT entry equal to its predecessor is padding and is skipped);
+// inside a block an optional causal mask and the sequence-length mask apply.
+// (replaces _sparse_attention_prefill_fwd_kernel, reference:
+// sparse-attention/nvidia/playground/kernels/block_sparse_attention_lut.py:22-172, and
+// sparse_attention_prefill_fwd_p, sparse-attention/muxi/playground/kernels/csrc/include/
+// block_sparse_attention_lut.cuh:30-236)
+//
+// Mapping.  A workgroup (4 waves) owns one 64-row query block of one (batch, head);
+// wave w owns queries 16w .. 16w+15.  Both products are computed transposed with
+// v_mfma_f32_16x16x32_f16 so that a lane always owns ONE query (column l%16):
+//   S^T = K Q^T : A = K tile (row = key, from LDS), B = Q^T (registers, pre-scaled by
+//                 sm_scale*log2(e) and rounded to fp16 like the reference);
+//                 D: lane (query l%16) holds keys 16t + 4*(l/16) + v of key tile t.
+//   softmax     : over a lane's 16 values and the 4 lanes {l, l^16, l^32, l^48}; the
+//                 running max / sum of a query live in its lanes, nothing is exchanged.
+//   O^T = V^T P^T: B = P^T is exactly what the lane already holds: for the k-step
+//                 covering keys 32s .. 32s+31 lane group g supplies keys 32s+4g+{0..3}
+//                 and 32s+16+4g+{0..3}; A = V^T rows read from an LDS copy of the V
+//                 tile that was transposed while staging (two 64-bit reads);
+//                 D: lane (query l%16) holds head-dim rows 16*dt + 4*(l/16) + v.
+// K and V tiles are staged once per block for the four waves; V is transposed on the
+// way in (each thread packs two adjacent keys into 32-bit LDS writes).
+#include "sq_common.h"
+#include "sq_kernels.h"
+
+namespace sq {
+
+template <int D>
+__global__ __launch_bounds__(256) void lut_attn_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ Kp,
+                                                       const half_t* __restrict__ V, half_t* __restrict__ O,
+                                                       const void* __restrict__ lut, int lut_is_64, int H, int S,
+                                                       int nblk_q, int nnz, int nvisit, float qk_scale, int causal) {
+    constexpr int KP = D + 8;    // halves per row of the K tile in LDS
+    constexpr int VP = 64 + 8;   // halves per row of the transposed V tile in LDS
+    constexpr int DK = D / 32;   // k-steps of S^T
+    constexpr int DT = D / 16;   // row tiles of O^T
+    __shared__ __attribute__((aligned(16))) half_t ks[64 * KP];
+    __shared__ __attribute__((aligned(16))) half_t vt[D * VP];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int lq = lane & 15;
+    const int g = lane >> 4;
+    const int qb = blockIdx.x;
+    const int zh = blockIdx.y;
+    const int h = zh % H;
+    const long base = (long)zh * S * D;
+    const int m = qb * 64 + 16 * wave + lq;  // this lane's query
+    const int mc = imin(m, S - 1);
+
+    // Q^T operand: q * (sm_scale * log2 e), rounded to fp16.
+    half8_t qf[DK];
+#pragma unroll
+    for (int s = 0; s < DK; s++) {
+        const half8_t raw = *(const half8_t*)(Q + base + (long)mc * D + 32 * s + 8 * g);
+#pragma unroll
+        for (int e = 0; e < 8; e++) qf[s][e] = (half_t)((float)raw[e] * qk_scale);
+    }
+
+    float m_i = -INFINITY, l_i = 0.f;
+    float4_t acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) acc[dt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+
+    const long lut_row = ((long)h * nblk_q + qb) * nnz;
+    int last = -1;
+    for (int j = 0; j < nvisit; j++) {
+        const int blk = lut_is_64 ? (int)((const long long*)lut)[lut_row + j] : ((const int*)lut)[lut_row + j];
+        const bool skip = (blk == last) || blk < 0 || (long)blk * 64 >= S;
+        last = blk;
+        if (skip) continue;  // uniform over the workgroup
+        const int n0 = blk * 64;
+
+        __syncthreads();  // the previous tiles are no longer read
+        // K tile: 64 keys x D halves, 16 bytes per thread per pass.
+#pragma unroll
+        for (int p = 0; p < D / 32; p++) {
+            const int idx = tid + 256 * p;
+            const int key = idx / (D / 8);
+            const int c8 = idx % (D / 8);
+            const u32x4_t v = *(const u32x4_t*)(Kp + base + (long)imin(n0 + key, S - 1) * D + 8 * c8);
+            *(u32x4_t*)(&ks[key * KP + 8 * c8]) = v;
+        }
+        // V tile, transposed: a thread takes keys 2kp, 2kp+1 and 8 head-dim values and
+        // writes 8 packed pairs vt[d][2kp .. 2kp+1].
+#pragma unroll
+        for (int p = 0; p < D / 64; p++) {
+            const int idx = tid + 256 * p;
+            const int kp = idx & 31;
+            const int c8 = idx >> 5;
+            const half8_t v0 = *(const half8_t*)(V + base + (long)imin(n0 + 2 * kp, S - 1) * D + 8 * c8);
+            const half8_t v1 = *(const half8_t*)(V + base + (long)imin(n0 + 2 * kp + 1, S - 1) * D + 8 * c8);
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const half2_t pr = {v0[e], v1[e]};
+                *(half2_t*)(&vt[(8 * c8 + e) * VP + 2 * kp]) = pr;
+            }
+        }
+        __syncthreads();
+
+        // S^T = K Q^T for the four 16-key tiles.
+        float4_t st[4];
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            st[t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < DK; s++) {
+                const half8_t a = *(const half8_t*)(&ks[(16 * t + lq) * KP + 32 * s + 8 * g]);
+                st[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[s], st[t], 0, 0, 0);
+            }
+        }
+        // Masks and the block maximum of this query.
+        float mx = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const int n = n0 + 16 * t + 4 * g + v;
+                const bool keep = (n < S) && (!causal || n <= m);
+                st[t][v] = keep ? st[t][v] : -INFINITY;
+                mx = fmaxf(mx, st[t][v]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_i, mx);
+        // A query with nothing visible so far keeps p = 0 and alpha = 1 (no NaN from inf - inf).
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = (m_i == -INFINITY) ? (m_new == -INFINITY ? 1.f : 0.f) : exp2f(m_i - m_new);
+        float rs = 0.f;
+        half8_t pk[2];
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float p = exp2f(st[t][v] - m_use);  // exp2(-inf) = 0 for masked entries
+                rs += p;
+                pk[t >> 1][4 * (t & 1) + v] = (half_t)p;
+            }
+        rs += __shfl_xor(rs, 16);
+        rs += __shfl_xor(rs, 32);
+        l_i = l_i * alpha + rs;
+        m_i = m_new;
+
+        // O^T = O^T * alpha + V^T P^T.
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+            acc[dt] *= alpha;
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                const half_t* vp = &vt[(16 * dt + lq) * VP + 32 * s + 4 * g];
+                const u32x2_t lo = *(const u32x2_t*)(vp);
+                const u32x2_t hi = *(const u32x2_t*)(vp + 16);
+                const u32x4_t a = {lo.x, lo.y, hi.x, hi.y};
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<half8_t>(a), pk[s], acc[dt], 0, 0, 0);
+            }
+        }
+    }
+
+    // O[m][16*dt + 4g + v] = acc / l.
+    if (m < S) {
+        const float inv = l_i > 0.f ? 1.f / l_i : 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+            half4_t o;
+#pragma unroll
+            for (int v = 0; v < 4; v++) o[v] = (half_t)(acc[dt][v] * inv);
+            *(half4_t*)(O + base + (long)m * D + 16 * dt + 4 * g) = o;
+        }
+    }
+}
+
+hipError_t launch_lut_attention(const void* q, const void* k, const void* v, void* o, const void* lut,
+                                int lut_elem_bytes, int Z, int H, int S, int D, int nnz, float sm_scale, int causal,
+                                hipStream_t st) {
+    const int nblk = (S + 63) / 64;
+    const dim3 grid(nblk, Z * H);
+    const float qk_scale = sm_scale * 1.44269504f;
+    const int use_nnz = nnz < nblk ? nnz : nblk;  // the reference clamps NNZ to ceil(S / 64) as well
+    // (the LUT row pitch stays nnz even when fewer entries are visited)
+    if (D == 64)
+        hipLaunchKernelGGL((lut_attn_kernel<64>), grid, dim3(256), 0, st, (const half_t*)q, (const half_t*)k,
+                           (const half_t*)v, (half_t*)o, lut, lut_elem_bytes == 8, H, S, nblk, nnz, use_nnz, qk_scale, causal);
+    else
+        hipLaunchKernelGGL((lut_attn_kernel<128>), grid, dim3(256), 0, st, (const half_t*)q, (const half_t*)k,
+                           (const half_t*)v, (half_t*)o, lut, lut_elem_bytes == 8, H, S, nblk, nnz, use_nnz, qk_scale, causal);
+    return hipGetLastError();
+}
+
+}  // namespace sq

@@ -34,4 +34,9 @@ hipError_t launch_skinny_tuned(const void* x, const void* w, const void* zs, voi
 hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
                              int tune, hipStream_t st);
 
+// sq_attn.hip: LUT block-sparse attention, prefill.  D in {64, 128}; lut int32 or int64 [H, ceil(S/64), nnz].
+hipError_t launch_lut_attention(const void* q, const void* k, const void* v, void* o, const void* lut,
+                                int lut_elem_bytes, int Z, int H, int S, int D, int nnz, float sm_scale, int causal,
+                                hipStream_t st);
+
 }  // namespace sq

@@ -32,6 +32,7 @@ SIGNATURES = {
     "sq_convert_awq_to_lmdeploy": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_repack_l2_to_l1": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "sq_convert_2bit_to_4bit": (_i, [_vp, _vp, _i, _i, _vp]),
+    "sq_lut_attention_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, ctypes.c_float, _i, _vp]),
 }
 
 _lib = None
@@ -129,4 +130,14 @@ def convert_2bit_to_4bit(w2, stream=None):
     out = torch.empty((n, k4 * 2), dtype=torch.uint8, device=w2.device)
     _check(lib().sq_convert_2bit_to_4bit(_ptr(w2), _ptr(out), n, k4 * 4, _stream(stream)),
            "sq_convert_2bit_to_4bit")
+    return out
+
+
+def lut_attention(q, k, v, lut, sm_scale, causal, stream=None):
+    """q, k, v fp16 [Z,H,S,D] contiguous; lut int32/int64 [H, ceil(S/64), nnz] -> out fp16 [Z,H,S,D]."""
+    z, h, s, d = q.shape
+    out = torch.empty_like(q)
+    _check(lib().sq_lut_attention_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lut), lut.element_size(), z, h, s, d,
+                                      lut.shape[-1], float(sm_scale), int(bool(causal)), _stream(stream)),
+           "sq_lut_attention_fwd")
     return out
