@@ -106,6 +106,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 TFLOP/s leg")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the fused-QKV, LUT-attention and end-to-end OPT-6.7B legs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch plain device copies of 256 MiB (reads 256 MiB, writes 256 MiB): the known-size "
                          "kernel that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
@@ -224,6 +226,15 @@ def main():
                               "launches": 5}
     if not args.no_prefill:
         out["prefill"] = prefill_leg(torch, capi, pool[0], shapes, g, dev, gen, stream)
+    if not args.no_extras:
+        # Additional, separately labelled legs; none of them feeds `value`.
+        try:
+            out["fused_qkv"] = fused_qkv_leg(torch, capi, m, g, dev, gen, stream, args.layers, bytes_per_step)
+            out["attention"] = attention_leg(torch, capi, dev)
+            from sqamd import opt_decode
+            out["e2e_opt67"] = opt_decode.run_e2e(batch=8, prompt=512, new_tokens=128)
+        except Exception as exc:  # an extra leg must never hide the headline line
+            out["extras_error"] = repr(exc)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(m, g, shapes)
     print(json.dumps(out))
@@ -254,6 +265,67 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
     tf = flops_total / time_total / 1e6
     return {"m": m, "tflops": round(tf, 1), "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
             "per_linear": res}
+
+
+def fused_qkv_leg(torch, capi, m, g, dev, gen, stream, layers, bytes_per_step):
+    """The same step with q/k/v served by ONE launch on the row-concatenated weight [12288, 4096]
+    (possible because layout L1 is row-major in N); four launches per step instead of six."""
+    shapes = [("qkv_proj", 12288, 4096), ("out_proj", 4096, 4096), ("fc1", 16384, 4096), ("fc2", 4096, 16384)]
+    pool = [[make_linear(n, k, g, dev, gen) for _, n, k in shapes] for _ in range(layers)]
+    xs = {k: torch.randn((m, k), device=dev, generator=gen).half() for k in (4096, 16384)}
+    ys = {n: torch.empty((m, n), dtype=torch.float16, device=dev) for n in (12288, 4096, 16384)}
+    steps = 2000
+    with torch.cuda.stream(stream):
+        def run(i):
+            for (w, zs), (_, n, k) in zip(pool[i % layers], shapes):
+                capi.gemm(xs[k], w, zs, n, k, g, out=ys[n], stream=stream)
+        for i in range(layers):
+            run(i)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(layers):
+                run(i)
+        for _ in range(10):
+            graph.replay()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps // layers):
+            graph.replay()
+        e1.record(stream)
+        stream.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / (steps // layers * layers)
+    return {"us_per_step": round(us, 2), "gbs": round(bytes_per_step / us / 1e3, 1), "launches_per_step": 4}
+
+
+def attention_leg(torch, capi, dev):
+    """LUT block-sparse attention (BASELINE configs[3]): batch 8, 16 heads, head dim 64, 64x64 blocks,
+    ~25 % density with the diagonal block kept, non-causal; flops = 4 * kept blocks * 64 * 64 * D."""
+    import lut_attention_oracle as att
+    res = {}
+    for s in (512, 4096):
+        z, h, d = 8, 16, 64
+        lay = att.synth_layout(h, s // 64, 0.25, False, seed=1)
+        lut = torch.from_numpy(att.layout_to_lut(lay)).to(dev)
+        kept = int(lay.sum()) * z
+        q = torch.randn((z, h, s, d), device=dev).half()
+        k = torch.randn_like(q)
+        v = torch.randn_like(q)
+        for _ in range(3):
+            capi.lut_attention(q, k, v, lut, d ** -0.5, False)
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            capi.lut_attention(q, k, v, lut, d ** -0.5, False)
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / 20
+        tf = 4.0 * kept * 64 * 64 * d / us / 1e6
+        res["seq%d" % s] = {"us": round(us, 1), "tflops": round(tf, 1),
+                            "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4)}
+    return res
 
 
 if __name__ == "__main__":

@@ -63,7 +63,9 @@ int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y, int 
     int kernel = algo & 0xFF;
     const int tune = (algo >> 8) & 0xFFFF;
     if (kernel == SQ_ALGO_AUTO) {
-        if (M <= 8)
+        // 5..8 tokens with a long K: the GEMV's staged activations would need several
+        // sequential rounds; the 16-column kernel is faster there (measured on fc2 shapes).
+        if (M <= 4 || (M <= 8 && K <= 8192))
             kernel = SQ_ALGO_GEMV_FIXUP;
         else if (M <= 32)
             kernel = SQ_ALGO_SKINNY;

@@ -1,0 +1,177 @@
+"""Random-init OPT-6.7B-shaped decoder with W4A16 linears: the end-to-end harness.
+
+This is the shape generator of BASELINE configuration 5, not a model port: 32
+pre-LN decoder layers, hidden 4096, 32 heads (head dim 128), FFN 16384 with ReLU,
+vocab 50272, learned positions with OPT's +2 offset, fp16 lm_head; q/k/v/out/fc1/fc2
+are `WALinear` modules (layout L1, group 128) with random packed weights -- the same
+six linears per layer, in the same order and with the same [1, tokens, K] call shape
+the reference feeds to gemm_awq_ut (test/nvidia/module/opt/modeling_opt_ours.py:
+158-164, 505-506, 598-611).  Attention is dense (the reference's decode path is dense
+too); the KV cache is fp16 and preallocated so that a decode step is a fixed kernel
+sequence that can be captured in a HIP graph.
+"""
+import math
+import time
+
+import torch
+from torch import nn
+
+from .qlinear import WALinear
+
+
+def _random_walinear(in_f, out_f, g, dev, gen):
+    lin = WALinear(in_f, out_f, w_bit=4, group_size=g, bias=True, dev=dev, layout="l1")
+    lin.weight = torch.randint(0, 256, (out_f, in_f // 2), dtype=torch.uint8, device=dev, generator=gen)
+    z = torch.randint(0, 16, (out_f, in_f // g), device=dev, generator=gen).half() + 64
+    s = (torch.randn((out_f, in_f // g), device=dev, generator=gen).abs() * 0.004 + 2e-4).half()
+    lin.zeros_scales = torch.stack([z, s], dim=-1).reshape(out_f, 2 * (in_f // g)).contiguous()
+    lin.bias = (torch.randn((1, out_f), device=dev, generator=gen) * 0.01).half()
+    return lin
+
+
+class DecoderLayer(nn.Module):
+    def __init__(self, hidden, heads, ffn, g, dev, gen):
+        super().__init__()
+        self.heads, self.hd = heads, hidden // heads
+        self.ln1 = nn.LayerNorm(hidden, device=dev, dtype=torch.float16)
+        self.ln2 = nn.LayerNorm(hidden, device=dev, dtype=torch.float16)
+        self.q_proj = _random_walinear(hidden, hidden, g, dev, gen)
+        self.k_proj = _random_walinear(hidden, hidden, g, dev, gen)
+        self.v_proj = _random_walinear(hidden, hidden, g, dev, gen)
+        self.out_proj = _random_walinear(hidden, hidden, g, dev, gen)
+        self.fc1 = _random_walinear(hidden, ffn, g, dev, gen)
+        self.fc2 = _random_walinear(ffn, hidden, g, dev, gen)
+
+    def forward(self, x, kc, vc, pos0, mask):
+        """x [B, T, H]; kc, vc [B, heads, Lmax, hd]; writes cache rows pos0 .. pos0+T-1."""
+        b, t, hdim = x.shape
+        h = self.ln1(x)
+        flat = h.reshape(1, b * t, hdim)  # the reference flattens to [1, bs*seq, K] as well
+        q = self.q_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
+        k = self.k_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
+        v = self.v_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
+        if isinstance(pos0, int):
+            kc[:, :, pos0:pos0 + t] = k
+            vc[:, :, pos0:pos0 + t] = v
+            a = nn.functional.scaled_dot_product_attention(q, kc[:, :, :pos0 + t], vc[:, :, :pos0 + t],
+                                                           is_causal=(t > 1))
+        else:  # graph-captured decode step: position lives in a device tensor, the mask hides unused rows
+            kc.index_copy_(2, pos0, k)
+            vc.index_copy_(2, pos0, v)
+            a = nn.functional.scaled_dot_product_attention(q, kc, vc, attn_mask=mask)
+        a = a.transpose(1, 2).reshape(1, b * t, hdim)
+        x = x + self.out_proj(a).view(b, t, hdim)
+        h = self.ln2(x).reshape(1, b * t, hdim)
+        h = torch.relu(self.fc1(h))
+        return x + self.fc2(h).view(b, t, hdim)
+
+
+class OPTDecoder(nn.Module):
+    def __init__(self, layers=32, hidden=4096, heads=32, ffn=16384, vocab=50272, max_pos=2048, group=128,
+                 dev="cuda", seed=0):
+        super().__init__()
+        gen = torch.Generator(device=dev)
+        gen.manual_seed(seed)
+        self.hidden, self.heads = hidden, heads
+        self.embed = (torch.randn((vocab, hidden), device=dev, generator=gen) * 0.02).half()
+        self.pos = (torch.randn((max_pos + 2, hidden), device=dev, generator=gen) * 0.02).half()
+        self.layers = nn.ModuleList([DecoderLayer(hidden, heads, ffn, group, dev, gen) for _ in range(layers)])
+        self.final_ln = nn.LayerNorm(hidden, device=dev, dtype=torch.float16)
+        self.lm_head = (torch.randn((vocab, hidden), device=dev, generator=gen) * 0.02).half()
+
+    def new_cache(self, batch, max_len):
+        hd = self.hidden // self.heads
+        shape = (batch, self.heads, max_len, hd)
+        dev = self.embed.device
+        return [(torch.zeros(shape, dtype=torch.float16, device=dev), torch.zeros(shape, dtype=torch.float16, device=dev))
+                for _ in self.layers]
+
+    @torch.no_grad()
+    def forward(self, ids, cache, pos0, pos_ids=None, mask=None):
+        b, t = ids.shape
+        if pos_ids is None:
+            pos_ids = torch.arange(pos0, pos0 + t, device=ids.device) + 2
+        x = self.embed[ids] + self.pos[pos_ids]
+        for layer, (kc, vc) in zip(self.layers, cache):
+            x = layer(x, kc, vc, pos0, mask)
+        x = self.final_ln(x[:, -1:])
+        return torch.matmul(x, self.lm_head.t())  # [B, 1, vocab]
+
+
+@torch.no_grad()
+def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed=0):
+    """Greedy generation on random token ids; returns timing and throughput figures."""
+    dev = "cuda"
+    model = OPTDecoder(layers=layers, dev=dev, seed=seed)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(seed + 1)
+    ids = torch.randint(0, 50272, (batch, prompt), device=dev, generator=gen)
+    max_len = prompt + new_tokens
+    cache = model.new_cache(batch, max_len)
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    logits = model(ids, cache, 0)
+    nxt = logits.argmax(-1)
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+
+    # One decode step with device-side position so that it can be replayed as a graph.
+    pos_t = torch.tensor([prompt], device=dev, dtype=torch.long)
+    mask = torch.zeros((1, 1, 1, max_len), device=dev, dtype=torch.float16)
+    tok = nxt.clone()
+    out_tok = torch.empty_like(tok)
+
+    def set_mask():
+        mask.fill_(float("-inf"))
+        mask[..., :int(pos_t.item()) + 1] = 0
+
+    def step():
+        lg = model(tok, cache, pos_t, pos_ids=pos_t + 2, mask=mask)
+        out_tok.copy_(lg.argmax(-1))
+
+    graph = None
+    if use_graph:
+        set_mask()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()  # warm-up outside capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+    generated = [tok.clone()]
+    mask.fill_(float("-inf"))
+    mask[..., :prompt] = 0
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(new_tokens - 1):
+        # the key/value row written by this step becomes visible to it
+        mask[..., prompt + i] = 0
+        if graph is not None:
+            graph.replay()
+        else:
+            step()
+        tok.copy_(out_tok)
+        pos_t += 1
+        generated.append(tok.clone())
+    torch.cuda.synchronize()
+    decode_s = time.perf_counter() - t0
+    steps = new_tokens - 1
+    return {
+        "batch": batch, "prompt": prompt, "new_tokens": new_tokens, "layers": layers,
+        "launch": "hip-graph replay" if graph is not None else "eager",
+        "prefill_ms": round(prefill_s * 1e3, 2),
+        "prefill_tok_per_s": round(batch * prompt / prefill_s, 1),
+        "decode_ms_per_step": round(decode_s * 1e3 / steps, 4),
+        "decode_tok_per_s": round(batch * steps / decode_s, 1),
+        "tokens_checksum": int(torch.stack(generated).sum().item()),
+    }
+
+
+if __name__ == "__main__":
+    import json
+    import sys
+    print(json.dumps(run_e2e(use_graph="--no-graph" not in sys.argv)))
