@@ -21,6 +21,8 @@
 #ifndef SQ_W4A16_H
 #define SQ_W4A16_H
 
+#include <stddef.h>
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -44,6 +46,8 @@ extern "C" {
 #define SQ_ALGO_GEMV_FIXUP 2     /* M <= 8: same, zero/scale applied per group in fp32 */
 #define SQ_ALGO_SKINNY 3         /* M <= 64: 16-column MFMA tiles, weights straight from registers */
 #define SQ_ALGO_GEMM 4           /* any M: LDS-tiled MFMA GEMM */
+#define SQ_ALGO_SKINNY_WS 5      /* M <= 32: 64-row tiles, K split over workgroups through a workspace
+                                    (sq_w4a16_gemm_ws only) */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int sq_version(void);
@@ -67,6 +71,22 @@ int sq_w4a16_gemm(const void* x, const void* w, const void* zs, void* y,
 int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y,
                      int M, int N, int K, int group_size, int layout, int algo,
                      void* stream);
+
+/* Same product with a caller-owned device workspace, which lets the 5 <= M <= 32
+ * range split K over workgroups (fp32 partial tiles, summed in a fixed order by the
+ * workgroup that finishes last, so results are bit-reproducible).  No counterpart
+ * in the reference.  The workspace must hold at least
+ * sq_w4a16_workspace_bytes(M, N, K) bytes, be 16-byte aligned, and have its first
+ * 64 KiB zeroed before the first call (every call leaves them zero); calls that
+ * share a workspace must not overlap in time.  Outside 5 <= M <= 32 (or with an
+ * explicit other algo) the call behaves like sq_w4a16_gemm_ex and ignores the
+ * workspace. */
+int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y,
+                     int M, int N, int K, int group_size, int layout, int algo,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/* Bytes sq_w4a16_gemm_ws needs for this shape (grows with N; M is capped at 32). */
+size_t sq_w4a16_workspace_bytes(int M, int N, int K);
 
 /* out[N,K] (fp16) = W_hat in natural k order, bit-identical to fp16
  * (q_fp16 - z_fp16) * s_fp16.  Replaces dequant

@@ -91,6 +91,30 @@ int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y, int 
     }
 }
 
+size_t sq_w4a16_workspace_bytes(int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    return sq::skinny2_workspace_bytes(M > 32 ? 32 : M, N, K);
+}
+
+int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
+                     int layout, int algo, void* workspace, size_t workspace_bytes, void* stream) {
+    const int kernel = algo & 0xFF;
+    const bool want = kernel == SQ_ALGO_SKINNY_WS || (kernel == SQ_ALGO_AUTO && M > 4 && M <= 32);
+    if (!want) return sq_w4a16_gemm_ex(x, w, zs, y, M, N, K, group_size, layout, algo, stream);
+    if (M < 0 || M > 32) return M < 0 ? SQ_ERR_BAD_SHAPE : SQ_ERR_BAD_ALGO;
+    const int rc = check_weight(N, K, group_size, layout);
+    if (rc != SQ_OK) return rc;
+    if (layout != SQ_LAYOUT_L1) return SQ_ERR_BAD_LAYOUT;
+    if (M == 0) return SQ_OK;
+    if (!x || !w || !zs || !y) return SQ_ERR_NULL_POINTER;
+    if (!aligned16(x) || !aligned16(w) || !aligned16(zs) || !aligned16(y)) return SQ_ERR_MISALIGNED;
+    if (!workspace || !aligned16(workspace) || workspace_bytes < sq::skinny2_workspace_bytes(M, N, K) ||
+        (N + 63) / 64 > 16384)
+        return SQ_ERR_WORKSPACE;
+    return launch_code(sq::launch_skinny2_tuned(x, w, zs, y, workspace, M, N, K, group_size, (algo >> 8) & 0xFFFF,
+                                                static_cast<hipStream_t>(stream)));
+}
+
 int sq_w4a16_gemm(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
                   int layout, void* stream) {
     return sq_w4a16_gemm_ex(x, w, zs, y, M, N, K, group_size, layout, SQ_ALGO_AUTO, stream);

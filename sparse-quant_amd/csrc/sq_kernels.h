@@ -30,6 +30,11 @@ hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void
 // sq_skinny.hip: M <= 64.  tune = waves | mode << 8 (mode 1 = exact, 2 = fixup).
 hipError_t launch_skinny_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
                                int tune, hipStream_t st);
+// sq_skinny2.hip: 5 <= M <= 32 with a workspace (counters + fp32 partial tiles).
+// tune = ksplit (1,2,4,8) | mode << 8 (1 = exact, 2 = fixup).
+size_t skinny2_workspace_bytes(int M, int N, int K);
+hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
+                                int g, int tune, hipStream_t st);
 // sq_gemm.hip: any M.  tune = 32-row tiles per workgroup (1,2,4).
 hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
                              int tune, hipStream_t st);

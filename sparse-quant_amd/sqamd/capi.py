@@ -26,6 +26,8 @@ SIGNATURES = {
     "sq_strerror": (ctypes.c_char_p, [_i]),
     "sq_w4a16_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "sq_w4a16_gemm_ex": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
+    "sq_w4a16_gemm_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp]),
+    "sq_w4a16_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
     "sq_w4a16_dequant": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "sq_transpose_merge_zeros_scales": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sq_convert_ours_to_awq": (_i, [_vp, _vp, _i, _i, _vp]),
@@ -86,6 +88,33 @@ def gemm(x, w, zs, n, k, group_size, layout=SQ_LAYOUT_L1, algo=SQ_ALGO_AUTO, out
         out = torch.empty((m, n), dtype=torch.float16, device=x.device)
     _check(lib().sq_w4a16_gemm_ex(_ptr(x), _ptr(w), _ptr(zs), _ptr(out), m, n, k, group_size, layout, algo,
                                   _stream(stream)), "sq_w4a16_gemm_ex")
+    return out
+
+
+SQ_ALGO_SKINNY_WS = 5
+_workspaces = {}
+
+
+def workspace(m, n, k, device, stream=None):
+    """A zero-initialised workspace tensor, cached per (device, stream) and grown on demand."""
+    need = lib().sq_w4a16_workspace_bytes(m, n, k)
+    key = (str(device), (stream or torch.cuda.current_stream()).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def gemm_ws(x, w, zs, n, k, group_size, algo=SQ_ALGO_AUTO, out=None, stream=None, ws=None):
+    """x fp16 [M,K] -> y fp16 [M,N] through sq_w4a16_gemm_ws (workspace-backed split-K for 5 <= M <= 32)."""
+    m = x.numel() // k
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
+    if ws is None:
+        ws = workspace(max(m, 1), n, k, x.device, stream)
+    _check(lib().sq_w4a16_gemm_ws(_ptr(x), _ptr(w), _ptr(zs), _ptr(out), m, n, k, group_size, SQ_LAYOUT_L1, algo,
+                                  _ptr(ws), ws.numel(), _stream(stream)), "sq_w4a16_gemm_ws")
     return out
 
 

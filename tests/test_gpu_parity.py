@@ -326,3 +326,60 @@ def test_walinear_module():
     x = torch.randn((1, 4, k), dtype=torch.float16, device=DEV)
     ref = torch.matmul(x.float(), qf.dequant_to_fp16(lin.weight.data, 2, 64).float().t()) + lin.bias.float()
     assert (q2(x).float() - ref).abs().max() <= TOL * ref.abs().max()
+
+
+# ------------------------------------------------------------------ workspace-backed split-K kernel (5 <= M <= 32)
+def check_gemm_ws(capi, m, n, k, g, algo, seed=0):
+    d = linear(n, k, g, seed)
+    x = orc.synth_x(m, k, seed=seed + 100)
+    y_ref = orc.gemm_ref(x, d["w_hat"])
+    y = capi.gemm_ws(to_dev(x), d["w_dev"], d["zs_dev"], n, k, g, algo=algo)
+    torch.cuda.synchronize()
+    y = y.float().cpu().numpy()
+    assert np.all(np.isfinite(y))
+    assert np.max(np.abs(y - y_ref)) <= TOL * np.max(np.abs(y_ref)), (m, n, k, g, hex(algo))
+
+
+@pytest.mark.parametrize("n,k,g", SMALL_SHAPES + [(520, 1056, 32), (4096, 4096, 128)])
+@pytest.mark.parametrize("m", [5, 8, 16, 17, 32])
+def test_skinny_ws_parity(capi, n, k, g, m):
+    check_gemm_ws(capi, m, n, k, g, capi.SQ_ALGO_AUTO)
+    for ksplit in (1, 2, 4, 8):
+        for mode in (1, 2):
+            check_gemm_ws(capi, m, n, k, g, capi.SQ_ALGO_SKINNY_WS | ((ksplit | (mode << 8)) << 8))
+
+
+def test_skinny_ws_properties_and_workspace_reuse(capi):
+    n, k, g = 4096, 16384, 128
+    d = linear(n, k, g, seed=12)
+    x = to_dev(orc.synth_x(16, k, seed=13))
+    ws = capi.workspace(16, n, k, x.device)
+    y1 = capi.gemm_ws(x, d["w_dev"], d["zs_dev"], n, k, g, ws=ws)
+    # the call leaves the counters zero, so the same workspace serves the next call; results are bit-reproducible
+    assert torch.count_nonzero(ws[:65536]).item() == 0
+    for _ in range(3):
+        assert torch.equal(y1, capi.gemm_ws(x, d["w_dev"], d["zs_dev"], n, k, g, ws=ws))
+    y2 = capi.gemm_ws(x * 2, d["w_dev"], d["zs_dev"], n, k, g, ws=ws)
+    normal = y1.abs() >= 2.0 ** -13
+    assert torch.equal(y2[normal], (y1 * 2)[normal])
+    e = torch.zeros((16, k), dtype=torch.float16, device=DEV)
+    cols = [(977 * i + 5) % k for i in range(16)]
+    for i, c in enumerate(cols):
+        e[i, c] = 1.0
+    ye = capi.gemm_ws(e, d["w_dev"], d["zs_dev"], n, k, g, ws=ws).cpu().numpy()
+    for i, c in enumerate(cols):
+        assert np.array_equal(ye[i].view(np.int16), d["w_hat"][:, c].view(np.int16))
+    # a smaller problem right after a larger one on the same workspace
+    check_gemm_ws(capi, 9, 200, 1536, 64, capi.SQ_ALGO_AUTO)
+    # outside 5..32 the call falls through to the workspace-free kernels
+    check_gemm_ws(capi, 1, 256, 1024, 128, capi.SQ_ALGO_AUTO)
+    check_gemm_ws(capi, 100, 256, 1024, 128, capi.SQ_ALGO_AUTO)
+
+
+def test_skinny_ws_rejects_small_workspace(capi):
+    d = linear(256, 1024, 128, seed=0)
+    x = to_dev(orc.synth_x(16, 1024))
+    tiny = torch.zeros(1024, dtype=torch.uint8, device=DEV)
+    with pytest.raises(capi.SqError) as ei:
+        capi.gemm_ws(x, d["w_dev"], d["zs_dev"], 256, 1024, 128, ws=tiny)
+    assert ei.value.code == capi.SQ_ERR_WORKSPACE
