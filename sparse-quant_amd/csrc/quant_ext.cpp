@@ -15,6 +15,7 @@
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 
+#include <map>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -89,6 +90,24 @@ std::pair<at::Tensor, at::Tensor> l1_view_of_l2(const at::Tensor& W, const at::T
     return {w1, zs1};
 }
 
+// Workspace of the split-K kernel (5..32 tokens): one zero-initialised buffer per
+// (device, stream), grown on demand and kept for the life of the process.  Calls on one
+// stream are ordered, which is what sharing a workspace requires.  Under HIP graph capture
+// the buffer must already exist (run the call once on the capturing stream beforehand).
+std::mutex g_ws_mutex;
+std::map<std::pair<int, void*>, at::Tensor> g_workspaces;
+
+at::Tensor workspace_for(const at::Tensor& like, void* stream, size_t bytes) {
+    std::lock_guard<std::mutex> lock(g_ws_mutex);
+    const auto key = std::make_pair((int)like.device().index(), stream);
+    auto it = g_workspaces.find(key);
+    if (it != g_workspaces.end() && (size_t)it->second.numel() >= bytes) return it->second;
+    const int64_t want = (int64_t)std::max<size_t>(bytes, (size_t)1 << 20);
+    at::Tensor ws = torch::zeros({want}, like.options().dtype(at::kByte));
+    g_workspaces[key] = ws;
+    return ws;
+}
+
 at::Tensor gemm_impl(const at::Tensor& I, const at::Tensor& W, const at::Tensor& ZS, int N, int group_size,
                      int algo) {
     SQ_CHECK_DEVICE(I);
@@ -130,8 +149,17 @@ at::Tensor gemm_impl(const at::Tensor& I, const at::Tensor& W, const at::Tensor&
         w_ptr = keep.first.data_ptr();
         zs_ptr = keep.second.data_ptr();
     }
+    void* stream = current_stream(I);
+    if (M > 4 && M <= 32 && ((algo & 0xFF) == SQ_ALGO_AUTO || (algo & 0xFF) == SQ_ALGO_SKINNY_WS)) {
+        const size_t ws_bytes = sq_w4a16_workspace_bytes((int)M, N, (int)K);
+        at::Tensor ws = workspace_for(I, stream, ws_bytes);
+        raise_if_error(sq_w4a16_gemm_ws(I.data_ptr(), w_ptr, zs_ptr, O.data_ptr(), (int)M, N, (int)K, group_size,
+                                        SQ_LAYOUT_L1, algo, ws.data_ptr(), (size_t)ws.numel(), stream),
+                       "gemm_awq_ut");
+        return O;
+    }
     raise_if_error(sq_w4a16_gemm_ex(I.data_ptr(), w_ptr, zs_ptr, O.data_ptr(), (int)M, N, (int)K, group_size,
-                                    SQ_LAYOUT_L1, algo, current_stream(I)),
+                                    SQ_LAYOUT_L1, algo, stream),
                    "gemm_awq_ut");
     return O;
 }

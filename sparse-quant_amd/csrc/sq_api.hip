@@ -99,7 +99,11 @@ size_t sq_w4a16_workspace_bytes(int M, int N, int K) {
 int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
                      int layout, int algo, void* workspace, size_t workspace_bytes, void* stream) {
     const int kernel = algo & 0xFF;
-    const bool want = kernel == SQ_ALGO_SKINNY_WS || (kernel == SQ_ALGO_AUTO && M > 4 && M <= 32);
+    // Measured on OPT-6.7B shapes: the split-K kernel wins once the weight is large enough
+    // (fc1/fc2 class) for 9..32 tokens, and for 5..8 tokens when K is long.
+    const bool large = (long)N * (long)K >= (1L << 25);
+    const bool want = kernel == SQ_ALGO_SKINNY_WS ||
+                      (kernel == SQ_ALGO_AUTO && ((M > 8 && M <= 32 && large) || (M > 4 && M <= 8 && K > 8192)));
     if (!want) return sq_w4a16_gemm_ex(x, w, zs, y, M, N, K, group_size, layout, algo, stream);
     if (M < 0 || M > 32) return M < 0 ? SQ_ERR_BAD_SHAPE : SQ_ERR_BAD_ALGO;
     const int rc = check_weight(N, K, group_size, layout);

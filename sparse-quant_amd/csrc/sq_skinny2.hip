@@ -1,18 +1,27 @@
 // Skinny GEMM for 5 <= M <= 32 with a caller-provided workspace (layout L1).
-// Still HBM-bound on the weight stream; the point of this kernel is to keep the
-// activation traffic (which a 16-row tile would re-read N/16 times) below the
-// weight traffic and to have enough workgroups for any N.
+// HBM-bound on the weight stream; everything else is arranged so that the vector
+// memory pipeline sees little besides that stream.
 //
 // Mapping.  v_mfma_f32_16x16x32_f16 with the weights as the B operand straight
 // from registers (lane l: row r + l%16, k = 128c + 32*(l/16) .. +31, one 128-bit
 // load, one 32-bit word per MFMA) and the activations as the A operand (token
 // l%16, the same k).  A workgroup owns 64 weight rows and one of `ksplit` K ranges;
-// its waves take the 128-wide chunks of that range round-robin, and every wave
-// reuses one set of activation registers for the four 16-row tiles of the 64 rows,
-// so x is read once per 4 weight loads.  Partial 16x16 tiles are summed across the
-// waves in LDS.  With ksplit > 1 each workgroup writes its fp32 partial tile to the
-// workspace and bumps a per-row-block counter; the workgroup that arrives last adds
-// the partials in a fixed order (bit-reproducible), writes Y and resets the counter.
+// its waves take pairs of 128-wide chunks of that range round-robin, and every wave
+// reuses one set of activation registers for the four 16-row tiles of the 64 rows.
+//
+// Activations: a lane needs 64 contiguous bytes of one token per chunk, which as a
+// direct load touches one cache line per lane.  Instead each wave loads its chunk
+// row-contiguously (16 lanes x 16 bytes = the 256 bytes of one token) and turns it
+// into operand order through a wave-private LDS buffer (pitch 272 bytes: both the
+// row-contiguous writes and the operand-order reads are bank-conflict free).
+// Zeros/scales of the workgroup's rows and K range are staged in LDS once, with
+// row-contiguous loads, when they fit (32 groups per row); otherwise lanes fetch
+// them per chunk.
+//
+// Partial 16x16 tiles are summed across the waves in LDS.  With ksplit > 1 each
+// workgroup writes its fp32 partial tile to the workspace and bumps a per-row-block
+// counter; the workgroup that arrives last adds the partials in a fixed order
+// (bit-reproducible), writes Y and resets the counter.
 //
 // Arithmetic modes as in the GEMV kernel: exact (per-weight fp16 (q-z)*s, any group
 // size) and, for g == 128 (one group per chunk), fixup: 64+q into the matrix core
@@ -23,16 +32,29 @@
 namespace sq {
 
 constexpr int SK2_COUNTER_BYTES = 65536;  // start of the workspace: one uint32 per 64-row block
+constexpr int SK2_XPITCH = 272;           // bytes per staged token row (256 + 16)
+constexpr int SK2_ZCOLS = 32;             // groups per row held in LDS
+constexpr int SK2_ZPITCH = 33;
 
-template <int MT, int NWV, bool FIXUP>
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int MT, int NWV, int S, bool FIXUP>
 __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __restrict__ W,
                                                            const half2_t* __restrict__ ZS,
                                                            const half_t* __restrict__ X, half_t* __restrict__ Y,
                                                            float* part, unsigned* counters, int M, int N, int K,
                                                            int gshift, int ksplit) {
     constexpr int TILE = 4 * MT * 4 * 64;  // floats a wave contributes: [rt][mt][v][lane]
-    __shared__ float red[NWV * TILE];
+    constexpr int XBUF = MT * 16 * SK2_XPITCH;
+    constexpr int SH_BYTES = NWV * XBUF > NWV * TILE * 4 ? NWV * XBUF : NWV * TILE * 4;
+    __shared__ __attribute__((aligned(16))) uint8_t sh[SH_BYTES];  // activation staging, later the wave partials
+    __shared__ uint32_t zsl[64 * SK2_ZPITCH];
     __shared__ unsigned last_flag;
+    float* red = (float*)sh;
 
     const NibbleMasks nm = nibble_masks();
     const int tid = threadIdx.x;
@@ -47,6 +69,24 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
     const int cps = (nchunks + ksplit - 1) / ksplit;
     const int c_begin = ks * cps;
     const int c_end = imin(c_begin + cps, nchunks);
+    const int gpc_shift = 7 - gshift;  // groups per chunk = 1 << gpc_shift
+    const int g_begin = c_begin << gpc_shift;
+    const int ng = imin((c_end - c_begin) << gpc_shift, groups - g_begin);
+    const bool zs_lds = ng > 0 && ng <= SK2_ZCOLS;
+
+    // Zeros/scales of the row block: loaded now (row-contiguous), parked in LDS after the
+    // first weight loads have been issued so that they do not delay the weight stream.
+    constexpr int ZPT = (64 * SK2_ZCOLS) / (64 * NWV);
+    uint32_t zreg[ZPT];
+    if (zs_lds) {
+#pragma unroll
+        for (int p = 0; p < ZPT; p++) {
+            const int idx = tid + p * 64 * NWV;
+            const int r = idx >> 5, col = idx & 31;
+            const int row = imin(rb * 64 + r, N - 1);
+            zreg[p] = ((const uint32_t*)ZS)[(long)row * groups + g_begin + (col < ng ? col : 0)];
+        }
+    }
 
     float4_t acc[4][MT];
 #pragma unroll
@@ -57,89 +97,133 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
                           (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
 
     const uint8_t* wrow[4];
-    const half2_t* zrow[4];
+    const uint32_t* zrow[4];
 #pragma unroll
     for (int rt = 0; rt < 4; rt++) {
         const int row = imin(rb * 64 + 16 * rt + li, N - 1);
         wrow[rt] = W + (long)row * (K >> 1);
-        zrow[rt] = ZS + (long)row * groups;
+        zrow[rt] = (const uint32_t*)ZS + (long)row * groups;
     }
+    uint8_t* xb = sh + wave * XBUF;
+    uint8_t* xb_wr = xb + (lane >> 4) * SK2_XPITCH + (lane & 15) * 16;  // token lane/16 (+4j), 16-byte column lane%16
+    const uint8_t* xb_rd = xb + li * SK2_XPITCH + lj * 64;              // token li (+16mt), k = 32 lj (+8t)
 
-    // Two chunks per trip: all eight weight loads are issued before the first use.
-    for (int c0 = c_begin + 2 * wave; c0 < c_end; c0 += 2 * NWV) {
-        u32x4_t wq[2][4];
-        half2_t zq[2][4];
-        int kcs[2];
-        bool valid[2];
+    // S chunks per wave and trip; every weight load of the trip is issued before the first
+    // use, the activations run one chunk ahead.  The trip count is uniform over the waves
+    // (the zeros/scales hand-over contains a barrier); a wave without chunks idles.
+    bool first = true;
+    for (int cb = c_begin; cb < c_end; cb += S * NWV) {
+        const int c0 = cb + S * wave;
+        const bool active = c0 < c_end;
+        u32x4_t wq[S][4];
+        u32x4_t xr[2][4 * MT];
+        uint32_t zq[S][4];
+        int zcol[S];
+        auto load_x = [&](int c, u32x4_t* dst) {
+            const int kx = (c << 7) + 8 * (lane & 15);
+            const bool xvalid = (c < c_end) && (kx < K);
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
-            const int kk = ((c0 + u) << 7) + 32 * lj;
-            valid[u] = (c0 + u < c_end) && (kk < K);
-            kcs[u] = valid[u] ? kk : 0;
-#pragma unroll
-            for (int rt = 0; rt < 4; rt++) {
-                wq[u][rt] = __builtin_nontemporal_load((const u32x4_t*)(wrow[rt] + (kcs[u] >> 1)));
-                zq[u][rt] = zrow[rt][kcs[u] >> gshift];
+            for (int j = 0; j < 4 * MT; j++) {
+                const int tok = imin(4 * j + (lane >> 4), M - 1);
+                const u32x4_t v = *(const u32x4_t*)(X + (long)tok * K + (xvalid ? kx : 0));
+                dst[j] = xvalid ? v : (u32x4_t){0u, 0u, 0u, 0u};
             }
+        };
+        if (active) {
+#pragma unroll
+            for (int u = 0; u < S; u++) {
+                const int c = c0 + u;
+                const int kk = (c << 7) + 32 * lj;
+                const bool valid = (c < c_end) && (kk < K);
+                const int kc = valid ? kk : 0;
+#pragma unroll
+                for (int rt = 0; rt < 4; rt++)
+                    wq[u][rt] = __builtin_nontemporal_load((const u32x4_t*)(wrow[rt] + (kc >> 1)));
+                zcol[u] = valid ? (((c - c_begin) << gpc_shift) + ((32 * lj) >> gshift)) : 0;
+                if (!zs_lds) {
+#pragma unroll
+                    for (int rt = 0; rt < 4; rt++) zq[u][rt] = zrow[rt][valid ? (kk >> gshift) : g_begin];
+                }
+            }
+            load_x(c0, xr[0]);
         }
+        if (first) {
+            if (zs_lds) {
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
-            u32x4_t xa[MT][4];
-#pragma unroll
-            for (int mt = 0; mt < MT; mt++) {
-                const u32x4_t* xp = (const u32x4_t*)(X + (long)imin(16 * mt + li, M - 1) * K + kcs[u]);
-#pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    const u32x4_t v = xp[t];
-                    xa[mt][t] = valid[u] ? v : (u32x4_t){0u, 0u, 0u, 0u};
+                for (int p = 0; p < ZPT; p++) {
+                    const int idx = tid + p * 64 * NWV;
+                    zsl[(idx >> 5) * SK2_ZPITCH + (idx & 31)] = zreg[p];
                 }
             }
-            float4_t xs[MT];
-            if (FIXUP) {
+            __syncthreads();
+            first = false;
+        }
+        if (active) {
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    xs[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+            for (int u = 0; u < S; u++) {
+                if (u + 1 < S) load_x(c0 + u + 1, xr[(u + 1) & 1]);
+                wave_lds_sync();  // the previous chunk's operand reads are done
 #pragma unroll
-                    for (int t = 0; t < 4; t++)
-                        xs[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<half8_t>(xa[mt][t]), ones, xs[mt], 0, 0,
-                                                                        0);
+                for (int j = 0; j < 4 * MT; j++) *(u32x4_t*)(xb_wr + 4 * j * SK2_XPITCH) = xr[u & 1][j];
+                wave_lds_sync();
+                u32x4_t xa[MT][4];
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                    for (int t = 0; t < 4; t++) xa[mt][t] = *(const u32x4_t*)(xb_rd + 16 * mt * SK2_XPITCH + 16 * t);
+                if (zs_lds) {
+#pragma unroll
+                    for (int rt = 0; rt < 4; rt++) zq[u][rt] = zsl[(16 * rt + li) * SK2_ZPITCH + zcol[u]];
                 }
-            }
+                float4_t xs[MT];
+                if (FIXUP) {
 #pragma unroll
-            for (int rt = 0; rt < 4; rt++) {
-                if (!FIXUP) {
-                    const half2_t z64 = {zq[u][rt].x, zq[u][rt].x};
-                    const half2_t sc = {zq[u][rt].y, zq[u][rt].y};
+                    for (int mt = 0; mt < MT; mt++) {
+                        xs[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int t = 0; t < 4; t++) {
-                        const half8_t wv = dequant8(wq[u][rt][t], z64, sc, nm);
+                        for (int t = 0; t < 4; t++)
+                            xs[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<half8_t>(xa[mt][t]), ones, xs[mt], 0,
+                                                                            0, 0);
+                    }
+                }
+#pragma unroll
+                for (int rt = 0; rt < 4; rt++) {
+                    const half2_t zsv = bit_cast<half2_t>(zq[u][rt]);
+                    if (!FIXUP) {
+                        const half2_t z64 = {zsv.x, zsv.x};
+                        const half2_t sc = {zsv.y, zsv.y};
+#pragma unroll
+                        for (int t = 0; t < 4; t++) {
+                            const half8_t wv = dequant8(wq[u][rt][t], z64, sc, nm);
+#pragma unroll
+                            for (int mt = 0; mt < MT; mt++)
+                                acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<half8_t>(xa[mt][t]), wv,
+                                                                                     acc[rt][mt], 0, 0, 0);
+                        }
+                    } else {
+                        float4_t tmp[MT];
+#pragma unroll
+                        for (int mt = 0; mt < MT; mt++) tmp[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int t = 0; t < 4; t++) {
+                            const half8_t wv = unpack8_raw(wq[u][rt][t], nm);
+#pragma unroll
+                            for (int mt = 0; mt < MT; mt++)
+                                tmp[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<half8_t>(xa[mt][t]), wv,
+                                                                                 tmp[mt], 0, 0, 0);
+                        }
+                        const float zf = (float)zsv.x;
+                        const float sf = (float)zsv.y;
 #pragma unroll
                         for (int mt = 0; mt < MT; mt++)
-                            acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<half8_t>(xa[mt][t]), wv,
-                                                                                 acc[rt][mt], 0, 0, 0);
+#pragma unroll
+                            for (int v = 0; v < 4; v++) acc[rt][mt][v] += sf * (tmp[mt][v] - zf * xs[mt][v]);
                     }
-                } else {
-                    float4_t tmp[MT];
-#pragma unroll
-                    for (int mt = 0; mt < MT; mt++) tmp[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int t = 0; t < 4; t++) {
-                        const half8_t wv = unpack8_raw(wq[u][rt][t], nm);
-#pragma unroll
-                        for (int mt = 0; mt < MT; mt++)
-                            tmp[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<half8_t>(xa[mt][t]), wv, tmp[mt],
-                                                                             0, 0, 0);
-                    }
-                    const float zf = (float)zq[u][rt].x;
-                    const float sf = (float)zq[u][rt].y;
-#pragma unroll
-                    for (int mt = 0; mt < MT; mt++)
-#pragma unroll
-                        for (int v = 0; v < 4; v++) acc[rt][mt][v] += sf * (tmp[mt][v] - zf * xs[mt][v]);
                 }
             }
         }
     }
+    __syncthreads();  // every wave is done with its staging buffer, which the partials now overwrite
 
     // Sum the waves' partial tiles: red[wave][rt][mt][v][lane].
 #pragma unroll
@@ -198,37 +282,29 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
     if (tid == 0) __hip_atomic_store(&counters[rb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-static int pick_ksplit(int N, int K, int nwv) {
-    const int nchunks = (K + 127) / 128;
-    const int row_blocks = (N + 63) / 64;
-    int ks = 1;
-    // enough workgroups for 256 CUs, but at least one chunk per wave and at most 8 partials
-    while (ks < 8 && row_blocks * ks < 256 && nchunks / (ks * 2) >= nwv) ks *= 2;
-    return ks;
-}
-
 size_t skinny2_workspace_bytes(int M, int N, int K) {
     const int mt = (M + 15) / 16;
     const int row_blocks = (N + 63) / 64;
     return (size_t)SK2_COUNTER_BYTES + (size_t)8 * row_blocks * (4 * mt * 4 * 64) * sizeof(float);
 }
 
-template <int MT, int NWV>
+template <int MT, int NWV, int S>
 static hipError_t launch_cfg(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                              int gshift, bool fixup, int ksplit, hipStream_t st) {
     const dim3 grid((N + 63) / 64, ksplit);
     unsigned* counters = (unsigned*)ws;
     float* part = (float*)((char*)ws + SK2_COUNTER_BYTES);
     if (fixup)
-        hipLaunchKernelGGL((skinny2_kernel<MT, NWV, true>), grid, dim3(64 * NWV), 0, st, (const uint8_t*)w,
+        hipLaunchKernelGGL((skinny2_kernel<MT, NWV, S, true>), grid, dim3(64 * NWV), 0, st, (const uint8_t*)w,
                            (const half2_t*)zs, (const half_t*)x, (half_t*)y, part, counters, M, N, K, gshift, ksplit);
     else
-        hipLaunchKernelGGL((skinny2_kernel<MT, NWV, false>), grid, dim3(64 * NWV), 0, st, (const uint8_t*)w,
+        hipLaunchKernelGGL((skinny2_kernel<MT, NWV, S, false>), grid, dim3(64 * NWV), 0, st, (const uint8_t*)w,
                            (const half2_t*)zs, (const half_t*)x, (half_t*)y, part, counters, M, N, K, gshift, ksplit);
     return hipGetLastError();
 }
 
-// tune = 0 for the heuristic, else ksplit (1,2,4,8) | mode << 8 (1 = exact, 2 = fixup).
+// tune = 0 for the heuristic, else ksplit (1,2,4,8) | mode << 8 (1 = exact, 2 = fixup) |
+// waves << 12 (4, 8; M <= 16).
 // The first 64 KiB of the workspace are counters and must be zero before the first call;
 // every call leaves them zero.
 hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
@@ -236,14 +312,24 @@ hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, vo
     int gshift = 0;
     while ((1 << gshift) < g) gshift++;
     const int mt = (M + 15) / 16;
-    const int nwv = mt == 1 ? 8 : 4;
+    const int nchunks = (K + 127) / 128;
+    const int row_blocks = (N + 63) / 64;
     int ksplit = tune & 0xFF;
-    if (ksplit != 1 && ksplit != 2 && ksplit != 4 && ksplit != 8) ksplit = pick_ksplit(N, K, nwv);
-    const int mode = (tune >> 8) & 0xFF;
+    int nwv = (tune >> 12) & 0xF;
+    if (ksplit != 1 && ksplit != 2 && ksplit != 4 && ksplit != 8) {
+        // about one workgroup per CU, each K range at least 8 chunks long
+        ksplit = 1;
+        while (ksplit < 8 && row_blocks * ksplit < 256 && nchunks / (ksplit * 2) >= 8) ksplit *= 2;
+    }
+    const int cps = (nchunks + ksplit - 1) / ksplit;
+    if (nwv != 4 && nwv != 8) nwv = (mt == 1 && cps >= 16) ? 8 : 4;
+    if (mt == 2) nwv = 4;
+    const int mode = (tune >> 8) & 0xF;
     bool fixup = (g == 128);
     if (mode == 1) fixup = false;
-    if (mt == 1) return launch_cfg<1, 8>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, st);
-    return launch_cfg<2, 4>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, st);
+    if (mt == 2) return launch_cfg<2, 4, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, st);
+    if (nwv == 8) return launch_cfg<1, 8, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, st);
+    return launch_cfg<1, 4, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, st);
 }
 
 }  // namespace sq

@@ -381,5 +381,38 @@ def test_skinny_ws_rejects_small_workspace(capi):
     x = to_dev(orc.synth_x(16, 1024))
     tiny = torch.zeros(1024, dtype=torch.uint8, device=DEV)
     with pytest.raises(capi.SqError) as ei:
-        capi.gemm_ws(x, d["w_dev"], d["zs_dev"], 256, 1024, 128, ws=tiny)
+        capi.gemm_ws(x, d["w_dev"], d["zs_dev"], 256, 1024, 128, algo=capi.SQ_ALGO_SKINNY_WS, ws=tiny)
     assert ei.value.code == capi.SQ_ERR_WORKSPACE
+    # where the dispatcher picks a workspace-free kernel the workspace is not looked at
+    capi.gemm_ws(x, d["w_dev"], d["zs_dev"], 256, 1024, 128, ws=tiny)
+
+
+@pytest.mark.parametrize("n,k", [(16384, 4096), (4096, 16384), (4096, 4096)])
+@pytest.mark.parametrize("m", [8, 16, 32])
+def test_quant_extension_decode_batches_use_workspace_path(n, k, m):
+    # gemm_awq_ut on decode batches of the fc1 / fc2 shapes goes through sq_w4a16_gemm_ws with the
+    # extension's own cached workspace; also replayed from a HIP graph (several replays, same bits).
+    import quant
+    g = 128
+    d = linear(n, k, g, seed=21)
+    x = to_dev(orc.synth_x(m, k, seed=22)).reshape(1, m, k)
+    y_ref = orc.gemm_ref(x.reshape(m, k).cpu().numpy(), d["w_hat"])
+    y = quant.gemm_awq_ut(x, d["w_dev"], d["zs_dev"], m, n, k, g)
+    assert y.shape == (1, m, n)
+    err = np.max(np.abs(y.float().cpu().numpy().reshape(m, n) - y_ref))
+    assert err <= TOL * np.max(np.abs(y_ref))
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        y_warm = quant.gemm_awq_ut(x, d["w_dev"], d["zs_dev"], m, n, k, g)  # creates this stream's workspace
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            y_graph = quant.gemm_awq_ut(x, d["w_dev"], d["zs_dev"], m, n, k, g)
+    assert torch.equal(y_warm, y)
+    for _ in range(3):
+        y_graph.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_graph, y)
