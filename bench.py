@@ -241,30 +241,65 @@ def main():
 
 
 def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10):
-    """TFLOP/s of the M=2048 linears of the same layer (BASELINE.json configs[2])."""
+    """TFLOP/s of the M=2048 linears of the same layer (BASELINE.json configs[2]).
+
+    Reported beside each figure: the library's dense fp16 GEMM (torch.matmul, no int4 work at all) on
+    the same shape in the same run, and the shader clock the chip sustains while the kernel runs
+    (a one-wave probe on a second stream).  Matrix-heavy kernels run power-limited on this part, so the
+    fraction of the nominal-clock peak is bounded well below 1 for any kernel; the dense figure shows
+    where that bound sits for these shapes."""
     res = {}
-    flops_total, time_total = 0.0, 0.0
+    flops_total, time_total, dense_time_total = 0.0, 0.0, 0.0
+    side = torch.cuda.Stream(device=dev)
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(reps):
+            fn()
+        e1.record(stream)
+        stream.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
+
+    def clock_under(fn, us):
+        n = max(8, int(3000.0 / us))           # about 3 ms of load on either side of the probe
+        for _ in range(n):
+            fn()
+        with torch.cuda.stream(side):
+            ticks = capi.clock_probe(spins=200000, stream=side)
+        for _ in range(2 * n):
+            fn()
+        torch.cuda.synchronize()
+        c, r = int(ticks[0].item()), int(ticks[1].item())
+        return round(c / (r / 100.0)) if r else None
+
     with torch.cuda.stream(stream):
         for (w, zs), (name, n, k) in list(zip(layer, shapes))[3:]:
             x = torch.randn((m, k), device=dev, generator=gen).half()
             y = torch.empty((m, n), dtype=torch.float16, device=dev)
-            for _ in range(3):
-                capi.gemm(x, w, zs, n, k, g, out=y, stream=stream)
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(reps):
-                capi.gemm(x, w, zs, n, k, g, out=y, stream=stream)
-            e1.record(stream)
-            stream.synchronize()
-            us = e0.elapsed_time(e1) * 1e3 / reps
+            wd = torch.randn((k, n), device=dev, generator=gen).half()
+            run = lambda: capi.gemm(x, w, zs, n, k, g, out=y, stream=stream)
+            dense = lambda: torch.matmul(x, wd, out=y)
+            us = timed(run)
+            us_dense = timed(dense)
             fl = 2.0 * m * n * k
-            res[name] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 1)}
+            res[name] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
+                         "shader_mhz_under_load": clock_under(run, us),
+                         "dense_fp16_library_us": round(us_dense, 1),
+                         "dense_fp16_library_tflops": round(fl / us_dense / 1e6, 1),
+                         "dense_fp16_library_shader_mhz": clock_under(dense, us_dense)}
             flops_total += fl
             time_total += us
+            dense_time_total += us_dense
+            del wd
     tf = flops_total / time_total / 1e6
+    tfd = flops_total / dense_time_total / 1e6
     return {"m": m, "tflops": round(tf, 1), "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
-            "per_linear": res}
+            "dense_fp16_library_tflops": round(tfd, 1), "vs_dense_fp16_library": round(tf / tfd, 3),
+            "nominal_shader_mhz": 2400, "per_linear": res}
 
 
 def fused_qkv_leg(torch, capi, m, g, dev, gen, stream, layers, bytes_per_step):

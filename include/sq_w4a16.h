@@ -139,6 +139,14 @@ int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out,
                          int lut_elem_bytes, int Z, int H, int S, int D, int nnz, float sm_scale, int causal,
                          void* stream);
 
+/* Diagnostic, no counterpart in the reference: a single wave spins for `spins`
+ * (1 .. 2^26) dependent multiply-adds and writes three uint64 to out: shader-clock
+ * ticks elapsed, ticks of the constant 100 MHz counter elapsed, and a dummy.  Run on
+ * a second stream beside a kernel it gives the clock the chip sustains under that
+ * kernel's load (matrix-heavy kernels run power-limited, well below the nominal
+ * clock that published peak rates assume). */
+int sq_clock_probe(void* out, int spins, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -187,4 +187,10 @@ int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out,
                                                 static_cast<hipStream_t>(stream)));
 }
 
+int sq_clock_probe(void* out, int spins, void* stream) {
+    if (!out) return SQ_ERR_NULL_POINTER;
+    if (spins <= 0 || spins > (1 << 26)) return SQ_ERR_BAD_SHAPE;
+    return launch_code(sq::launch_clock_probe(out, spins, static_cast<hipStream_t>(stream)));
+}
+
 }  // extern "C"

@@ -209,13 +209,27 @@ static hipError_t launch_mi(const void* x, const void* w, const void* zs, void* 
     return hipGetLastError();
 }
 
-// tune = 0 for the heuristic, else the number of 32-row tiles per workgroup (1, 2 or 4).
+// tune = 0 for the heuristic, else the number of 32-row tiles per workgroup (1, 2 or 4), or 8 / 9 / 10 for
+// the software-pipelined kernel (128 rows at two waves per SIMD, 128 rows at one, 256 rows at one).
 hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
                              int tune, hipStream_t st) {
     int gshift = 0;
     while ((1 << gshift) < g) gshift++;
     int mi = tune & 0xFF;
-    if (mi != 1 && mi != 2 && mi != 4) mi = M > 64 ? 4 : (M > 32 ? 2 : 1);
+    if (mi >= 8 && mi <= 10) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, mi - 8, st);
+    if (mi != 1 && mi != 2 && mi != 4) {
+        if (M > 64) {
+            // Measured on MI355X (the chip runs these kernels at a power-limited clock, so fewer
+            // instructions per flop is what counts): the 256-row tile halves the unpack work per
+            // flop and wins whenever its grid fills the 256 CUs evenly; otherwise the 128-row
+            // tiles, pipelined variant for long K.
+            const long t256 = (long)((N + 255) / 256) * ((M + 255) / 256);
+            const long rounds = (t256 + 255) / 256;
+            if (t256 * 10 >= rounds * 256 * 8) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, 2, st);
+            if (K >= 8192) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, 1, st);
+        }
+        mi = M > 64 ? 4 : (M > 32 ? 2 : 1);
+    }
     switch (mi) {
         case 1: return launch_mi<1>(x, w, zs, y, M, N, K, gshift, st);
         case 2: return launch_mi<2>(x, w, zs, y, M, N, K, gshift, st);

@@ -19,6 +19,7 @@ hipError_t launch_awq_to_lmdeploy(const void* src, void* dst, int K, int N, hipS
 hipError_t launch_l2_to_l1(const void* w_l2, const void* zs_l2, void* w_l1, void* zs_l1, int N, int K, int g,
                            hipStream_t st);
 hipError_t launch_2bit_to_4bit(const void* src, void* dst, int N, int K, hipStream_t st);
+hipError_t launch_clock_probe(void* out, int spins, hipStream_t st);
 
 // The *_tuned launchers take a kernel-specific tuning word (0 = built-in heuristic).
 // sq_gemv.hip: M <= 8.  tune = row steps per workgroup (1,2,4) | waves << 8.
@@ -38,6 +39,10 @@ hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, vo
 // sq_gemm.hip: any M.  tune = 32-row tiles per workgroup (1,2,4).
 hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
                              int tune, hipStream_t st);
+
+// sq_gemm2.hip: software-pipelined 128 x 256 tile variant for M > 64.
+hipError_t launch_gemm_pipe(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
+                            int variant, hipStream_t st);
 
 // sq_attn.hip: LUT block-sparse attention, prefill.  D in {64, 128}; lut int32 or int64 [H, ceil(S/64), nnz].
 hipError_t launch_lut_attention(const void* q, const void* k, const void* v, void* o, const void* lut,

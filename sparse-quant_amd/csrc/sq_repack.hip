@@ -166,4 +166,27 @@ hipError_t launch_2bit_to_4bit(const void* src, void* dst, int N, int K, hipStre
     return hipGetLastError();
 }
 
+// Diagnostic: one wave spins for `spins` dependent multiply-adds and reports how many
+// shader-clock ticks and how many ticks of the constant 100 MHz counter went by, so that a
+// caller running it beside a kernel on another stream can read the clock the chip sustains
+// under that kernel's load.
+__global__ void clock_probe_kernel(unsigned long long* out, int spins) {
+    const unsigned long long c0 = __builtin_readcyclecounter();
+    const unsigned long long r0 = wall_clock64();
+    float a = (float)threadIdx.x;
+    for (int i = 0; i < spins; i++) a = a * 1.0001f + 0.5f;
+    const unsigned long long c1 = __builtin_readcyclecounter();
+    const unsigned long long r1 = wall_clock64();
+    if (threadIdx.x == 0) {
+        out[0] = c1 - c0;
+        out[1] = r1 - r0;
+        out[2] = (unsigned long long)a;
+    }
+}
+
+hipError_t launch_clock_probe(void* out, int spins, hipStream_t st) {
+    hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, st, (unsigned long long*)out, spins);
+    return hipGetLastError();
+}
+
 }  // namespace sq

@@ -23,7 +23,7 @@ LIB_PATH = os.path.join(PKG_ROOT, "libsq_w4a16.so")
 EXT_PATH = os.path.join(PKG_ROOT, "quant" + sysconfig.get_config_var("EXT_SUFFIX"))
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-HIP_SOURCES = ["sq_api.hip", "sq_dequant.hip", "sq_repack.hip", "sq_gemv.hip", "sq_gemv2.hip", "sq_skinny.hip", "sq_skinny2.hip", "sq_gemm.hip",
+HIP_SOURCES = ["sq_api.hip", "sq_dequant.hip", "sq_repack.hip", "sq_gemv.hip", "sq_gemv2.hip", "sq_skinny.hip", "sq_skinny2.hip", "sq_gemm.hip", "sq_gemm2.hip",
                "sq_attn.hip"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
              # keep the compiler from forming packed-fp32 instructions

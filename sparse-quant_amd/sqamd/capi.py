@@ -34,6 +34,7 @@ SIGNATURES = {
     "sq_convert_awq_to_lmdeploy": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_repack_l2_to_l1": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "sq_convert_2bit_to_4bit": (_i, [_vp, _vp, _i, _i, _vp]),
+    "sq_clock_probe": (_i, [_vp, _i, _vp]),
     "sq_lut_attention_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, ctypes.c_float, _i, _vp]),
 }
 
@@ -169,4 +170,13 @@ def lut_attention(q, k, v, lut, sm_scale, causal, stream=None):
     _check(lib().sq_lut_attention_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lut), lut.element_size(), z, h, s, d,
                                       lut.shape[-1], float(sm_scale), int(bool(causal)), _stream(stream)),
            "sq_lut_attention_fwd")
+    return out
+
+
+def clock_probe(spins=400000, stream=None):
+    """Launch the clock probe on `stream`; returns the uint64[3] result tensor (read it after a sync):
+    shader ticks, 100 MHz ticks, dummy."""
+    dev = torch.device("cuda", torch.cuda.current_device())
+    out = torch.zeros(3, dtype=torch.int64, device=dev)
+    _check(lib().sq_clock_probe(_ptr(out), int(spins), _stream(stream)), "sq_clock_probe")
     return out

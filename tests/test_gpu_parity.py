@@ -111,7 +111,7 @@ def test_gemm_parity_small(capi, n, k, g, m):
     check_gemm(capi, m, n, k, g, capi.SQ_ALGO_GEMM)
 
 
-@pytest.mark.parametrize("mi", [1, 2, 4])
+@pytest.mark.parametrize("mi", [1, 2, 4, 8, 9, 10])
 def test_gemm_every_tile_height_is_correct(capi, mi):
     for m in (5, 70, 260):
         check_gemm(capi, m, 264, 704, 64, capi.SQ_ALGO_GEMM | (mi << 8))
