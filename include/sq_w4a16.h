@@ -89,6 +89,24 @@ int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y,
 /* Bytes sq_w4a16_gemm_ws needs for this shape (grows with N; M is capped at 32). */
 size_t sq_w4a16_workspace_bytes(int M, int N, int K);
 
+/* The same product with the element-wise tail of the linear folded into the kernel's
+ * store: Y = act(X * W_hat^T + bias) + residual, computed on the fp32 accumulator and
+ * rounded to fp16 once.  bias fp16 [N] or NULL; residual fp16 [M, N] or NULL (must not
+ * overlap y); act SQ_ACT_NONE or SQ_ACT_RELU.  workspace may be NULL (then the
+ * workspace-free kernels are used); otherwise as for sq_w4a16_gemm_ws.  Replaces the
+ * separate `out + bias` of WALinear.forward (reference:
+ * test/nvidia/module/qlinear/qlinear.py:69-70), the ReLU after fc1 and the residual
+ * adds of the decoder layer (reference:
+ * test/nvidia/module/opt/modeling_opt_ours.py:590,608-609,614), in the role of the
+ * fused gemm_awq_residual_ut family the reference scripts import from a package that
+ * is not part of it (quantization/nvidia/script/gemm_awq_test.py). */
+#define SQ_ACT_NONE 0
+#define SQ_ACT_RELU 1
+int sq_w4a16_gemm_fused(const void* x, const void* w, const void* zs, const void* bias,
+                        const void* residual, void* y, int M, int N, int K, int group_size,
+                        int layout, int act, int algo, void* workspace, size_t workspace_bytes,
+                        void* stream);
+
 /* out[N,K] (fp16) = W_hat in natural k order, bit-identical to fp16
  * (q_fp16 - z_fp16) * s_fp16.  Replaces dequant
  * (reference: quantization/tianshu/backend/gemm_quant.cu:153-164 and

@@ -108,8 +108,9 @@ at::Tensor workspace_for(const at::Tensor& like, void* stream, size_t bytes) {
     return ws;
 }
 
-at::Tensor gemm_impl(const at::Tensor& I, const at::Tensor& W, const at::Tensor& ZS, int N, int group_size,
-                     int algo) {
+at::Tensor gemm_impl(const at::Tensor& I, const at::Tensor& W, const at::Tensor& ZS, int N, int group_size, int algo,
+                     const c10::optional<at::Tensor>& bias = c10::nullopt,
+                     const c10::optional<at::Tensor>& residual = c10::nullopt, int act = SQ_ACT_NONE) {
     SQ_CHECK_DEVICE(I);
     SQ_CHECK_DEVICE(W);
     SQ_CHECK_DEVICE(ZS);
@@ -149,17 +150,33 @@ at::Tensor gemm_impl(const at::Tensor& I, const at::Tensor& W, const at::Tensor&
         w_ptr = keep.first.data_ptr();
         zs_ptr = keep.second.data_ptr();
     }
-    void* stream = current_stream(I);
-    if (M > 4 && M <= 32 && ((algo & 0xFF) == SQ_ALGO_AUTO || (algo & 0xFF) == SQ_ALGO_SKINNY_WS)) {
-        const size_t ws_bytes = sq_w4a16_workspace_bytes((int)M, N, (int)K);
-        at::Tensor ws = workspace_for(I, stream, ws_bytes);
-        raise_if_error(sq_w4a16_gemm_ws(I.data_ptr(), w_ptr, zs_ptr, O.data_ptr(), (int)M, N, (int)K, group_size,
-                                        SQ_LAYOUT_L1, algo, ws.data_ptr(), (size_t)ws.numel(), stream),
-                       "gemm_awq_ut");
-        return O;
+    const void* bias_ptr = nullptr;
+    const void* res_ptr = nullptr;
+    if (bias.has_value() && bias->defined()) {
+        SQ_CHECK_DEVICE((*bias));
+        SQ_CHECK_CONTIGUOUS((*bias));
+        SQ_CHECK_DTYPE((*bias), at::kHalf);
+        if (bias->numel() != N) throw std::invalid_argument("bias must have N elements!");
+        bias_ptr = bias->data_ptr();
     }
-    raise_if_error(sq_w4a16_gemm_ex(I.data_ptr(), w_ptr, zs_ptr, O.data_ptr(), (int)M, N, (int)K, group_size,
-                                    SQ_LAYOUT_L1, algo, stream),
+    if (residual.has_value() && residual->defined()) {
+        SQ_CHECK_DEVICE((*residual));
+        SQ_CHECK_CONTIGUOUS((*residual));
+        SQ_CHECK_DTYPE((*residual), at::kHalf);
+        if (residual->numel() != M * (int64_t)N) throw std::invalid_argument("residual must have M*N elements!");
+        res_ptr = residual->data_ptr();
+    }
+    void* stream = current_stream(I);
+    void* ws_ptr = nullptr;
+    size_t ws_bytes = 0;
+    at::Tensor ws;
+    if (M > 4 && M <= 32 && ((algo & 0xFF) == SQ_ALGO_AUTO || (algo & 0xFF) == SQ_ALGO_SKINNY_WS)) {
+        ws = workspace_for(I, stream, sq_w4a16_workspace_bytes((int)M, N, (int)K));
+        ws_ptr = ws.data_ptr();
+        ws_bytes = (size_t)ws.numel();
+    }
+    raise_if_error(sq_w4a16_gemm_fused(I.data_ptr(), w_ptr, zs_ptr, bias_ptr, res_ptr, O.data_ptr(), (int)M, N, (int)K,
+                                       group_size, SQ_LAYOUT_L1, act, algo, ws_ptr, ws_bytes, stream),
                    "gemm_awq_ut");
     return O;
 }
@@ -172,6 +189,28 @@ at::Tensor gemm_awq_ut(at::Tensor I, at::Tensor W, at::Tensor W_zeros_scales, co
     (void)M;
     (void)K;
     return gemm_impl(I, W, W_zeros_scales, N, group_size, SQ_ALGO_AUTO);
+}
+
+// I W_hat^T + R in one launch; R [bs, seq, N] fp16.  Call shape of the fused variant the
+// reference's kernel test imports (reference: quantization/nvidia/script/gemm_awq_test.py:63-65).
+at::Tensor gemm_awq_residual_ut(at::Tensor I, at::Tensor W, at::Tensor W_zeros_scales, at::Tensor R, const int M,
+                                const int N, const int K, const int group_size) {
+    (void)M;
+    (void)K;
+    return gemm_impl(I, W, W_zeros_scales, N, group_size, SQ_ALGO_AUTO, c10::nullopt, R, SQ_ACT_NONE);
+}
+
+// act(I W_hat^T + bias) + residual in one launch; bias [N] / residual [bs, seq, N] optional,
+// act "none" or "relu".
+at::Tensor gemm_awq_fused_ut(at::Tensor I, at::Tensor W, at::Tensor W_zeros_scales, c10::optional<at::Tensor> bias,
+                             c10::optional<at::Tensor> residual, const std::string& act, const int N,
+                             const int group_size) {
+    int a = SQ_ACT_NONE;
+    if (act == "relu")
+        a = SQ_ACT_RELU;
+    else if (act != "none" && !act.empty())
+        throw std::invalid_argument("unknown activation: " + act);
+    return gemm_impl(I, W, W_zeros_scales, N, group_size, SQ_ALGO_AUTO, bias, residual, a);
 }
 
 // Same with an explicit kernel id (SQ_ALGO_* | tuning word << 8); for tests and benchmarks.
@@ -291,6 +330,10 @@ PYBIND11_MODULE(quant, m) {
     m.def("convert_awq_to_lmdeploy", &convert_awq_to_lmdeploy);
     // Additions without a counterpart in the reference's module.
     m.def("gemm_awq_algo", &gemm_awq_algo);
+    m.def("gemm_awq_residual_ut", &gemm_awq_residual_ut);
+    m.def("gemm_awq_fused_ut", &gemm_awq_fused_ut, py::arg("I"), py::arg("W"), py::arg("W_zeros_scales"),
+          py::arg("bias") = py::none(), py::arg("residual") = py::none(), py::arg("act") = "none", py::arg("N"),
+          py::arg("group_size"));
     m.def("convert_2bit_to_4bit", &convert_2bit_to_4bit);
     m.def("clear_repack_cache", &clear_repack_cache);
     m.def("repack_cache_size", &repack_cache_size);

@@ -25,6 +25,65 @@ int check_weight(int N, int K, int g, int layout) {
     return SQ_OK;
 }
 
+// One dispatcher behind every GEMM entry point.  `workspace` may be null: then the kernels
+// that need one are not considered (and an explicit SQ_ALGO_SKINNY_WS is an error).
+int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
+                  int layout, int algo, sq::Epilogue epi, void* workspace, size_t workspace_bytes, void* stream) {
+    if (M < 0) return SQ_ERR_BAD_SHAPE;
+    const int rc = check_weight(N, K, group_size, layout);
+    if (rc != SQ_OK) return rc;
+    // The GEMM kernels consume layout L1; an L2 weight is converted once with
+    // sq_repack_l2_to_l1 by the caller (the `quant` extension caches the result).
+    if (layout != SQ_LAYOUT_L1) return SQ_ERR_BAD_LAYOUT;
+    if (M == 0) return SQ_OK;
+    if (!x || !w || !zs || !y) return SQ_ERR_NULL_POINTER;
+    if (!aligned16(x) || !aligned16(w) || !aligned16(zs) || !aligned16(y)) return SQ_ERR_MISALIGNED;
+    if ((long)M * (long)K > (1L << 40) || (long)M * (long)N > (1L << 40)) return SQ_ERR_BAD_SHAPE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+
+    int kernel = algo & 0xFF;
+    const int tune = (algo >> 8) & 0xFFFF;
+    if (kernel == SQ_ALGO_AUTO) {
+        // Measured on OPT-6.7B shapes.  With a workspace the split-K kernel wins once the
+        // weight is large enough (fc1/fc2 class) for 9..32 tokens, and for 5..8 tokens when K
+        // is long.  Without one: the GEMV up to 4 tokens (up to 8 when K is short: its staged
+        // activations would otherwise need several sequential rounds), the 16-column kernel up
+        // to 32, the tiled GEMM beyond.
+        const bool large = (long)N * (long)K >= (1L << 25);
+        if (workspace && ((M > 8 && M <= 32 && large) || (M > 4 && M <= 8 && K > 8192)))
+            kernel = SQ_ALGO_SKINNY_WS;
+        else if (M <= 4 || (M <= 8 && K <= 8192))
+            kernel = SQ_ALGO_GEMV_FIXUP;
+        else if (M <= 32)
+            kernel = SQ_ALGO_SKINNY;
+        else
+            kernel = SQ_ALGO_GEMM;
+    }
+    switch (kernel) {
+        case SQ_ALGO_GEMV:
+        case SQ_ALGO_GEMV_FIXUP:
+            if (M > 8) return SQ_ERR_BAD_ALGO;
+            if (tune & 0x8000)
+                return launch_code(sq::launch_gemv_tuned(x, w, zs, y, M, N, K, group_size,
+                                                         kernel == SQ_ALGO_GEMV_FIXUP, tune & 0x7FFF, epi, st));
+            return launch_code(sq::launch_gemv2_tuned(x, w, zs, y, M, N, K, group_size,
+                                                      kernel == SQ_ALGO_GEMV_FIXUP, tune, epi, st));
+        case SQ_ALGO_SKINNY:
+            if (M > 64) return SQ_ERR_BAD_ALGO;
+            return launch_code(sq::launch_skinny_tuned(x, w, zs, y, M, N, K, group_size, tune, epi, st));
+        case SQ_ALGO_SKINNY_WS:
+            if (M > 32) return SQ_ERR_BAD_ALGO;
+            if (!workspace || !aligned16(workspace) || workspace_bytes < sq::skinny2_workspace_bytes(M, N, K) ||
+                (N + 63) / 64 > 16384)
+                return SQ_ERR_WORKSPACE;
+            return launch_code(sq::launch_skinny2_tuned(x, w, zs, y, workspace, M, N, K, group_size, tune, epi, st));
+        case SQ_ALGO_GEMM:
+            return launch_code(sq::launch_gemm_tuned(x, w, zs, y, M, N, K, group_size, tune, epi, st));
+        default:
+            return SQ_ERR_BAD_ALGO;
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -48,47 +107,8 @@ const char* sq_strerror(int code) {
 
 int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
                      int layout, int algo, void* stream) {
-    if (M < 0) return SQ_ERR_BAD_SHAPE;
-    const int rc = check_weight(N, K, group_size, layout);
-    if (rc != SQ_OK) return rc;
-    // The GEMM kernels consume layout L1; an L2 weight is converted once with
-    // sq_repack_l2_to_l1 by the caller (the `quant` extension caches the result).
-    if (layout != SQ_LAYOUT_L1) return SQ_ERR_BAD_LAYOUT;
-    if (M == 0) return SQ_OK;
-    if (!x || !w || !zs || !y) return SQ_ERR_NULL_POINTER;
-    if (!aligned16(x) || !aligned16(w) || !aligned16(zs) || !aligned16(y)) return SQ_ERR_MISALIGNED;
-    if ((long)M * (long)K > (1L << 40) || (long)M * (long)N > (1L << 40)) return SQ_ERR_BAD_SHAPE;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-
-    int kernel = algo & 0xFF;
-    const int tune = (algo >> 8) & 0xFFFF;
-    if (kernel == SQ_ALGO_AUTO) {
-        // 5..8 tokens with a long K: the GEMV's staged activations would need several
-        // sequential rounds; the 16-column kernel is faster there (measured on fc2 shapes).
-        if (M <= 4 || (M <= 8 && K <= 8192))
-            kernel = SQ_ALGO_GEMV_FIXUP;
-        else if (M <= 32)
-            kernel = SQ_ALGO_SKINNY;
-        else
-            kernel = SQ_ALGO_GEMM;
-    }
-    switch (kernel) {
-        case SQ_ALGO_GEMV:
-        case SQ_ALGO_GEMV_FIXUP:
-            if (M > 8) return SQ_ERR_BAD_ALGO;
-            if (tune & 0x8000)
-                return launch_code(sq::launch_gemv_tuned(x, w, zs, y, M, N, K, group_size,
-                                                         kernel == SQ_ALGO_GEMV_FIXUP, tune & 0x7FFF, st));
-            return launch_code(sq::launch_gemv2_tuned(x, w, zs, y, M, N, K, group_size,
-                                                      kernel == SQ_ALGO_GEMV_FIXUP, tune, st));
-        case SQ_ALGO_SKINNY:
-            if (M > 64) return SQ_ERR_BAD_ALGO;
-            return launch_code(sq::launch_skinny_tuned(x, w, zs, y, M, N, K, group_size, tune, st));
-        case SQ_ALGO_GEMM:
-            return launch_code(sq::launch_gemm_tuned(x, w, zs, y, M, N, K, group_size, tune, st));
-        default:
-            return SQ_ERR_BAD_ALGO;
-    }
+    return gemm_dispatch(x, w, zs, y, M, N, K, group_size, layout, algo, sq::Epilogue{nullptr, nullptr, 0}, nullptr, 0,
+                         stream);
 }
 
 size_t sq_w4a16_workspace_bytes(int M, int N, int K) {
@@ -98,25 +118,18 @@ size_t sq_w4a16_workspace_bytes(int M, int N, int K) {
 
 int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
                      int layout, int algo, void* workspace, size_t workspace_bytes, void* stream) {
-    const int kernel = algo & 0xFF;
-    // Measured on OPT-6.7B shapes: the split-K kernel wins once the weight is large enough
-    // (fc1/fc2 class) for 9..32 tokens, and for 5..8 tokens when K is long.
-    const bool large = (long)N * (long)K >= (1L << 25);
-    const bool want = kernel == SQ_ALGO_SKINNY_WS ||
-                      (kernel == SQ_ALGO_AUTO && ((M > 8 && M <= 32 && large) || (M > 4 && M <= 8 && K > 8192)));
-    if (!want) return sq_w4a16_gemm_ex(x, w, zs, y, M, N, K, group_size, layout, algo, stream);
-    if (M < 0 || M > 32) return M < 0 ? SQ_ERR_BAD_SHAPE : SQ_ERR_BAD_ALGO;
-    const int rc = check_weight(N, K, group_size, layout);
-    if (rc != SQ_OK) return rc;
-    if (layout != SQ_LAYOUT_L1) return SQ_ERR_BAD_LAYOUT;
-    if (M == 0) return SQ_OK;
-    if (!x || !w || !zs || !y) return SQ_ERR_NULL_POINTER;
-    if (!aligned16(x) || !aligned16(w) || !aligned16(zs) || !aligned16(y)) return SQ_ERR_MISALIGNED;
-    if (!workspace || !aligned16(workspace) || workspace_bytes < sq::skinny2_workspace_bytes(M, N, K) ||
-        (N + 63) / 64 > 16384)
-        return SQ_ERR_WORKSPACE;
-    return launch_code(sq::launch_skinny2_tuned(x, w, zs, y, workspace, M, N, K, group_size, (algo >> 8) & 0xFFFF,
-                                                static_cast<hipStream_t>(stream)));
+    return gemm_dispatch(x, w, zs, y, M, N, K, group_size, layout, algo, sq::Epilogue{nullptr, nullptr, 0}, workspace,
+                         workspace_bytes, stream);
+}
+
+int sq_w4a16_gemm_fused(const void* x, const void* w, const void* zs, const void* bias, const void* residual, void* y,
+                        int M, int N, int K, int group_size, int layout, int act, int algo, void* workspace,
+                        size_t workspace_bytes, void* stream) {
+    if (act != SQ_ACT_NONE && act != SQ_ACT_RELU) return SQ_ERR_BAD_ALGO;
+    if (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)) return SQ_ERR_MISALIGNED;
+    if (residual && (reinterpret_cast<uintptr_t>(residual) & 1u)) return SQ_ERR_MISALIGNED;
+    const sq::Epilogue epi{static_cast<const sq::half_t*>(bias), static_cast<const sq::half_t*>(residual), act};
+    return gemm_dispatch(x, w, zs, y, M, N, K, group_size, layout, algo, epi, workspace, workspace_bytes, stream);
 }
 
 int sq_w4a16_gemm(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,

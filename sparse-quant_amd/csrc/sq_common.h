@@ -111,4 +111,18 @@ __device__ __forceinline__ u32x4_t quad_bcast(u32x4_t v) {
 
 __device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
 
+// What happens to an fp32 accumulator on its way to Y[m, n]: + bias[n], activation,
+// + residual[m, n] (each optional), one rounding to fp16 at the end.
+struct Epilogue {
+    const half_t* bias;      // [N] or null
+    const half_t* residual;  // [M, N] or null; must not overlap Y
+    int act;                 // 0 = none, 1 = ReLU
+};
+__device__ __forceinline__ half_t epilogue(float v, int m, int n, int N, const Epilogue& e) {
+    if (e.bias) v += (float)e.bias[n];
+    if (e.act == 1) v = fmaxf(v, 0.f);
+    if (e.residual) v += (float)e.residual[(long)m * N + n];
+    return (half_t)v;
+}
+
 }  // namespace sq

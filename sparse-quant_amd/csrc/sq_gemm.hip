@@ -38,7 +38,7 @@ __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1
 template <int MI>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS,
                                                    const half_t* __restrict__ X, half_t* __restrict__ Y, int M,
-                                                   int N, int K, int gshift) {
+                                                   int N, int K, int gshift, Epilogue epi) {
     constexpr int BM = 32 * MI;
     // Activation tile, two stages, row pitch 128 B (64 halves, no padding); the eight
     // 16-byte chunks of row R are stored at chunk position c ^ swz(R); 8 consecutive
@@ -195,28 +195,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int m = m0 + 32 * mi + 8 * (v >> 2) + 4 * lc + (v & 3);
-                if (m < M && n < N) Y[(long)m * N + n] = (half_t)acc[mi][ni][v];
+                if (m < M && n < N) Y[(long)m * N + n] = epilogue(acc[mi][ni][v], m, n, N, epi);
             }
         }
 }
 
 template <int MI>
 static hipError_t launch_mi(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int gshift,
-                            hipStream_t st) {
+                            Epilogue epi, hipStream_t st) {
     const dim3 grid((N + GEMM_BN - 1) / GEMM_BN, (M + 32 * MI - 1) / (32 * MI));
     hipLaunchKernelGGL((gemm_kernel<MI>), grid, dim3(256), 0, st, (const uint8_t*)w, (const half2_t*)zs,
-                       (const half_t*)x, (half_t*)y, M, N, K, gshift);
+                       (const half_t*)x, (half_t*)y, M, N, K, gshift, epi);
     return hipGetLastError();
 }
 
 // tune = 0 for the heuristic, else the number of 32-row tiles per workgroup (1, 2 or 4), or 8 / 9 / 10 for
 // the software-pipelined kernel (128 rows at two waves per SIMD, 128 rows at one, 256 rows at one).
 hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                             int tune, hipStream_t st) {
+                             int tune, Epilogue epi, hipStream_t st) {
     int gshift = 0;
     while ((1 << gshift) < g) gshift++;
     int mi = tune & 0xFF;
-    if (mi >= 8 && mi <= 10) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, mi - 8, st);
+    if (mi >= 8 && mi <= 10) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, mi - 8, epi, st);
     if (mi != 1 && mi != 2 && mi != 4) {
         if (M > 64) {
             // Measured on MI355X (the chip runs these kernels at a power-limited clock, so fewer
@@ -225,15 +225,15 @@ hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void*
             // tiles, pipelined variant for long K.
             const long t256 = (long)((N + 255) / 256) * ((M + 255) / 256);
             const long rounds = (t256 + 255) / 256;
-            if (t256 * 10 >= rounds * 256 * 8) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, 2, st);
-            if (K >= 8192) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, 1, st);
+            if (t256 * 10 >= rounds * 256 * 8) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, 2, epi, st);
+            if (K >= 8192) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, 1, epi, st);
         }
         mi = M > 64 ? 4 : (M > 32 ? 2 : 1);
     }
     switch (mi) {
-        case 1: return launch_mi<1>(x, w, zs, y, M, N, K, gshift, st);
-        case 2: return launch_mi<2>(x, w, zs, y, M, N, K, gshift, st);
-        default: return launch_mi<4>(x, w, zs, y, M, N, K, gshift, st);
+        case 1: return launch_mi<1>(x, w, zs, y, M, N, K, gshift, epi, st);
+        case 2: return launch_mi<2>(x, w, zs, y, M, N, K, gshift, epi, st);
+        default: return launch_mi<4>(x, w, zs, y, M, N, K, gshift, epi, st);
     }
 }
 

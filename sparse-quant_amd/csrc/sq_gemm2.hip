@@ -26,7 +26,7 @@ __device__ __forceinline__ int swz2(int row) { return (row & 7) ^ ((row >> 3) & 
 template <int MI, int OCC>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void gemm_pipe_kernel(
     const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS, const half_t* __restrict__ X,
-    half_t* __restrict__ Y, int M, int N, int K, int gshift) {
+    half_t* __restrict__ Y, int M, int N, int K, int gshift, Epilogue epi) {
     constexpr int G2_BM = 32 * MI;
     __shared__ __attribute__((aligned(1024))) uint8_t xs[2][G2_BM * 128];
 
@@ -184,29 +184,29 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int m = m0 + 32 * mi + 8 * (v >> 2) + 4 * lc + (v & 3);
-                if (m < M && n < N) Y[(long)m * N + n] = (half_t)acc[mi][ni][v];
+                if (m < M && n < N) Y[(long)m * N + n] = epilogue(acc[mi][ni][v], m, n, N, epi);
             }
         }
 }
 
 template <int MI, int OCC>
 static hipError_t launch_pipe_cfg(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int gshift,
-                                  hipStream_t st) {
+                                  Epilogue epi, hipStream_t st) {
     const dim3 grid((N + G2_BN - 1) / G2_BN, (M + 32 * MI - 1) / (32 * MI));
     hipLaunchKernelGGL((gemm_pipe_kernel<MI, OCC>), grid, dim3(256), 0, st, (const uint8_t*)w, (const half2_t*)zs,
-                       (const half_t*)x, (half_t*)y, M, N, K, gshift);
+                       (const half_t*)x, (half_t*)y, M, N, K, gshift, epi);
     return hipGetLastError();
 }
 
 // variant: 0 = 128-row tile, two waves per SIMD; 1 = 128-row tile, one wave per SIMD;
 // 2 = 256-row tile, one wave per SIMD.
 hipError_t launch_gemm_pipe(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                            int variant, hipStream_t st) {
+                            int variant, Epilogue epi, hipStream_t st) {
     int gshift = 0;
     while ((1 << gshift) < g) gshift++;
-    if (variant == 0) return launch_pipe_cfg<4, 2>(x, w, zs, y, M, N, K, gshift, st);
-    if (variant == 1) return launch_pipe_cfg<4, 1>(x, w, zs, y, M, N, K, gshift, st);
-    return launch_pipe_cfg<8, 1>(x, w, zs, y, M, N, K, gshift, st);
+    if (variant == 0) return launch_pipe_cfg<4, 2>(x, w, zs, y, M, N, K, gshift, epi, st);
+    if (variant == 1) return launch_pipe_cfg<4, 1>(x, w, zs, y, M, N, K, gshift, epi, st);
+    return launch_pipe_cfg<8, 1>(x, w, zs, y, M, N, K, gshift, epi, st);
 }
 
 }  // namespace sq

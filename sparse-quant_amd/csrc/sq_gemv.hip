@@ -29,7 +29,7 @@ namespace sq {
 template <int RS, int MROWS, bool FIXUP>
 __global__ __launch_bounds__(1024) void gemv_kernel(const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS,
                                                     const half_t* __restrict__ X, half_t* __restrict__ Y, int M,
-                                                    int N, int K, int gshift) {
+                                                    int N, int K, int gshift, Epilogue epi) {
     constexpr int MT = (MROWS + 3) / 4;
     extern __shared__ float red[];
 
@@ -171,49 +171,49 @@ __global__ __launch_bounds__(1024) void gemv_kernel(const uint8_t* __restrict__ 
         const int m = (t >> 2) % MROWS;
         const int rs = (t >> 2) / MROWS;
         const int row = row0 + 4 * rs + ri;
-        if (row < N && m < M) Y[(long)m * N + row] = (half_t)sum;
+        if (row < N && m < M) Y[(long)m * N + row] = epilogue(sum, m, row, N, epi);
     }
 }
 
 template <int RS, int MROWS>
 static hipError_t launch_cfg(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int gshift,
-                             bool fixup, int nwaves, hipStream_t st) {
+                             bool fixup, int nwaves, Epilogue epi, hipStream_t st) {
     const int rows = 4 * RS;
     const dim3 grid((N + rows - 1) / rows);
     const dim3 block(64 * nwaves);
     const size_t lds = (size_t)nwaves * 4 * RS * MROWS * 4 * sizeof(float);
     if (fixup)
         hipLaunchKernelGGL((gemv_kernel<RS, MROWS, true>), grid, block, lds, st, (const uint8_t*)w,
-                           (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift);
+                           (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift, epi);
     else
         hipLaunchKernelGGL((gemv_kernel<RS, MROWS, false>), grid, block, lds, st, (const uint8_t*)w,
-                           (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift);
+                           (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift, epi);
     return hipGetLastError();
 }
 
 template <int MROWS>
 static hipError_t launch_rows(int rs, const void* x, const void* w, const void* zs, void* y, int M, int N, int K,
-                              int gshift, bool fixup, int nwaves, hipStream_t st) {
+                              int gshift, bool fixup, int nwaves, Epilogue epi, hipStream_t st) {
     switch (rs) {
-        case 1: return launch_cfg<1, MROWS>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, st);
-        case 2: return launch_cfg<2, MROWS>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, st);
-        default: return launch_cfg<4, MROWS>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, st);
+        case 1: return launch_cfg<1, MROWS>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, epi, st);
+        case 2: return launch_cfg<2, MROWS>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, epi, st);
+        default: return launch_cfg<4, MROWS>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, epi, st);
     }
 }
 
 // tune = 0 for the built-in heuristic, else (row steps per workgroup) | (waves << 8).
 hipError_t launch_gemv_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                             bool fixup, int tune, hipStream_t st) {
+                             bool fixup, int tune, Epilogue epi, hipStream_t st) {
     int gshift = 0;
     while ((1 << gshift) < g) gshift++;
     const int nslices = (K + 511) / 512;
     int rs = tune & 0xFF, nwaves = (tune >> 8) & 0xFF;
     if (rs != 1 && rs != 2 && rs != 4) rs = (N >= 8192) ? 4 : 2;
     if (nwaves < 1 || nwaves > 16) nwaves = nslices >= 32 ? 16 : (nslices >= 8 ? 8 : (nslices >= 4 ? 4 : nslices));
-    if (M <= 1) return launch_rows<1>(rs, x, w, zs, y, M, N, K, gshift, fixup, nwaves, st);
-    if (M <= 2) return launch_rows<2>(rs, x, w, zs, y, M, N, K, gshift, fixup, nwaves, st);
-    if (M <= 4) return launch_rows<4>(rs, x, w, zs, y, M, N, K, gshift, fixup, nwaves, st);
-    return launch_rows<8>(rs, x, w, zs, y, M, N, K, gshift, fixup, nwaves, st);
+    if (M <= 1) return launch_rows<1>(rs, x, w, zs, y, M, N, K, gshift, fixup, nwaves, epi, st);
+    if (M <= 2) return launch_rows<2>(rs, x, w, zs, y, M, N, K, gshift, fixup, nwaves, epi, st);
+    if (M <= 4) return launch_rows<4>(rs, x, w, zs, y, M, N, K, gshift, fixup, nwaves, epi, st);
+    return launch_rows<8>(rs, x, w, zs, y, M, N, K, gshift, fixup, nwaves, epi, st);
 }
 
 

@@ -35,7 +35,7 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
                                                              const half2_t* __restrict__ ZS,
                                                              const half_t* __restrict__ X,
                                                              half_t* __restrict__ Y, int M, int N, int K,
-                                                             int gshift) {
+                                                             int gshift, Epilogue epi) {
     constexpr int MT = (MROWS + 3) / 4;
     constexpr int PITCH = 1024 * S + 16;                 // bytes per staged activation row
     constexpr int NT = 64 * NR * KS;
@@ -171,7 +171,7 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
         v += __shfl_xor(v, 16);
         v += __shfl_xor(v, 32);
         if (KS == 1) {
-            if (lane < 4 && out_row < N && m < M) Y[(long)m * N + out_row] = (half_t)v;
+            if (lane < 4 && out_row < N && m < M) Y[(long)m * N + out_row] = epilogue(v, m, out_row, N, epi);
         } else if (lane < 4) {
             red[wq_][wr][m][i] = v;
         }
@@ -186,57 +186,57 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
 #pragma unroll
             for (int q = 0; q < KS; q++) sum += red[q][r][m][ri];
             const int orow = blockIdx.x * (4 * NR) + 4 * r + ri;
-            if (orow < N && m < M) Y[(long)m * N + orow] = (half_t)sum;
+            if (orow < N && m < M) Y[(long)m * N + orow] = epilogue(sum, m, orow, N, epi);
         }
     }
 }
 
 template <int MROWS, int NR, int KS, int S>
 static hipError_t launch_cfg(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int gshift,
-                             bool fixup, hipStream_t st) {
+                             bool fixup, Epilogue epi, hipStream_t st) {
     const dim3 grid((N + 4 * NR - 1) / (4 * NR));
     if (fixup)
         hipLaunchKernelGGL((gemv2_kernel<MROWS, NR, KS, S, true>), grid, dim3(64 * NR * KS), 0, st, (const uint8_t*)w,
-                           (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift);
+                           (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift, epi);
     else
         hipLaunchKernelGGL((gemv2_kernel<MROWS, NR, KS, S, false>), grid, dim3(64 * NR * KS), 0, st,
-                           (const uint8_t*)w, (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift);
+                           (const uint8_t*)w, (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift, epi);
     return hipGetLastError();
 }
 
 // Staged activations are kept under 48 KiB of LDS: KS * MROWS * S KiB.
 template <int MROWS, int S>
 static hipError_t launch_steps(int nr, int ks, const void* x, const void* w, const void* zs, void* y, int M, int N,
-                               int K, int gshift, bool fixup, hipStream_t st) {
+                               int K, int gshift, bool fixup, Epilogue epi, hipStream_t st) {
     constexpr int KS_MAX = 48 / (MROWS * S) >= 4 ? 4 : (48 / (MROWS * S) >= 2 ? 2 : 1);
     if (ks > KS_MAX) ks = KS_MAX;
     while (nr * ks > 16) nr >>= 1;
 #define SQ_CASE(NR_, KS_)                                                                    \
     if (nr == NR_ && ks == KS_) {                                                           \
         if constexpr (KS_ <= KS_MAX)                                                        \
-            return launch_cfg<MROWS, NR_, KS_, S>(x, w, zs, y, M, N, K, gshift, fixup, st); \
+            return launch_cfg<MROWS, NR_, KS_, S>(x, w, zs, y, M, N, K, gshift, fixup, epi, st); \
     }
     SQ_CASE(2, 1) SQ_CASE(4, 1) SQ_CASE(8, 1)
     SQ_CASE(2, 2) SQ_CASE(4, 2) SQ_CASE(8, 2)
     SQ_CASE(2, 4) SQ_CASE(4, 4)
 #undef SQ_CASE
-    return launch_cfg<MROWS, 4, 1, S>(x, w, zs, y, M, N, K, gshift, fixup, st);
+    return launch_cfg<MROWS, 4, 1, S>(x, w, zs, y, M, N, K, gshift, fixup, epi, st);
 }
 
 template <int MROWS>
 static hipError_t launch_rows(int nr, int ks, int steps, const void* x, const void* w, const void* zs, void* y,
-                              int M, int N, int K, int gshift, bool fixup, hipStream_t st) {
+                              int M, int N, int K, int gshift, bool fixup, Epilogue epi, hipStream_t st) {
     constexpr int S_MAX = (MROWS >= 4) ? 4 : 8;
-    if (steps >= 8 && S_MAX >= 8) return launch_steps<MROWS, S_MAX>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, st);
-    if (steps >= 4) return launch_steps<MROWS, 4>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, st);
-    return launch_steps<MROWS, 2>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, st);
+    if (steps >= 8 && S_MAX >= 8) return launch_steps<MROWS, S_MAX>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
+    if (steps >= 4) return launch_steps<MROWS, 4>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
+    return launch_steps<MROWS, 2>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
 }
 
 // tune = 0 for the built-in heuristic, else (row groups per workgroup: 2,4,8) |
 // (k ranges per workgroup: 1,2,4) << 4.  A workgroup covers 4 * row groups rows; the
 // number of k-steps a wave issues per round (2, 4 or 8) follows from K and the k ranges.
 hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                              bool fixup, int tune, hipStream_t st) {
+                              bool fixup, int tune, Epilogue epi, hipStream_t st) {
     int gshift = 0;
     while ((1 << gshift) < g) gshift++;
     int nr = tune & 0xF, ks = (tune >> 4) & 0xF;
@@ -246,10 +246,10 @@ hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void
     if (ks != 1 && ks != 2 && ks != 4) ks = nsteps > 16 ? 4 : (((long)N * K >= (1L << 25) && nsteps >= 8) ? 2 : 1);
     if (nr != 2 && nr != 4 && nr != 8) nr = ks == 4 ? 2 : 4;
     const int spw = (nsteps + ks - 1) / ks;
-    if (M <= 1) return launch_rows<1>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, st);
-    if (M <= 2) return launch_rows<2>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, st);
-    if (M <= 4) return launch_rows<4>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, st);
-    return launch_rows<8>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, st);
+    if (M <= 1) return launch_rows<1>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
+    if (M <= 2) return launch_rows<2>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
+    if (M <= 4) return launch_rows<4>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
+    return launch_rows<8>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
 }
 
 }  // namespace sq

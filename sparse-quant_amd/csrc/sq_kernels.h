@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "sq_common.h"
+
 namespace sq {
 
 // sq_dequant.hip
@@ -24,25 +26,25 @@ hipError_t launch_clock_probe(void* out, int spins, hipStream_t st);
 // The *_tuned launchers take a kernel-specific tuning word (0 = built-in heuristic).
 // sq_gemv.hip: M <= 8.  tune = row steps per workgroup (1,2,4) | waves << 8.
 hipError_t launch_gemv_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                             bool fixup, int tune, hipStream_t st);
+                             bool fixup, int tune, Epilogue epi, hipStream_t st);
 // sq_gemv2.hip: M <= 8, streaming formulation.  tune = waves per workgroup (1,2,4,8).
 hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                              bool fixup, int tune, hipStream_t st);
+                              bool fixup, int tune, Epilogue epi, hipStream_t st);
 // sq_skinny.hip: M <= 64.  tune = waves | mode << 8 (mode 1 = exact, 2 = fixup).
 hipError_t launch_skinny_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                               int tune, hipStream_t st);
+                               int tune, Epilogue epi, hipStream_t st);
 // sq_skinny2.hip: 5 <= M <= 32 with a workspace (counters + fp32 partial tiles).
 // tune = ksplit (1,2,4,8) | mode << 8 (1 = exact, 2 = fixup).
 size_t skinny2_workspace_bytes(int M, int N, int K);
 hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
-                                int g, int tune, hipStream_t st);
+                                int g, int tune, Epilogue epi, hipStream_t st);
 // sq_gemm.hip: any M.  tune = 32-row tiles per workgroup (1,2,4).
 hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                             int tune, hipStream_t st);
+                             int tune, Epilogue epi, hipStream_t st);
 
 // sq_gemm2.hip: software-pipelined 128 x 256 tile variant for M > 64.
 hipError_t launch_gemm_pipe(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                            int variant, hipStream_t st);
+                            int variant, Epilogue epi, hipStream_t st);
 
 // sq_attn.hip: LUT block-sparse attention, prefill.  D in {64, 128}; lut int32 or int64 [H, ceil(S/64), nnz].
 hipError_t launch_lut_attention(const void* q, const void* k, const void* v, void* o, const void* lut,

@@ -23,7 +23,7 @@ namespace sq {
 template <int MT, bool FIXUP>
 __global__ __launch_bounds__(512) void skinny_kernel(const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS,
                                                      const half_t* __restrict__ X, half_t* __restrict__ Y, int M,
-                                                     int N, int K, int gshift) {
+                                                     int N, int K, int gshift, Epilogue epi) {
     extern __shared__ float red[];
     const NibbleMasks nm = nibble_masks();
     const int lane = threadIdx.x & 63;
@@ -113,28 +113,28 @@ __global__ __launch_bounds__(512) void skinny_kernel(const uint8_t* __restrict__
         const int mt = t >> 8;
         const int m = 16 * mt + 4 * (l >> 4) + v;
         const int n = row0 + (l & 15);
-        if (m < M && n < N) Y[(long)m * N + n] = (half_t)sum;
+        if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum, m, n, N, epi);
     }
 }
 
 template <int MT>
 static hipError_t launch_mt(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int gshift,
-                            bool fixup, int nwaves, hipStream_t st) {
+                            bool fixup, int nwaves, Epilogue epi, hipStream_t st) {
     const dim3 grid((N + 15) / 16);
     const dim3 block(64 * nwaves);
     const size_t lds = (size_t)nwaves * MT * 4 * 64 * sizeof(float);
     if (fixup)
         hipLaunchKernelGGL((skinny_kernel<MT, true>), grid, block, lds, st, (const uint8_t*)w, (const half2_t*)zs,
-                           (const half_t*)x, (half_t*)y, M, N, K, gshift);
+                           (const half_t*)x, (half_t*)y, M, N, K, gshift, epi);
     else
         hipLaunchKernelGGL((skinny_kernel<MT, false>), grid, block, lds, st, (const uint8_t*)w, (const half2_t*)zs,
-                           (const half_t*)x, (half_t*)y, M, N, K, gshift);
+                           (const half_t*)x, (half_t*)y, M, N, K, gshift, epi);
     return hipGetLastError();
 }
 
 // tune = 0 for the heuristic, else waves | (mode << 8) with mode 1 = exact, 2 = fixup.
 hipError_t launch_skinny_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                               int tune, hipStream_t st) {
+                               int tune, Epilogue epi, hipStream_t st) {
     int gshift = 0;
     while ((1 << gshift) < g) gshift++;
     int nwaves = tune & 0xFF;
@@ -146,10 +146,10 @@ hipError_t launch_skinny_tuned(const void* x, const void* w, const void* zs, voi
     if (mode == 2 && g == 128) fixup = true;
     const int mt = (M + 15) / 16;
     switch (mt) {
-        case 1: return launch_mt<1>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, st);
-        case 2: return launch_mt<2>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, st);
-        case 3: return launch_mt<3>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, st);
-        default: return launch_mt<4>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, st);
+        case 1: return launch_mt<1>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, epi, st);
+        case 2: return launch_mt<2>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, epi, st);
+        case 3: return launch_mt<3>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, epi, st);
+        default: return launch_mt<4>(x, w, zs, y, M, N, K, gshift, fixup, nwaves, epi, st);
     }
 }
 

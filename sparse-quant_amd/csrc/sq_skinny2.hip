@@ -47,7 +47,7 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
                                                            const half2_t* __restrict__ ZS,
                                                            const half_t* __restrict__ X, half_t* __restrict__ Y,
                                                            float* part, unsigned* counters, int M, int N, int K,
-                                                           int gshift, int ksplit) {
+                                                           int gshift, int ksplit, Epilogue epi) {
     constexpr int TILE = 4 * MT * 4 * 64;  // floats a wave contributes: [rt][mt][v][lane]
     constexpr int XBUF = MT * 16 * SK2_XPITCH;
     constexpr int SH_BYTES = NWV * XBUF > NWV * TILE * 4 ? NWV * XBUF : NWV * TILE * 4;
@@ -244,7 +244,7 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
             const int l = t & 63, v = (t >> 6) & 3, mt = (t >> 8) % MT, rt = (t >> 8) / MT;
             const int m = 16 * mt + 4 * (l >> 4) + v;
             const int n = rb * 64 + 16 * rt + (l & 15);
-            if (m < M && n < N) Y[(long)m * N + n] = (half_t)sum;
+            if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum, m, n, N, epi);
         }
         return;
     }
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
         const int l = t & 63, v = (t >> 6) & 3, mt = (t >> 8) % MT, rt = (t >> 8) / MT;
         const int m = 16 * mt + 4 * (l >> 4) + v;
         const int n = rb * 64 + 16 * rt + (l & 15);
-        if (m < M && n < N) Y[(long)m * N + n] = (half_t)sum;
+        if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum, m, n, N, epi);
     }
     // leave the workspace ready for the next call
     if (tid == 0) __hip_atomic_store(&counters[rb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -290,16 +290,16 @@ size_t skinny2_workspace_bytes(int M, int N, int K) {
 
 template <int MT, int NWV, int S>
 static hipError_t launch_cfg(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
-                             int gshift, bool fixup, int ksplit, hipStream_t st) {
+                             int gshift, bool fixup, int ksplit, Epilogue epi, hipStream_t st) {
     const dim3 grid((N + 63) / 64, ksplit);
     unsigned* counters = (unsigned*)ws;
     float* part = (float*)((char*)ws + SK2_COUNTER_BYTES);
     if (fixup)
         hipLaunchKernelGGL((skinny2_kernel<MT, NWV, S, true>), grid, dim3(64 * NWV), 0, st, (const uint8_t*)w,
-                           (const half2_t*)zs, (const half_t*)x, (half_t*)y, part, counters, M, N, K, gshift, ksplit);
+                           (const half2_t*)zs, (const half_t*)x, (half_t*)y, part, counters, M, N, K, gshift, ksplit, epi);
     else
         hipLaunchKernelGGL((skinny2_kernel<MT, NWV, S, false>), grid, dim3(64 * NWV), 0, st, (const uint8_t*)w,
-                           (const half2_t*)zs, (const half_t*)x, (half_t*)y, part, counters, M, N, K, gshift, ksplit);
+                           (const half2_t*)zs, (const half_t*)x, (half_t*)y, part, counters, M, N, K, gshift, ksplit, epi);
     return hipGetLastError();
 }
 
@@ -308,7 +308,7 @@ static hipError_t launch_cfg(const void* x, const void* w, const void* zs, void*
 // The first 64 KiB of the workspace are counters and must be zero before the first call;
 // every call leaves them zero.
 hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
-                                int g, int tune, hipStream_t st) {
+                                int g, int tune, Epilogue epi, hipStream_t st) {
     int gshift = 0;
     while ((1 << gshift) < g) gshift++;
     const int mt = (M + 15) / 16;
@@ -327,9 +327,9 @@ hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, vo
     const int mode = (tune >> 8) & 0xF;
     bool fixup = (g == 128);
     if (mode == 1) fixup = false;
-    if (mt == 2) return launch_cfg<2, 4, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, st);
-    if (nwv == 8) return launch_cfg<1, 8, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, st);
-    return launch_cfg<1, 4, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, st);
+    if (mt == 2) return launch_cfg<2, 4, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
+    if (nwv == 8) return launch_cfg<1, 8, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
+    return launch_cfg<1, 4, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
 }
 
 }  // namespace sq

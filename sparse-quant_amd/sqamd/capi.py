@@ -27,6 +27,7 @@ SIGNATURES = {
     "sq_w4a16_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "sq_w4a16_gemm_ex": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "sq_w4a16_gemm_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp]),
+    "sq_w4a16_gemm_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp]),
     "sq_w4a16_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
     "sq_w4a16_dequant": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "sq_transpose_merge_zeros_scales": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
@@ -116,6 +117,23 @@ def gemm_ws(x, w, zs, n, k, group_size, algo=SQ_ALGO_AUTO, out=None, stream=None
         ws = workspace(max(m, 1), n, k, x.device, stream)
     _check(lib().sq_w4a16_gemm_ws(_ptr(x), _ptr(w), _ptr(zs), _ptr(out), m, n, k, group_size, SQ_LAYOUT_L1, algo,
                                   _ptr(ws), ws.numel(), _stream(stream)), "sq_w4a16_gemm_ws")
+    return out
+
+
+SQ_ACT_NONE, SQ_ACT_RELU = 0, 1
+
+
+def gemm_fused(x, w, zs, n, k, group_size, bias=None, residual=None, act=SQ_ACT_NONE, algo=SQ_ALGO_AUTO, out=None,
+               stream=None, ws=None, use_workspace=True):
+    """y = act(x W_hat^T + bias) + residual through sq_w4a16_gemm_fused."""
+    m = x.numel() // k
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
+    if ws is None and use_workspace and 4 < m <= 32:
+        ws = workspace(m, n, k, x.device, stream)
+    _check(lib().sq_w4a16_gemm_fused(_ptr(x), _ptr(w), _ptr(zs), _ptr(bias), _ptr(residual), _ptr(out), m, n, k,
+                                     group_size, SQ_LAYOUT_L1, act, algo, _ptr(ws), 0 if ws is None else ws.numel(),
+                                     _stream(stream)), "sq_w4a16_gemm_fused")
     return out
 
 

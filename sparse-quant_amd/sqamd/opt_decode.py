@@ -41,15 +41,20 @@ class DecoderLayer(nn.Module):
         self.out_proj = _random_walinear(hidden, hidden, g, dev, gen)
         self.fc1 = _random_walinear(hidden, ffn, g, dev, gen)
         self.fc2 = _random_walinear(ffn, hidden, g, dev, gen)
+        self.qkv_proj = None
 
     def forward(self, x, kc, vc, pos0, mask):
         """x [B, T, H]; kc, vc [B, heads, Lmax, hd]; writes cache rows pos0 .. pos0+T-1."""
         b, t, hdim = x.shape
         h = self.ln1(x)
         flat = h.reshape(1, b * t, hdim)  # the reference flattens to [1, bs*seq, K] as well
-        q = self.q_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
-        k = self.k_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
-        v = self.v_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
+        if self.qkv_proj is not None:
+            qkv = self.qkv_proj(flat).view(b, t, 3, self.heads, self.hd)
+            q, k, v = (qkv[:, :, j].transpose(1, 2) for j in range(3))
+        else:
+            q = self.q_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
+            k = self.k_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
+            v = self.v_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
         if isinstance(pos0, int):
             kc[:, :, pos0:pos0 + t] = k
             vc[:, :, pos0:pos0 + t] = v
@@ -60,10 +65,23 @@ class DecoderLayer(nn.Module):
             vc.index_copy_(2, pos0, v)
             a = nn.functional.scaled_dot_product_attention(q, kc, vc, attn_mask=mask)
         a = a.transpose(1, 2).reshape(1, b * t, hdim)
-        x = x + self.out_proj(a).view(b, t, hdim)
+        # bias, ReLU and the two residual adds ride in the kernels' stores
+        x = self.out_proj(a, residual=x.reshape(1, b * t, hdim)).view(b, t, hdim)
         h = self.ln2(x).reshape(1, b * t, hdim)
-        h = torch.relu(self.fc1(h))
-        return x + self.fc2(h).view(b, t, hdim)
+        h = self.fc1(h, act="relu")
+        return self.fc2(h, residual=x.reshape(1, b * t, hdim)).view(b, t, hdim)
+
+    def fuse_qkv(self):
+        """Serve q, k and v with one launch: layout L1 is row-major in N, so the three weights
+        (and their zeros_scales and biases) concatenate along the output dimension."""
+        ps = (self.q_proj, self.k_proj, self.v_proj)
+        fused = WALinear(ps[0].in_features, 3 * ps[0].out_features, group_size=ps[0].group_size, bias=True,
+                         dev=ps[0].weight.device)
+        fused.weight = torch.cat([p.weight for p in ps], 0).contiguous()
+        fused.zeros_scales = torch.cat([p.zeros_scales for p in ps], 0).contiguous()
+        fused.bias = torch.cat([p.bias for p in ps], 1).contiguous()
+        self.qkv_proj = fused
+        self.q_proj = self.k_proj = self.v_proj = None
 
 
 class OPTDecoder(nn.Module):
@@ -99,10 +117,13 @@ class OPTDecoder(nn.Module):
 
 
 @torch.no_grad()
-def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed=0):
+def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed=0, fuse_qkv=True):
     """Greedy generation on random token ids; returns timing and throughput figures."""
     dev = "cuda"
     model = OPTDecoder(layers=layers, dev=dev, seed=seed)
+    if fuse_qkv:
+        for layer in model.layers:
+            layer.fuse_qkv()
     gen = torch.Generator(device=dev)
     gen.manual_seed(seed + 1)
     ids = torch.randint(0, 50272, (batch, prompt), device=dev, generator=gen)
@@ -140,7 +161,7 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with torch.cuda.graph(graph, stream=side):  # same stream as the warm-up: per-stream workspaces exist
             step()
     generated = [tok.clone()]
     mask.fill_(float("-inf"))
@@ -163,6 +184,7 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
     return {
         "batch": batch, "prompt": prompt, "new_tokens": new_tokens, "layers": layers,
         "launch": "hip-graph replay" if graph is not None else "eager",
+        "fused": "bias+relu+residual in the GEMM store" + ("; q/k/v one launch" if fuse_qkv else ""),
         "prefill_ms": round(prefill_s * 1e3, 2),
         "prefill_tok_per_s": round(batch * prompt / prefill_s, 1),
         "decode_ms_per_step": round(decode_s * 1e3 / steps, 4),

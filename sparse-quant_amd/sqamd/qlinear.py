@@ -4,7 +4,8 @@ Mirror of the reference's module (test/muxi/module/qlinear/qlinear.py:8-106 and
 test/nvidia/module/qlinear/qlinear.py:10-92): same constructor arguments, the same
 buffer names, shapes and dtypes (so a state_dict saved by the reference loads
 unchanged), the same forward contract `gemm_awq_ut(x, weight, zeros_scales, ...) +
-bias`.  `layout` selects which of the reference's two buffer conventions is used:
+bias` (the bias add is folded into the kernel; `forward` also takes an optional
+residual and activation for the decoder layer's fused tails).  `layout` selects which of the reference's two buffer conventions is used:
 
     "l1" (default)  weight uint8 [N, K*w_bit/8], zeros_scales fp16 [N, 2K/g], g default 64
     "l2"            weight int32 [K, N*w_bit/32], zeros_scales fp16 [K/g, 2N], g default 128
@@ -48,7 +49,10 @@ class WALinear(nn.Module):
             self.register_buffer("bias", None)
 
     @torch.no_grad()
-    def forward(self, x):
+    def forward(self, x, residual=None, act="none"):
+        """y = act(x W_hat^T + bias) + residual.  With the defaults this is the reference's
+        forward (gemm_awq_ut, then + bias); bias, activation and residual all ride in the
+        kernel's store instead of separate element-wise launches."""
         weight = self.weight
         if self.w_bit == 2:
             if self.layout != "l1":
@@ -56,12 +60,12 @@ class WALinear(nn.Module):
             weight = quant.convert_2bit_to_4bit(weight)
         lead = x.shape[:-1]
         x3 = x.reshape(1, -1, x.shape[-1]) if x.dim() != 3 else x
-        y = quant.gemm_awq_ut(x3.contiguous(), weight, self.zeros_scales, x3.shape[-2], self.out_features,
-                              self.in_features, self.group_size)
-        y = y.reshape(*lead, self.out_features)
-        if self.bias is not None:
-            y = y + self.bias
-        return y
+        res3 = None
+        if residual is not None:
+            res3 = residual.reshape(x3.shape[0], x3.shape[1], self.out_features).contiguous()
+        y = quant.gemm_awq_fused_ut(x3.contiguous(), weight, self.zeros_scales, self.bias, res3, act,
+                                    self.out_features, self.group_size)
+        return y.reshape(*lead, self.out_features)
 
     @staticmethod
     def from_float(module, w_config, a_config=None, quantize_output=False, layout="l1"):

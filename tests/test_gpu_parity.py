@@ -416,3 +416,100 @@ def test_quant_extension_decode_batches_use_workspace_path(n, k, m):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y_graph, y)
+
+
+# ------------------------------------------------------------------ fused epilogue: act(x W^T + bias) + residual
+def fused_ref(x, w_hat, bias, residual, act):
+    y = orc.gemm_ref(x, w_hat).astype(np.float64)
+    if bias is not None:
+        y = y + bias.astype(np.float64)[None, :]
+    if act:
+        y = np.maximum(y, 0.0)
+    if residual is not None:
+        y = y + residual.astype(np.float64)
+    return y
+
+
+FUSED_CASES = [  # (m, n, k, g, algo name, tune) -- one per kernel family and tile variant
+    (1, 256, 1024, 128, "GEMV", 0), (3, 136, 640, 32, "GEMV_FIXUP", 0), (8, 200, 1536, 64, "GEMV_FIXUP", 2 | (4 << 4)),
+    (5, 256, 1024, 128, "GEMV", 0x8000 | 1 | (4 << 8)), (17, 136, 640, 32, "SKINNY", 0), (32, 256, 1024, 128, "SKINNY", 0),
+    (9, 520, 1056, 32, "SKINNY_WS", 1), (16, 264, 2048, 128, "SKINNY_WS", 4), (32, 256, 1024, 128, "SKINNY_WS", 2),
+    (70, 264, 704, 64, "GEMM", 1), (70, 264, 704, 64, "GEMM", 2), (300, 520, 1056, 32, "GEMM", 4),
+    (300, 520, 1056, 32, "GEMM", 8), (300, 520, 1056, 32, "GEMM", 9), (300, 520, 1056, 32, "GEMM", 10),
+]
+
+
+@pytest.mark.parametrize("m,n,k,g,algo_name,tune", FUSED_CASES)
+@pytest.mark.parametrize("use_bias,use_res,act", [(True, False, 0), (False, True, 0), (True, True, 1), (False, False, 1)])
+def test_fused_epilogue_every_kernel(capi, m, n, k, g, algo_name, tune, use_bias, use_res, act):
+    d = linear(n, k, g, seed=31)
+    rng = np.random.default_rng(32)
+    x = orc.synth_x(m, k, seed=33)
+    bias = rng.normal(0, 2.0, size=n).astype(np.float16) if use_bias else None
+    res = rng.normal(0, 2.0, size=(m, n)).astype(np.float16) if use_res else None
+    y_ref = fused_ref(x, d["w_hat"], bias, res, act)
+    algo = getattr(capi, "SQ_ALGO_" + algo_name) | (tune << 8)
+    y = capi.gemm_fused(to_dev(x), d["w_dev"], d["zs_dev"], n, k, g, bias=None if bias is None else to_dev(bias),
+                        residual=None if res is None else to_dev(res), act=act, algo=algo)
+    torch.cuda.synchronize()
+    y = y.float().cpu().numpy()
+    scale = np.max(np.abs(orc.gemm_ref(x, d["w_hat"])))
+    assert np.max(np.abs(y - y_ref)) <= TOL * scale
+    if act and not use_res:
+        assert y.min() >= 0.0
+
+
+def test_fused_epilogue_is_exactly_the_unfused_sum_in_fp32(capi):
+    # With bias = 0 and residual = 0 the fused call returns the same bits as the plain one; with a
+    # one-hot activation the result is fp16(W_hat[n, c] + bias[n] + residual) rounded once.
+    n, k, g = 4096, 4096, 128
+    d = linear(n, k, g, seed=7)
+    x = to_dev(orc.synth_x(4, k, seed=8))
+    zb = torch.zeros(n, dtype=torch.float16, device=DEV)
+    zr = torch.zeros((4, n), dtype=torch.float16, device=DEV)
+    assert torch.equal(capi.gemm_fused(x, d["w_dev"], d["zs_dev"], n, k, g, bias=zb, residual=zr),
+                       capi.gemm(x, d["w_dev"], d["zs_dev"], n, k, g))
+    e = torch.zeros((1, k), dtype=torch.float16, device=DEV)
+    e[0, 77] = 1.0
+    rng = np.random.default_rng(3)
+    bias = rng.normal(0, 1, size=n).astype(np.float16)
+    res = rng.normal(0, 1, size=(1, n)).astype(np.float16)
+    # (exact-W_hat arithmetic mode: the default mode applies the scale in fp32 and is not W_hat to the bit)
+    y = capi.gemm_fused(e, d["w_dev"], d["zs_dev"], n, k, g, bias=to_dev(bias), residual=to_dev(res),
+                        algo=capi.SQ_ALGO_GEMV).cpu().numpy()
+    want = (d["w_hat"][:, 77].astype(np.float32) + bias.astype(np.float32) + res[0].astype(np.float32)).astype(np.float16)
+    assert np.array_equal(y[0].view(np.int16), want.view(np.int16))
+
+
+def test_fused_rejects_bad_activation(capi):
+    d = linear(256, 1024, 128, seed=0)
+    x = to_dev(orc.synth_x(2, 1024))
+    with pytest.raises(capi.SqError) as ei:
+        capi.gemm_fused(x, d["w_dev"], d["zs_dev"], 256, 1024, 128, act=7)
+    assert ei.value.code == capi.SQ_ERR_BAD_ALGO
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 200])
+def test_quant_extension_fused_variants(m):
+    import quant
+    from sqamd.qlinear import WALinear
+    n, k, g = 512, 2048, 128
+    d = linear(n, k, g, seed=41)
+    rng = np.random.default_rng(42)
+    x = to_dev(orc.synth_x(m, k, seed=43)).reshape(1, m, k)
+    r = to_dev(rng.normal(0, 2.0, size=(1, m, n)).astype(np.float16))
+    b = to_dev(rng.normal(0, 2.0, size=(1, n)).astype(np.float16))
+    plain = quant.gemm_awq_ut(x, d["w_dev"], d["zs_dev"], m, n, k, g).float()
+    y = quant.gemm_awq_residual_ut(x, d["w_dev"], d["zs_dev"], r, m, n, k, g)
+    assert torch.allclose(y.float(), plain + r.float(), atol=2e-2, rtol=2e-2)  # the reference test's own tolerance
+    lin = WALinear(k, n, w_bit=4, group_size=g, bias=True, dev=DEV)
+    lin.weight, lin.zeros_scales, lin.bias = d["w_dev"], d["zs_dev"], b
+    y2 = lin(x.reshape(m, k), residual=r.reshape(m, n), act="relu")
+    want = torch.relu(plain.reshape(m, n) + b.float()) + r.reshape(m, n).float()
+    assert y2.shape == (m, n)
+    assert torch.allclose(y2.float(), want, atol=2e-2, rtol=2e-2)
+    assert torch.allclose(lin(x).float(), plain + b.float(), atol=2e-2, rtol=2e-2)
+    with pytest.raises((RuntimeError, ValueError)):
+        quant.gemm_awq_fused_ut(x, d["w_dev"], d["zs_dev"], None, None, "gelu", n, g)
+    with pytest.raises((RuntimeError, ValueError)):
+        quant.gemm_awq_residual_ut(x, d["w_dev"], d["zs_dev"], r[:, :, :8].contiguous(), m, n, k, g)
