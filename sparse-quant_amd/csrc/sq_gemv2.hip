@@ -22,7 +22,8 @@
 //   exact : B = fp16((q - z) * s), bit-identical to the reference's W_hat.
 //   fixup : B = 64 + q (bit pattern only); per run of 32 k the lane adds
 //           s * (sum x*(64+q) - (64+z) * sum x): zero and scale are applied once per
-//           run in fp32 instead of once per weight in fp16.
+//           run in fp32 instead of once per weight in fp16 (with more than 4 tokens the
+//           zero-point term comes from a second matrix instruction instead of staged sums).
 // (replaces w4a16_bs1_kernel / w4a16_bs2_kernel, reference:
 // quantization/muxi/backend/w4a16_gemm.cuh:14-151,153-326)
 #include "sq_common.h"
@@ -37,6 +38,10 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
                                                              half_t* __restrict__ Y, int M, int N, int K,
                                                              int gshift, Epilogue epi) {
     constexpr int MT = (MROWS + 3) / 4;
+    // Fixup mode, where the zero point is applied: with up to 4 tokens through per-run activation
+    // sums staged beside the activations; with more, where that vector arithmetic starts to
+    // bound the kernel, by a second matrix instruction with B = -(64 + z).
+    constexpr bool ZMFMA = MROWS > 4;
     constexpr int PITCH = 1024 * S + 16;                 // bytes per staged activation row
     constexpr int NT = 64 * NR * KS;
     constexpr int STAGE_TOTAL = KS * MROWS * S * 64;     // 128-bit words staged per round
@@ -104,7 +109,7 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
             const int m = (idx / (S * 64)) % MROWS;
             const int w8 = idx % (S * 64);
             if (idx < STAGE_TOTAL) *(u32x4_t*)(&xbuf[q][m * PITCH + w8 * 16]) = xr[p];
-            if (FIXUP) {
+            if (FIXUP && !ZMFMA) {
                 const half8_t h = bit_cast<half8_t>(xr[p]);
                 float sum = 0.f;
 #pragma unroll
@@ -142,6 +147,8 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
                 float4_t tmp[MT];
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++) tmp[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                const half_t nz = -p.x;
+                const half4_t nzb = {nz, nz, nz, nz};
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
                     const half8_t wv = unpack8_raw(wq[s][t], nm);
@@ -149,6 +156,10 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
                     for (int mt = 0; mt < MT; mt++) {
                         tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, wv.lo, tmp[mt], 0, 0, 0);
                         tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].hi, wv.hi, tmp[mt], 0, 0, 0);
+                        if (ZMFMA) {
+                            tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, nzb, tmp[mt], 0, 0, 0);
+                            tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].hi, nzb, tmp[mt], 0, 0, 0);
+                        }
                     }
                 }
                 const float zf = (float)p.x;
@@ -158,7 +169,8 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
                 for (int mt = 0; mt < MT; mt++)
 #pragma unroll
                     for (int j = 0; j < 4; j++)
-                        if (4 * mt + j < MROWS) acc[mt][j] += sf * (tmp[mt][j] - zf * xs[4 * mt + j]);
+                        if (4 * mt + j < MROWS)
+                            acc[mt][j] += ZMFMA ? sf * tmp[mt][j] : sf * (tmp[mt][j] - zf * xs[4 * mt + j]);
             }
         }
     }

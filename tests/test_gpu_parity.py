@@ -174,13 +174,22 @@ def test_zero_output_when_q_equals_z(capi, algo_name, m):
 
 
 def test_gemv_rows_do_not_depend_on_batch(capi):
+    # A token's output does not depend on which other tokens share the launch.  The fixup mode has two
+    # arithmetic paths (up to 4 tokens / 5 to 8 tokens), so the comparison stays inside each; the exact
+    # mode has one.
     n, k, g = 1024, 4096, 128
     d = linear(n, k, g, seed=9)
     x = to_dev(orc.synth_x(8, k, seed=10))
-    y8 = capi.gemm(x, d["w_dev"], d["zs_dev"], n, k, g, algo=capi.SQ_ALGO_GEMV_FIXUP)
+    run = lambda t, algo: capi.gemm(t.contiguous(), d["w_dev"], d["zs_dev"], n, k, g, algo=algo)
+    y4 = run(x[:4], capi.SQ_ALGO_GEMV_FIXUP)
+    for m in (0, 3):
+        assert torch.equal(run(x[m:m + 1], capi.SQ_ALGO_GEMV_FIXUP)[0], y4[m])
+    y8 = run(x, capi.SQ_ALGO_GEMV_FIXUP)
+    y5 = run(x[3:8], capi.SQ_ALGO_GEMV_FIXUP)
+    assert torch.equal(y5, y8[3:8])
+    y8e = run(x, capi.SQ_ALGO_GEMV)
     for m in (0, 3, 7):
-        y1 = capi.gemm(x[m:m + 1].contiguous(), d["w_dev"], d["zs_dev"], n, k, g, algo=capi.SQ_ALGO_GEMV_FIXUP)
-        assert torch.equal(y1[0], y8[m])
+        assert torch.equal(run(x[m:m + 1], capi.SQ_ALGO_GEMV)[0], y8e[m])
 
 
 # ------------------------------------------------------------------ edge cases
