@@ -20,6 +20,7 @@ Also printed on the same JSON line:
   cpu_baseline  the CPU restatement of the same path (oracle/) timed on this box's
                 host cores on one step
   prefill       TFLOP/s of the M = 2048 linears (second half of the metric)
+  decode_batch  GB/s of the same six linears at M = 4, 8, 16, 32
 
 `--m`, `--group` and `--shapes` select other points of the same workload family.
 """
@@ -229,6 +230,7 @@ def main():
     if not args.no_extras:
         # Additional, separately labelled legs; none of them feeds `value`.
         try:
+            out["decode_batch"] = decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream)
             out["fused_qkv"] = fused_qkv_leg(torch, capi, m, g, dev, gen, stream, args.layers, bytes_per_step)
             out["attention"] = attention_leg(torch, capi, dev)
             from sqamd import opt_decode
@@ -300,6 +302,43 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
     return {"m": m, "tflops": round(tf, 1), "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
             "dense_fp16_library_tflops": round(tfd, 1), "vs_dense_fp16_library": round(tf / tfd, 3),
             "nominal_shader_mhz": 2400, "per_linear": res}
+
+
+def decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream):
+    """GB/s of the same six linears at decode batches M = 4, 8, 16, 32 (BASELINE.json configs[1]), through
+    the product dispatch with its workspace (sq_w4a16_gemm_ws), HIP-graph replay over the rotating pool."""
+    res = {}
+    for m in (4, 8, 16, 32):
+        xs = {k: torch.randn((m, k), device=dev, generator=gen).half() for k in {k for _, _, k in shapes}}
+        ys = {n: torch.empty((m, n), dtype=torch.float16, device=dev) for n in {n for _, n, _ in shapes}}
+        bytes_per_step = sum(algorithmic_bytes(m, n, k, g) for _, n, k in shapes)
+        with torch.cuda.stream(stream):
+            ws = capi.workspace(m, 16384, 16384, dev, stream)
+
+            def run(i):
+                for (w, zs), (_, n, k) in zip(pool[i % len(pool)], shapes):
+                    capi.gemm_ws(xs[k], w, zs, n, k, g, out=ys[n], stream=stream, ws=ws)
+            for i in range(len(pool)):
+                run(i)
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(len(pool)):
+                    run(i)
+            for _ in range(5):
+                graph.replay()
+            reps = 60
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(reps):
+                graph.replay()
+            e1.record(stream)
+            stream.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * len(pool))
+        res["m%d" % m] = {"us_per_step": round(us, 2), "gbs": round(bytes_per_step / us / 1e3, 1),
+                          "frac_of_hbm_peak": round(bytes_per_step / us / 1e3 / HBM_PEAK_GBS, 4)}
+    return res
 
 
 def fused_qkv_leg(torch, capi, m, g, dev, gen, stream, layers, bytes_per_step):

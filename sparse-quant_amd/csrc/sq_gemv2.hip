@@ -255,7 +255,10 @@ hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void
     const int nsteps = (K + 511) / 512;
     // Measured on MI355X (cold weights, M = 1): K = 16384 wants 4 k ranges x 2 row groups,
     // 16384 x 4096 wants 2 x 4, 4096 x 4096 wants 1 x 4.
-    if (ks != 1 && ks != 2 && ks != 4) ks = nsteps > 16 ? 4 : (((long)N * K >= (1L << 25) && nsteps >= 8) ? 2 : 1);
+    if (ks != 1 && ks != 2 && ks != 4) {
+        ks = nsteps > 16 ? 4 : (((long)N * K >= (1L << 25) && nsteps >= 8) ? 2 : 1);
+        if (M >= 3 && M <= 4 && ks == 1 && nsteps >= 8) ks = 2;  // 4096 x 4096 with 3..4 tokens: 4.5 vs 5.6 us
+    }
     if (nr != 2 && nr != 4 && nr != 8) nr = ks == 4 ? 2 : 4;
     const int spw = (nsteps + ks - 1) / ks;
     if (M <= 1) return launch_rows<1>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
