@@ -20,8 +20,9 @@
 //                 and 32s+16+4g+{0..3}; A = V^T rows read from an LDS copy of the V
 //                 tile that was transposed while staging (two 64-bit reads);
 //                 D: lane (query l%16) holds head-dim rows 16*dt + 4*(l/16) + v.
-// K and V tiles are staged once per block for the four waves; V is transposed on the
-// way in (each thread packs two adjacent keys into 32-bit LDS writes).
+// K and V tiles are staged once per block for the four waves (global -> registers one
+// visited block ahead -> LDS); V is transposed on the way in (each thread packs two
+// adjacent keys into 32-bit LDS writes).
 #include "sq_common.h"
 #include "sq_kernels.h"
 
@@ -32,8 +33,14 @@ __global__ __launch_bounds__(256) void lut_attn_kernel(const half_t* __restrict_
                                                        const half_t* __restrict__ V, half_t* __restrict__ O,
                                                        const void* __restrict__ lut, int lut_is_64, int H, int S,
                                                        int nblk_q, int nnz, int nvisit, float qk_scale, int causal) {
-    constexpr int KP = D + 8;    // halves per row of the K tile in LDS
-    constexpr int VP = 64 + 8;   // halves per row of the transposed V tile in LDS
+#ifndef SQ_ATTN_KPAD
+#define SQ_ATTN_KPAD 16
+#endif
+#ifndef SQ_ATTN_VPAD
+#define SQ_ATTN_VPAD 12
+#endif
+    constexpr int KP = D + SQ_ATTN_KPAD;    // halves per row of the K tile in LDS
+    constexpr int VP = 64 + SQ_ATTN_VPAD;   // halves per row of the transposed V tile in LDS
     constexpr int DK = D / 32;   // k-steps of S^T
     constexpr int DT = D / 16;   // row tiles of O^T
     __shared__ __attribute__((aligned(16))) half_t ks[64 * KP];
@@ -66,40 +73,72 @@ __global__ __launch_bounds__(256) void lut_attn_kernel(const half_t* __restrict_
     for (int dt = 0; dt < DT; dt++) acc[dt] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
     const long lut_row = ((long)h * nblk_q + qb) * nnz;
-    int last = -1;
-    for (int j = 0; j < nvisit; j++) {
-        const int blk = lut_is_64 ? (int)((const long long*)lut)[lut_row + j] : ((const int*)lut)[lut_row + j];
-        const bool skip = (blk == last) || blk < 0 || (long)blk * 64 >= S;
-        last = blk;
-        if (skip) continue;  // uniform over the workgroup
-        const int n0 = blk * 64;
-
-        __syncthreads();  // the previous tiles are no longer read
+    // Tiles travel global -> registers -> LDS; the registers of the next visited block are
+    // requested before the current block is consumed, so their latency hides behind it.
+    u32x4_t kreg[D / 32];
+    half8_t v0reg[D / 64], v1reg[D / 64];
+    auto fetch = [&](int n0) {
         // K tile: 64 keys x D halves, 16 bytes per thread per pass.
 #pragma unroll
         for (int p = 0; p < D / 32; p++) {
             const int idx = tid + 256 * p;
             const int key = idx / (D / 8);
             const int c8 = idx % (D / 8);
-            const u32x4_t v = *(const u32x4_t*)(Kp + base + (long)imin(n0 + key, S - 1) * D + 8 * c8);
-            *(u32x4_t*)(&ks[key * KP + 8 * c8]) = v;
+            kreg[p] = *(const u32x4_t*)(Kp + base + (long)imin(n0 + key, S - 1) * D + 8 * c8);
         }
-        // V tile, transposed: a thread takes keys 2kp, 2kp+1 and 8 head-dim values and
-        // writes 8 packed pairs vt[d][2kp .. 2kp+1].
+        // V tile: a thread takes keys 2kp, 2kp+1 and 8 head-dim values.
 #pragma unroll
         for (int p = 0; p < D / 64; p++) {
             const int idx = tid + 256 * p;
             const int kp = idx & 31;
             const int c8 = idx >> 5;
-            const half8_t v0 = *(const half8_t*)(V + base + (long)imin(n0 + 2 * kp, S - 1) * D + 8 * c8);
-            const half8_t v1 = *(const half8_t*)(V + base + (long)imin(n0 + 2 * kp + 1, S - 1) * D + 8 * c8);
+            v0reg[p] = *(const half8_t*)(V + base + (long)imin(n0 + 2 * kp, S - 1) * D + 8 * c8);
+            v1reg[p] = *(const half8_t*)(V + base + (long)imin(n0 + 2 * kp + 1, S - 1) * D + 8 * c8);
+        }
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int p = 0; p < D / 32; p++) {
+            const int idx = tid + 256 * p;
+            const int key = idx / (D / 8);
+            const int c8 = idx % (D / 8);
+            *(u32x4_t*)(&ks[key * KP + 8 * c8]) = kreg[p];
+        }
+        // V transposed: 8 packed pairs vt[d][2kp .. 2kp+1] per pass.
+#pragma unroll
+        for (int p = 0; p < D / 64; p++) {
+            const int idx = tid + 256 * p;
+            const int kp = idx & 31;
+            const int c8 = idx >> 5;
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                const half2_t pr = {v0[e], v1[e]};
+                const half2_t pr = {v0reg[p][e], v1reg[p][e]};
                 *(half2_t*)(&vt[(8 * c8 + e) * VP + 2 * kp]) = pr;
             }
         }
+    };
+    // Next visited block (first key index) or -1; a LUT entry equal to its predecessor is
+    // padding.  Uniform over the workgroup.
+    int jn = 0, last = -1;
+    auto advance = [&]() {
+        while (jn < nvisit) {
+            const int blk = lut_is_64 ? (int)((const long long*)lut)[lut_row + jn] : ((const int*)lut)[lut_row + jn];
+            jn++;
+            const bool skip = (blk == last) || blk < 0 || (long)blk * 64 >= S;
+            last = blk;
+            if (!skip) return blk * 64;
+        }
+        return -1;
+    };
+
+    int n0 = advance();
+    if (n0 >= 0) fetch(n0);
+    while (n0 >= 0) {
+        __syncthreads();  // the previous tiles are no longer read
+        stash();
         __syncthreads();
+        const int n1 = advance();
+        if (n1 >= 0) fetch(n1);
 
         // S^T = K Q^T for the four 16-key tiles.
         float4_t st[4];
@@ -112,30 +151,40 @@ __global__ __launch_bounds__(256) void lut_attn_kernel(const half_t* __restrict_
                 st[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[s], st[t], 0, 0, 0);
             }
         }
-        // Masks and the block maximum of this query.
+        // Masks (only where the block touches the end of the sequence or the causal diagonal;
+        // the test is uniform over the workgroup) and the block maximum of this query.
+        const bool need_mask = (n0 + 64 > S) || (causal && n0 + 63 > qb * 64);
+        if (need_mask) {
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const int n = n0 + 16 * t + 4 * g + v;
+                    const bool keep = (n < S) && (!causal || n <= m);
+                    st[t][v] = keep ? st[t][v] : -INFINITY;
+                }
+        }
         float mx = -INFINITY;
 #pragma unroll
         for (int t = 0; t < 4; t++)
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const int n = n0 + 16 * t + 4 * g + v;
-                const bool keep = (n < S) && (!causal || n <= m);
-                st[t][v] = keep ? st[t][v] : -INFINITY;
-                mx = fmaxf(mx, st[t][v]);
-            }
+            for (int v = 0; v < 4; v++) mx = fmaxf(mx, st[t][v]);
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
         const float m_new = fmaxf(m_i, mx);
         // A query with nothing visible so far keeps p = 0 and alpha = 1 (no NaN from inf - inf).
+        // exp2 is the bare v_exp_f32: arguments are <= 0 and results below the normal range
+        // may flush to zero, which is far below the fp16 resolution of P.
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = (m_i == -INFINITY) ? (m_new == -INFINITY ? 1.f : 0.f) : exp2f(m_i - m_new);
+        const float alpha = (m_i == -INFINITY) ? (m_new == -INFINITY ? 1.f : 0.f)
+                                               : __builtin_amdgcn_exp2f(m_i - m_new);
         float rs = 0.f;
         half8_t pk[2];
 #pragma unroll
         for (int t = 0; t < 4; t++)
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const float p = exp2f(st[t][v] - m_use);  // exp2(-inf) = 0 for masked entries
+                const float p = __builtin_amdgcn_exp2f(st[t][v] - m_use);  // exp2(-inf) = 0 for masked entries
                 rs += p;
                 pk[t >> 1][4 * (t & 1) + v] = (half_t)p;
             }
@@ -143,11 +192,15 @@ __global__ __launch_bounds__(256) void lut_attn_kernel(const half_t* __restrict_
         rs += __shfl_xor(rs, 32);
         l_i = l_i * alpha + rs;
         m_i = m_new;
+        // The accumulators are rescaled only when some query of the wave saw its maximum grow.
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+            for (int dt = 0; dt < DT; dt++) acc[dt] *= alpha;
+        }
 
-        // O^T = O^T * alpha + V^T P^T.
+        // O^T += V^T P^T.
 #pragma unroll
         for (int dt = 0; dt < DT; dt++) {
-            acc[dt] *= alpha;
 #pragma unroll
             for (int s = 0; s < 2; s++) {
                 const half_t* vp = &vt[(16 * dt + lq) * VP + 32 * s + 4 * g];
@@ -157,6 +210,7 @@ __global__ __launch_bounds__(256) void lut_attn_kernel(const half_t* __restrict_
                 acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<half8_t>(a), pk[s], acc[dt], 0, 0, 0);
             }
         }
+        n0 = n1;
     }
 
     // O[m][16*dt + 4g + v] = acc / l.

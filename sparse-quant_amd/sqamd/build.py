@@ -30,6 +30,16 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-W
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 
+# Kernels whose accumulators are also touched by vector arithmetic (per-group fixups, softmax
+# rescaling): keep matrix-instruction results in ordinary VGPRs so that the compiler does not
+# shuttle them through the accumulation registers (hundreds of v_accvgpr moves otherwise).
+PER_FILE_FLAGS = {
+    "sq_gemv2.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "sq_skinny2.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "sq_attn.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
+
+
 def _run(cmd):
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops' is not a recognized feature" not in l)
@@ -48,7 +58,7 @@ def build_lib(verbose=True):
 
     def compile_one(pair):
         src, obj = pair
-        _run([hipcc] + HIP_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+        _run([hipcc] + HIP_FLAGS + PER_FILE_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj])
         return obj
 
     with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
