@@ -44,13 +44,13 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
     int kernel = algo & 0xFF;
     const int tune = (algo >> 8) & 0xFFFF;
     if (kernel == SQ_ALGO_AUTO) {
-        // Measured on OPT-6.7B shapes.  With a workspace the split-K kernel wins once the
-        // weight is large enough (fc1/fc2 class) for 9..32 tokens, and for 5..8 tokens when K
-        // is long.  Without one: the GEMV up to 4 tokens (up to 8 when K is short: its staged
+        // Measured on OPT-6.7B shapes.  With a workspace the split-K kernel wins for 5..32
+        // tokens once the weight is large enough (fc1/fc2 class) or K is long, and for 17..32
+        // tokens on any weight.  Without one: the GEMV up to 4 tokens (up to 8 when K is short: its staged
         // activations would otherwise need several sequential rounds), the 16-column kernel up
         // to 32, the tiled GEMM beyond.
         const bool large = (long)N * (long)K >= (1L << 25);
-        if (workspace && ((M > 8 && M <= 32 && large) || (M > 4 && M <= 8 && K > 8192)))
+        if (workspace && M > 4 && M <= 32 && (large || M > 16 || K > 8192))
             kernel = SQ_ALGO_SKINNY_WS;
         else if (M <= 4 || (M <= 8 && K <= 8192))
             kernel = SQ_ALGO_GEMV_FIXUP;

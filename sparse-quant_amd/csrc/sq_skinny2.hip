@@ -36,23 +36,47 @@ constexpr int SK2_XPITCH = 272;           // bytes per staged token row (256 + 1
 constexpr int SK2_ZCOLS = 32;             // groups per row held in LDS
 constexpr int SK2_ZPITCH = 33;
 
+// 128-bit global accesses at the device-coherent level (cache policy sc1, what agent-scope
+// relaxed atomics use), for data exchanged between workgroups inside one kernel.  The eight
+// loads and the wait for them are one asm statement, so the compiler never sees a register
+// whose data is still in flight.
+__device__ __forceinline__ void store_coherent_x4(float* p, float4_t v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void load8_coherent_x4(const float* const (&p)[8], float4_t (&v)[8]) {
+    asm volatile(
+        "global_load_dwordx4 %0, %8, off sc1\n\t"
+        "global_load_dwordx4 %1, %9, off sc1\n\t"
+        "global_load_dwordx4 %2, %10, off sc1\n\t"
+        "global_load_dwordx4 %3, %11, off sc1\n\t"
+        "global_load_dwordx4 %4, %12, off sc1\n\t"
+        "global_load_dwordx4 %5, %13, off sc1\n\t"
+        "global_load_dwordx4 %6, %14, off sc1\n\t"
+        "global_load_dwordx4 %7, %15, off sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
+        : "memory");
+}
+
 __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <int MT, int NWV, int S, bool FIXUP>
+template <int MT, int NWV, int S, int RT, bool FIXUP>
 __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __restrict__ W,
                                                            const half2_t* __restrict__ ZS,
                                                            const half_t* __restrict__ X, half_t* __restrict__ Y,
                                                            float* part, unsigned* counters, int M, int N, int K,
                                                            int gshift, int ksplit, Epilogue epi) {
-    constexpr int TILE = 4 * MT * 4 * 64;  // floats a wave contributes: [rt][mt][v][lane]
+    constexpr int TILE = RT * MT * 4 * 64;  // floats a wave contributes: [rt][mt][v][lane]
+    constexpr int ROWS = 16 * RT;           // weight rows per workgroup
     constexpr int XBUF = MT * 16 * SK2_XPITCH;
     constexpr int SH_BYTES = NWV * XBUF > NWV * TILE * 4 ? NWV * XBUF : NWV * TILE * 4;
     __shared__ __attribute__((aligned(16))) uint8_t sh[SH_BYTES];  // activation staging, later the wave partials
-    __shared__ uint32_t zsl[64 * SK2_ZPITCH];
+    __shared__ uint32_t zsl[ROWS * SK2_ZPITCH];
     __shared__ unsigned last_flag;
     float* red = (float*)sh;
 
@@ -76,31 +100,31 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
 
     // Zeros/scales of the row block: loaded now (row-contiguous), parked in LDS after the
     // first weight loads have been issued so that they do not delay the weight stream.
-    constexpr int ZPT = (64 * SK2_ZCOLS) / (64 * NWV);
+    constexpr int ZPT = (ROWS * SK2_ZCOLS) / (64 * NWV);
     uint32_t zreg[ZPT];
     if (zs_lds) {
 #pragma unroll
         for (int p = 0; p < ZPT; p++) {
             const int idx = tid + p * 64 * NWV;
             const int r = idx >> 5, col = idx & 31;
-            const int row = imin(rb * 64 + r, N - 1);
+            const int row = imin(rb * ROWS + r, N - 1);
             zreg[p] = ((const uint32_t*)ZS)[(long)row * groups + g_begin + (col < ng ? col : 0)];
         }
     }
 
-    float4_t acc[4][MT];
+    float4_t acc[RT][MT];
 #pragma unroll
-    for (int rt = 0; rt < 4; rt++)
+    for (int rt = 0; rt < RT; rt++)
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) acc[rt][mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
     const half8_t ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f,
                           (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
 
-    const uint8_t* wrow[4];
-    const uint32_t* zrow[4];
+    const uint8_t* wrow[RT];
+    const uint32_t* zrow[RT];
 #pragma unroll
-    for (int rt = 0; rt < 4; rt++) {
-        const int row = imin(rb * 64 + 16 * rt + li, N - 1);
+    for (int rt = 0; rt < RT; rt++) {
+        const int row = imin(rb * ROWS + 16 * rt + li, N - 1);
         wrow[rt] = W + (long)row * (K >> 1);
         zrow[rt] = (const uint32_t*)ZS + (long)row * groups;
     }
@@ -115,9 +139,9 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
     for (int cb = c_begin; cb < c_end; cb += S * NWV) {
         const int c0 = cb + S * wave;
         const bool active = c0 < c_end;
-        u32x4_t wq[S][4];
+        u32x4_t wq[S][RT];
         u32x4_t xr[2][4 * MT];
-        uint32_t zq[S][4];
+        uint32_t zq[S][RT];
         int zcol[S];
         auto load_x = [&](int c, u32x4_t* dst) {
             const int kx = (c << 7) + 8 * (lane & 15);
@@ -130,19 +154,27 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
             }
         };
         if (active) {
+            // (cache-allocating loads, the S chunks of a row back to back: consecutive chunks
+            // share a 128-byte line, which is then requested from L2 once instead of per chunk)
+            int kcs[S];
+#pragma unroll
+            for (int u = 0; u < S; u++) {
+                const int kk = ((c0 + u) << 7) + 32 * lj;
+                kcs[u] = ((c0 + u < c_end) && (kk < K)) ? kk : 0;
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+                for (int u = 0; u < S; u++) wq[u][rt] = *(const u32x4_t*)(wrow[rt] + (kcs[u] >> 1));
 #pragma unroll
             for (int u = 0; u < S; u++) {
                 const int c = c0 + u;
                 const int kk = (c << 7) + 32 * lj;
                 const bool valid = (c < c_end) && (kk < K);
-                const int kc = valid ? kk : 0;
-#pragma unroll
-                for (int rt = 0; rt < 4; rt++)
-                    wq[u][rt] = __builtin_nontemporal_load((const u32x4_t*)(wrow[rt] + (kc >> 1)));
                 zcol[u] = valid ? (((c - c_begin) << gpc_shift) + ((32 * lj) >> gshift)) : 0;
                 if (!zs_lds) {
 #pragma unroll
-                    for (int rt = 0; rt < 4; rt++) zq[u][rt] = zrow[rt][valid ? (kk >> gshift) : g_begin];
+                    for (int rt = 0; rt < RT; rt++) zq[u][rt] = zrow[rt][valid ? (kk >> gshift) : g_begin];
                 }
             }
             load_x(c0, xr[0]);
@@ -173,7 +205,7 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
                     for (int t = 0; t < 4; t++) xa[mt][t] = *(const u32x4_t*)(xb_rd + 16 * mt * SK2_XPITCH + 16 * t);
                 if (zs_lds) {
 #pragma unroll
-                    for (int rt = 0; rt < 4; rt++) zq[u][rt] = zsl[(16 * rt + li) * SK2_ZPITCH + zcol[u]];
+                    for (int rt = 0; rt < RT; rt++) zq[u][rt] = zsl[(16 * rt + li) * SK2_ZPITCH + zcol[u]];
                 }
                 float4_t xs[MT];
                 if (FIXUP) {
@@ -187,7 +219,7 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
                     }
                 }
 #pragma unroll
-                for (int rt = 0; rt < 4; rt++) {
+                for (int rt = 0; rt < RT; rt++) {
                     const half2_t zsv = bit_cast<half2_t>(zq[u][rt]);
                     if (!FIXUP) {
                         const half2_t z64 = {zsv.x, zsv.x};
@@ -227,7 +259,7 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
 
     // Sum the waves' partial tiles: red[wave][rt][mt][v][lane].
 #pragma unroll
-    for (int rt = 0; rt < 4; rt++)
+    for (int rt = 0; rt < RT; rt++)
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
@@ -243,7 +275,7 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
             for (int p = 0; p < NWV; p++) sum += red[p * TILE + t];
             const int l = t & 63, v = (t >> 6) & 3, mt = (t >> 8) % MT, rt = (t >> 8) / MT;
             const int m = 16 * mt + 4 * (l >> 4) + v;
-            const int n = rb * 64 + 16 * rt + (l & 15);
+            const int n = rb * ROWS + 16 * rt + (l & 15);
             if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum, m, n, N, epi);
         }
         return;
@@ -253,12 +285,14 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
     // release/acquire fence (which would write back and invalidate the whole L2) is needed:
     // the wait for outstanding vector memory operations orders the partial stores before
     // the counter increment, and the last arriver reads the partials past its own caches.
+    // (128-bit accesses with the same cache policy bit the compiler gives those atomics: the
+    // exchange is bound by the number of requests, not by bytes.)
     float* mine = part + ((long)ks * gridDim.x + rb) * TILE;
-    for (int t = tid; t < TILE; t += 64 * NWV) {
-        float sum = 0.f;
+    for (int t4 = tid * 4; t4 < TILE; t4 += 4 * 64 * NWV) {
+        float4_t sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int p = 0; p < NWV; p++) sum += red[p * TILE + t];
-        __hip_atomic_store(mine + t, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int p = 0; p < NWV; p++) sum += *(const float4_t*)(&red[p * TILE + t4]);
+        store_coherent_x4(mine + t4, sum);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -268,15 +302,25 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
     }
     __syncthreads();
     if (!last_flag) return;
-    for (int t = tid; t < TILE; t += 64 * NWV) {
-        float sum = 0.f;
-        for (int q = 0; q < ksplit; q++)
-            sum += __hip_atomic_load(part + ((long)q * gridDim.x + rb) * TILE + t, __ATOMIC_RELAXED,
-                                     __HIP_MEMORY_SCOPE_AGENT);
-        const int l = t & 63, v = (t >> 6) & 3, mt = (t >> 8) % MT, rt = (t >> 8) / MT;
-        const int m = 16 * mt + 4 * (l >> 4) + v;
-        const int n = rb * 64 + 16 * rt + (l & 15);
-        if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum, m, n, N, epi);
+    for (int t4 = tid * 4; t4 < TILE; t4 += 4 * 64 * NWV) {
+        // eight loads regardless of ksplit (absent partials re-read partial 0 and are dropped)
+        const float* src[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) src[q] = part + ((long)(q < ksplit ? q : 0) * gridDim.x + rb) * TILE + t4;
+        float4_t pv[8];
+        load8_coherent_x4(src, pv);
+        float4_t sum = pv[0];
+#pragma unroll
+        for (int q = 1; q < 8; q++)
+            if (q < ksplit) sum += pv[q];  // fixed order
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int t = t4 + e;
+            const int l = t & 63, v = (t >> 6) & 3, mt = (t >> 8) % MT, rt = (t >> 8) / MT;
+            const int m = 16 * mt + 4 * (l >> 4) + v;
+            const int n = rb * ROWS + 16 * rt + (l & 15);
+            if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum[e], m, n, N, epi);
+        }
     }
     // leave the workspace ready for the next call
     if (tid == 0) __hip_atomic_store(&counters[rb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -288,17 +332,17 @@ size_t skinny2_workspace_bytes(int M, int N, int K) {
     return (size_t)SK2_COUNTER_BYTES + (size_t)8 * row_blocks * (4 * mt * 4 * 64) * sizeof(float);
 }
 
-template <int MT, int NWV, int S>
+template <int MT, int NWV, int S, int RT>
 static hipError_t launch_cfg(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                              int gshift, bool fixup, int ksplit, Epilogue epi, hipStream_t st) {
-    const dim3 grid((N + 63) / 64, ksplit);
+    const dim3 grid((N + 16 * RT - 1) / (16 * RT), ksplit);
     unsigned* counters = (unsigned*)ws;
     float* part = (float*)((char*)ws + SK2_COUNTER_BYTES);
     if (fixup)
-        hipLaunchKernelGGL((skinny2_kernel<MT, NWV, S, true>), grid, dim3(64 * NWV), 0, st, (const uint8_t*)w,
+        hipLaunchKernelGGL((skinny2_kernel<MT, NWV, S, RT, true>), grid, dim3(64 * NWV), 0, st, (const uint8_t*)w,
                            (const half2_t*)zs, (const half_t*)x, (half_t*)y, part, counters, M, N, K, gshift, ksplit, epi);
     else
-        hipLaunchKernelGGL((skinny2_kernel<MT, NWV, S, false>), grid, dim3(64 * NWV), 0, st, (const uint8_t*)w,
+        hipLaunchKernelGGL((skinny2_kernel<MT, NWV, S, RT, false>), grid, dim3(64 * NWV), 0, st, (const uint8_t*)w,
                            (const half2_t*)zs, (const half_t*)x, (half_t*)y, part, counters, M, N, K, gshift, ksplit, epi);
     return hipGetLastError();
 }
@@ -313,13 +357,17 @@ hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, vo
     while ((1 << gshift) < g) gshift++;
     const int mt = (M + 15) / 16;
     const int nchunks = (K + 127) / 128;
-    const int row_blocks = (N + 63) / 64;
     int ksplit = tune & 0xFF;
     int nwv = (tune >> 12) & 0xF;
+    // Four 16-row tiles per wave (64 rows per workgroup); eight were measured and are slower:
+    // the registers they need leave one wave per SIMD.
+    const int row_blocks = (N + 63) / 64;
     if (ksplit != 1 && ksplit != 2 && ksplit != 4 && ksplit != 8) {
-        // about one workgroup per CU, each K range at least 8 chunks long
+        // At most one workgroup per CU (a second round of workgroups costs more than idle CUs:
+        // 12288 rows run 11.5 us as 192 workgroups, 16.5 us as 384), each K range at least 8
+        // chunks long.
         ksplit = 1;
-        while (ksplit < 8 && row_blocks * ksplit < 256 && nchunks / (ksplit * 2) >= 8) ksplit *= 2;
+        while (ksplit < 8 && row_blocks * ksplit * 2 <= 256 && nchunks / (ksplit * 2) >= 8) ksplit *= 2;
     }
     const int cps = (nchunks + ksplit - 1) / ksplit;
     if (nwv != 4 && nwv != 8) nwv = (mt == 1 && cps >= 16) ? 8 : 4;
@@ -327,9 +375,9 @@ hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, vo
     const int mode = (tune >> 8) & 0xF;
     bool fixup = (g == 128);
     if (mode == 1) fixup = false;
-    if (mt == 2) return launch_cfg<2, 4, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
-    if (nwv == 8) return launch_cfg<1, 8, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
-    return launch_cfg<1, 4, 2>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
+    if (mt == 2) return launch_cfg<2, 4, 2, 4>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
+    if (nwv == 8) return launch_cfg<1, 8, 2, 4>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
+    return launch_cfg<1, 4, 2, 4>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
 }
 
 }  // namespace sq

@@ -358,6 +358,8 @@ def test_skinny_ws_parity(capi, n, k, g, m):
     for ksplit in (1, 2, 4, 8):
         for mode in (1, 2):
             check_gemm_ws(capi, m, n, k, g, capi.SQ_ALGO_SKINNY_WS | ((ksplit | (mode << 8)) << 8))
+            # 4-wave workgroups
+            check_gemm_ws(capi, m, n, k, g, capi.SQ_ALGO_SKINNY_WS | ((ksplit | (mode << 8) | (4 << 12)) << 8))
 
 
 def test_skinny_ws_properties_and_workspace_reuse(capi):
