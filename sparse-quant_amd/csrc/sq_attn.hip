@@ -28,21 +28,29 @@
 
 namespace sq {
 
-template <int D>
-__global__ __launch_bounds__(256) void lut_attn_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ Kp,
-                                                       const half_t* __restrict__ V, half_t* __restrict__ O,
-                                                       const void* __restrict__ lut, int lut_is_64, int H, int S,
-                                                       int nblk_q, int nnz, int nvisit, float qk_scale, int causal) {
 #ifndef SQ_ATTN_KPAD
 #define SQ_ATTN_KPAD 16
 #endif
 #ifndef SQ_ATTN_VPAD
 #define SQ_ATTN_VPAD 12
 #endif
-    constexpr int KP = D + SQ_ATTN_KPAD;    // halves per row of the K tile in LDS
-    constexpr int VP = 64 + SQ_ATTN_VPAD;   // halves per row of the transposed V tile in LDS
-    constexpr int DK = D / 32;   // k-steps of S^T
-    constexpr int DT = D / 16;   // row tiles of O^T
+
+// QT = 16-query tiles per wave: the workgroup has 4 / QT waves, and every K / V operand read
+// from LDS feeds QT matrix instructions.  QT = 2 was measured (3 % slower at D = 64, 30 %
+// slower at D = 128, where it needs more than 256 registers); QT = 1 is what is launched.
+template <int D, int QT>
+__global__ __launch_bounds__(256 / QT) void lut_attn_kernel(const half_t* __restrict__ Q, const half_t* __restrict__ Kp,
+                                                            const half_t* __restrict__ V, half_t* __restrict__ O,
+                                                            const void* __restrict__ lut, int lut_is_64, int H, int S,
+                                                            int nblk_q, int nnz, int nvisit, float qk_scale,
+                                                            int causal) {
+    constexpr int NT = 256 / QT;                 // threads per workgroup
+    constexpr int KP = D + SQ_ATTN_KPAD;         // halves per row of the K tile in LDS
+    constexpr int VP = 64 + SQ_ATTN_VPAD;        // halves per row of the transposed V tile in LDS
+    constexpr int DK = D / 32;                   // k-steps of S^T
+    constexpr int DT = D / 16;                   // row tiles of O^T
+    constexpr int KPASS = (64 * D / 8) / NT;     // 16-byte words of the K tile per thread
+    constexpr int VPASS = (32 * D / 8) / NT;     // key pairs x 8 head-dim values of the V tile per thread
     __shared__ __attribute__((aligned(16))) half_t ks[64 * KP];
     __shared__ __attribute__((aligned(16))) half_t vt[D * VP];
 
@@ -55,41 +63,49 @@ __global__ __launch_bounds__(256) void lut_attn_kernel(const half_t* __restrict_
     const int zh = blockIdx.y;
     const int h = zh % H;
     const long base = (long)zh * S * D;
-    const int m = qb * 64 + 16 * wave + lq;  // this lane's query
-    const int mc = imin(m, S - 1);
+    int m[QT];  // this lane's queries
+#pragma unroll
+    for (int qt = 0; qt < QT; qt++) m[qt] = qb * 64 + 16 * (QT * wave + qt) + lq;
 
-    // Q^T operand: q * (sm_scale * log2 e), rounded to fp16.
-    half8_t qf[DK];
+    // Q^T operands: q * (sm_scale * log2 e), rounded to fp16.
+    half8_t qf[QT][DK];
 #pragma unroll
-    for (int s = 0; s < DK; s++) {
-        const half8_t raw = *(const half8_t*)(Q + base + (long)mc * D + 32 * s + 8 * g);
+    for (int qt = 0; qt < QT; qt++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) qf[s][e] = (half_t)((float)raw[e] * qk_scale);
+        for (int s = 0; s < DK; s++) {
+            const half8_t raw = *(const half8_t*)(Q + base + (long)imin(m[qt], S - 1) * D + 32 * s + 8 * g);
+#pragma unroll
+            for (int e = 0; e < 8; e++) qf[qt][s][e] = (half_t)((float)raw[e] * qk_scale);
+        }
+
+    float m_i[QT], l_i[QT];
+    float4_t acc[QT][DT];
+#pragma unroll
+    for (int qt = 0; qt < QT; qt++) {
+        m_i[qt] = -INFINITY;
+        l_i[qt] = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) acc[qt][dt] = (float4_t){0.f, 0.f, 0.f, 0.f};
     }
-
-    float m_i = -INFINITY, l_i = 0.f;
-    float4_t acc[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; dt++) acc[dt] = (float4_t){0.f, 0.f, 0.f, 0.f};
 
     const long lut_row = ((long)h * nblk_q + qb) * nnz;
     // Tiles travel global -> registers -> LDS; the registers of the next visited block are
     // requested before the current block is consumed, so their latency hides behind it.
-    u32x4_t kreg[D / 32];
-    half8_t v0reg[D / 64], v1reg[D / 64];
+    u32x4_t kreg[KPASS];
+    half8_t v0reg[VPASS], v1reg[VPASS];
     auto fetch = [&](int n0) {
         // K tile: 64 keys x D halves, 16 bytes per thread per pass.
 #pragma unroll
-        for (int p = 0; p < D / 32; p++) {
-            const int idx = tid + 256 * p;
+        for (int p = 0; p < KPASS; p++) {
+            const int idx = tid + NT * p;
             const int key = idx / (D / 8);
             const int c8 = idx % (D / 8);
             kreg[p] = *(const u32x4_t*)(Kp + base + (long)imin(n0 + key, S - 1) * D + 8 * c8);
         }
         // V tile: a thread takes keys 2kp, 2kp+1 and 8 head-dim values.
 #pragma unroll
-        for (int p = 0; p < D / 64; p++) {
-            const int idx = tid + 256 * p;
+        for (int p = 0; p < VPASS; p++) {
+            const int idx = tid + NT * p;
             const int kp = idx & 31;
             const int c8 = idx >> 5;
             v0reg[p] = *(const half8_t*)(V + base + (long)imin(n0 + 2 * kp, S - 1) * D + 8 * c8);
@@ -98,16 +114,16 @@ __global__ __launch_bounds__(256) void lut_attn_kernel(const half_t* __restrict_
     };
     auto stash = [&]() {
 #pragma unroll
-        for (int p = 0; p < D / 32; p++) {
-            const int idx = tid + 256 * p;
+        for (int p = 0; p < KPASS; p++) {
+            const int idx = tid + NT * p;
             const int key = idx / (D / 8);
             const int c8 = idx % (D / 8);
             *(u32x4_t*)(&ks[key * KP + 8 * c8]) = kreg[p];
         }
         // V transposed: 8 packed pairs vt[d][2kp .. 2kp+1] per pass.
 #pragma unroll
-        for (int p = 0; p < D / 64; p++) {
-            const int idx = tid + 256 * p;
+        for (int p = 0; p < VPASS; p++) {
+            const int idx = tid + NT * p;
             const int kp = idx & 31;
             const int c8 = idx >> 5;
 #pragma unroll
@@ -140,65 +156,72 @@ __global__ __launch_bounds__(256) void lut_attn_kernel(const half_t* __restrict_
         const int n1 = advance();
         if (n1 >= 0) fetch(n1);
 
-        // S^T = K Q^T for the four 16-key tiles.
-        float4_t st[4];
+        // S^T = K Q^T for the four 16-key tiles; a K operand serves all QT query tiles.
+        float4_t st[QT][4];
 #pragma unroll
         for (int t = 0; t < 4; t++) {
-            st[t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int qt = 0; qt < QT; qt++) st[qt][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int s = 0; s < DK; s++) {
                 const half8_t a = *(const half8_t*)(&ks[(16 * t + lq) * KP + 32 * s + 8 * g]);
-                st[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[s], st[t], 0, 0, 0);
+#pragma unroll
+                for (int qt = 0; qt < QT; qt++)
+                    st[qt][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[qt][s], st[qt][t], 0, 0, 0);
             }
         }
         // Masks (only where the block touches the end of the sequence or the causal diagonal;
-        // the test is uniform over the workgroup) and the block maximum of this query.
+        // the test is uniform over the workgroup).
         const bool need_mask = (n0 + 64 > S) || (causal && n0 + 63 > qb * 64);
-        if (need_mask) {
+        half8_t pk[QT][2];
+#pragma unroll
+        for (int qt = 0; qt < QT; qt++) {
+            if (need_mask) {
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const int n = n0 + 16 * t + 4 * g + v;
+                        const bool keep = (n < S) && (!causal || n <= m[qt]);
+                        st[qt][t][v] = keep ? st[qt][t][v] : -INFINITY;
+                    }
+            }
+            // block maximum of this query
+            float mx = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int v = 0; v < 4; v++) mx = fmaxf(mx, st[qt][t][v]);
+            mx = fmaxf(mx, __shfl_xor(mx, 16));
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float m_new = fmaxf(m_i[qt], mx);
+            // A query with nothing visible so far keeps p = 0 and alpha = 1 (no NaN from inf - inf).
+            // exp2 is the bare v_exp_f32: arguments are <= 0 and results below the normal range
+            // may flush to zero, which is far below the fp16 resolution of P.
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            const float alpha = (m_i[qt] == -INFINITY) ? (m_new == -INFINITY ? 1.f : 0.f)
+                                                       : __builtin_amdgcn_exp2f(m_i[qt] - m_new);
+            float rs = 0.f;
 #pragma unroll
             for (int t = 0; t < 4; t++)
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
-                    const int n = n0 + 16 * t + 4 * g + v;
-                    const bool keep = (n < S) && (!causal || n <= m);
-                    st[t][v] = keep ? st[t][v] : -INFINITY;
+                    const float p = __builtin_amdgcn_exp2f(st[qt][t][v] - m_use);  // exp2(-inf) = 0 for masked entries
+                    rs += p;
+                    pk[qt][t >> 1][4 * (t & 1) + v] = (half_t)p;
                 }
-        }
-        float mx = -INFINITY;
+            rs += __shfl_xor(rs, 16);
+            rs += __shfl_xor(rs, 32);
+            l_i[qt] = l_i[qt] * alpha + rs;
+            m_i[qt] = m_new;
+            // The accumulators are rescaled only when some query of the wave saw its maximum grow.
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
-        for (int t = 0; t < 4; t++)
-#pragma unroll
-            for (int v = 0; v < 4; v++) mx = fmaxf(mx, st[t][v]);
-        mx = fmaxf(mx, __shfl_xor(mx, 16));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_i, mx);
-        // A query with nothing visible so far keeps p = 0 and alpha = 1 (no NaN from inf - inf).
-        // exp2 is the bare v_exp_f32: arguments are <= 0 and results below the normal range
-        // may flush to zero, which is far below the fp16 resolution of P.
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = (m_i == -INFINITY) ? (m_new == -INFINITY ? 1.f : 0.f)
-                                               : __builtin_amdgcn_exp2f(m_i - m_new);
-        float rs = 0.f;
-        half8_t pk[2];
-#pragma unroll
-        for (int t = 0; t < 4; t++)
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const float p = __builtin_amdgcn_exp2f(st[t][v] - m_use);  // exp2(-inf) = 0 for masked entries
-                rs += p;
-                pk[t >> 1][4 * (t & 1) + v] = (half_t)p;
+                for (int dt = 0; dt < DT; dt++) acc[qt][dt] *= alpha;
             }
-        rs += __shfl_xor(rs, 16);
-        rs += __shfl_xor(rs, 32);
-        l_i = l_i * alpha + rs;
-        m_i = m_new;
-        // The accumulators are rescaled only when some query of the wave saw its maximum grow.
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
-#pragma unroll
-            for (int dt = 0; dt < DT; dt++) acc[dt] *= alpha;
         }
 
-        // O^T += V^T P^T.
+        // O^T += V^T P^T; a V operand serves all QT query tiles.
 #pragma unroll
         for (int dt = 0; dt < DT; dt++) {
 #pragma unroll
@@ -207,21 +230,27 @@ __global__ __launch_bounds__(256) void lut_attn_kernel(const half_t* __restrict_
                 const u32x2_t lo = *(const u32x2_t*)(vp);
                 const u32x2_t hi = *(const u32x2_t*)(vp + 16);
                 const u32x4_t a = {lo.x, lo.y, hi.x, hi.y};
-                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<half8_t>(a), pk[s], acc[dt], 0, 0, 0);
+#pragma unroll
+                for (int qt = 0; qt < QT; qt++)
+                    acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bit_cast<half8_t>(a), pk[qt][s], acc[qt][dt],
+                                                                         0, 0, 0);
             }
         }
         n0 = n1;
     }
 
     // O[m][16*dt + 4g + v] = acc / l.
-    if (m < S) {
-        const float inv = l_i > 0.f ? 1.f / l_i : 0.f;
 #pragma unroll
-        for (int dt = 0; dt < DT; dt++) {
-            half4_t o;
+    for (int qt = 0; qt < QT; qt++) {
+        if (m[qt] < S) {
+            const float inv = l_i[qt] > 0.f ? 1.f / l_i[qt] : 0.f;
 #pragma unroll
-            for (int v = 0; v < 4; v++) o[v] = (half_t)(acc[dt][v] * inv);
-            *(half4_t*)(O + base + (long)m * D + 16 * dt + 4 * g) = o;
+            for (int dt = 0; dt < DT; dt++) {
+                half4_t o;
+#pragma unroll
+                for (int v = 0; v < 4; v++) o[v] = (half_t)(acc[qt][dt][v] * inv);
+                *(half4_t*)(O + base + (long)m[qt] * D + 16 * dt + 4 * g) = o;
+            }
         }
     }
 }
@@ -234,12 +263,15 @@ hipError_t launch_lut_attention(const void* q, const void* k, const void* v, voi
     const float qk_scale = sm_scale * 1.44269504f;
     const int use_nnz = nnz < nblk ? nnz : nblk;  // the reference clamps NNZ to ceil(S / 64) as well
     // (the LUT row pitch stays nnz even when fewer entries are visited)
+#define SQ_ATTN_LAUNCH(D_, QT_)                                                                                   \
+    hipLaunchKernelGGL((lut_attn_kernel<D_, QT_>), grid, dim3(256 / QT_), 0, st, (const half_t*)q, (const half_t*)k, \
+                       (const half_t*)v, (half_t*)o, lut, lut_elem_bytes == 8, H, S, nblk, nnz, use_nnz, qk_scale,   \
+                       causal)
     if (D == 64)
-        hipLaunchKernelGGL((lut_attn_kernel<64>), grid, dim3(256), 0, st, (const half_t*)q, (const half_t*)k,
-                           (const half_t*)v, (half_t*)o, lut, lut_elem_bytes == 8, H, S, nblk, nnz, use_nnz, qk_scale, causal);
+        SQ_ATTN_LAUNCH(64, 1);
     else
-        hipLaunchKernelGGL((lut_attn_kernel<128>), grid, dim3(256), 0, st, (const half_t*)q, (const half_t*)k,
-                           (const half_t*)v, (half_t*)o, lut, lut_elem_bytes == 8, H, S, nblk, nnz, use_nnz, qk_scale, causal);
+        SQ_ATTN_LAUNCH(128, 1);
+#undef SQ_ATTN_LAUNCH
     return hipGetLastError();
 }
 
