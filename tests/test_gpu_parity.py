@@ -526,3 +526,47 @@ def test_quant_extension_fused_variants(m):
         quant.gemm_awq_fused_ut(x, d["w_dev"], d["zs_dev"], None, None, "gelu", n, g)
     with pytest.raises((RuntimeError, ValueError)):
         quant.gemm_awq_residual_ut(x, d["w_dev"], d["zs_dev"], r[:, :, :8].contiguous(), m, n, k, g)
+
+
+# ------------------------------------------------------------------ the reference's own kernel-test grids
+REF_DIMS = [(4096, 4096), (5120, 5120), (11008, 4096), (13696, 5120)]  # (in, out), gemm_awq_test.py "Dim"
+
+
+@pytest.mark.parametrize("k,n", REF_DIMS)
+def test_reference_grid_uint8_layout(k, n):
+    """quantization/muxi/script/gemm_awq_test.py:26-34,80-109: batch 1, sequence lengths 1..512, group 128,
+    x ~ N(0, 0.5), allclose(atol = rtol = 2e-2) against x @ W_hat^T (seeded here)."""
+    import quant
+    from sqamd import quant_funcs as qf
+    torch.manual_seed(k + n)
+    g = 128
+    lin = torch.nn.Linear(k, n, bias=False, device=DEV, dtype=torch.float16)
+    qweight, zeros_scales = qf.quant_muxi(lin.weight.data, k, n, n_bit=4, group_size=g)
+    w_fp16 = qf.dequant_to_fp16(lin.weight.data, 4, g).float()
+    for seq in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512):
+        x = torch.empty((1, seq, k), dtype=torch.float16, device=DEV).normal_(mean=0.0, std=0.5)
+        out = quant.gemm_awq_ut(x, qweight, zeros_scales, seq, n, k, g)
+        ref = torch.matmul(x.float(), w_fp16.t())
+        assert torch.allclose(ref, out.float(), atol=2e-2, rtol=2e-2), (k, n, seq)
+
+
+@pytest.mark.parametrize("k,n", REF_DIMS)
+def test_reference_grid_int32_layout(k, n):
+    """quantization/nvidia/script/gemm_awq_test.py:33-38,89-114: sequence lengths 1 and 128, batch sizes
+    1..64, group 128, weights in the tensor-core tile layout produced by the converter chain."""
+    import quant
+    from sqamd import quant_funcs as qf
+    torch.manual_seed(k * 3 + n)
+    g = 128
+    lin = torch.nn.Linear(k, n, bias=False, device=DEV, dtype=torch.float16)
+    qweight, zeros_scales = qf.quant_lmdeploy(lin.weight.data, k, n, group_size=g)
+    assert qweight.dtype == torch.int32 and tuple(qweight.shape) == (k, n // 8)
+    w_fp16 = qf.dequant_to_fp16(lin.weight.data, 4, g).float()
+    for seq in (1, 128):
+        for bs in (1, 2, 4, 8, 16, 32, 48, 64):
+            x = torch.empty((bs, seq, k), dtype=torch.float16, device=DEV).normal_(mean=0.0, std=0.5)
+            out = quant.gemm_awq_ut(x, qweight, zeros_scales, bs * seq, n, k, g)
+            ref = torch.matmul(x.float(), w_fp16.t())
+            assert tuple(out.shape) == (bs, seq, n)
+            assert torch.allclose(ref, out.float(), atol=2e-2, rtol=2e-2), (k, n, bs, seq)
+    quant.clear_repack_cache()
