@@ -80,7 +80,8 @@ int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y,
  * 64 KiB zeroed before the first call (every call leaves them zero); calls that
  * share a workspace must not overlap in time.  With SQ_ALGO_AUTO the split-K kernel
  * is taken where it is the fastest (5..32 tokens on weights of 2^25 elements or more
- * or with K > 8192, 17..32 tokens on any weight); everywhere else, and with an explicit other
+ * or with K > 8192, 17..32 tokens on any weight; 33..64 tokens on such weights and up to
+ * 128 tokens with K > 8192 run as blocks of 32 tokens); everywhere else, and with an explicit other
  * algo, the call behaves like sq_w4a16_gemm_ex and ignores the workspace. */
 int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y,
                      int M, int N, int K, int group_size, int layout, int algo,

@@ -218,17 +218,25 @@ hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void*
     int mi = tune & 0xFF;
     if (mi >= 8 && mi <= 10) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, mi - 8, epi, st);
     if (mi != 1 && mi != 2 && mi != 4) {
-        if (M > 64) {
-            // Measured on MI355X (the chip runs these kernels at a power-limited clock, so fewer
-            // instructions per flop is what counts): the 256-row tile halves the unpack work per
-            // flop and wins whenever its grid fills the 256 CUs evenly; otherwise the 128-row
-            // tiles, pipelined variant for long K.
-            const long t256 = (long)((N + 255) / 256) * ((M + 255) / 256);
-            const long rounds = (t256 + 255) / 256;
-            if (t256 * 10 >= rounds * 256 * 8) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, 2, epi, st);
+        // Measured on MI355X.  Large M (the chip runs these kernels at a power-limited clock, so
+        // fewer instructions per flop is what counts): the 256-row tile halves the unpack work
+        // per flop and wins whenever its grid fills the 256 CUs evenly; otherwise 128-row tiles,
+        // pipelined variant for long K.  Smaller M: filling the CUs matters more than the tile's
+        // efficiency, so the tallest tile that still gives about 160 workgroups is taken
+        // (4096 x 4096 at M = 512: 46 us with 32-row tiles, 71 us with 128-row tiles).
+        const long ncol = (N + 255) / 256;
+        auto ntiles = [&](int rows) { return ncol * ((M + rows - 1) / rows); };
+        const long t256 = ntiles(256);
+        const long rounds = (t256 + 255) / 256;
+        if (M > 64 && t256 * 10 >= rounds * 256 * 8) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, 2, epi, st);
+        if (M > 64 && ntiles(128) >= 160) {
             if (K >= 8192) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, 1, epi, st);
+            mi = 4;
+        } else if (M > 32 && ntiles(64) >= 160) {
+            mi = 2;
+        } else {
+            mi = 1;
         }
-        mi = M > 64 ? 4 : (M > 32 ? 2 : 1);
     }
     switch (mi) {
         case 1: return launch_mi<1>(x, w, zs, y, M, N, K, gshift, epi, st);

@@ -570,3 +570,27 @@ def test_reference_grid_int32_layout(k, n):
             assert tuple(out.shape) == (bs, seq, n)
             assert torch.allclose(ref, out.float(), atol=2e-2, rtol=2e-2), (k, n, bs, seq)
     quant.clear_repack_cache()
+
+
+# ------------------------------------------------------------------ 33..512 tokens through the dispatcher
+@pytest.mark.parametrize("n,k,g", [(520, 1056, 32), (4096, 4096, 128), (16384, 4096, 128), (4096, 16384, 128)])
+@pytest.mark.parametrize("m", [33, 48, 64, 65, 100, 128, 129, 200, 512])
+def test_mid_size_batches_auto_dispatch(capi, n, k, g, m):
+    # with a workspace (token blocks through the split-K kernel where the GEMM grid would be tiny) ...
+    check_gemm_ws(capi, m, n, k, g, capi.SQ_ALGO_AUTO)
+    # ... and without one
+    check_gemm(capi, m, n, k, g, capi.SQ_ALGO_AUTO)
+
+
+def test_mid_size_batch_fused_epilogue_blocks(capi):
+    # bias / ReLU / residual reach every 32-token block of a blocked launch
+    m, n, k, g = 100, 4096, 16384, 128
+    d = linear(n, k, g, seed=51)
+    rng = np.random.default_rng(52)
+    x = orc.synth_x(m, k, seed=53)
+    bias = rng.normal(0, 2.0, size=n).astype(np.float16)
+    res = rng.normal(0, 2.0, size=(m, n)).astype(np.float16)
+    y = capi.gemm_fused(to_dev(x), d["w_dev"], d["zs_dev"], n, k, g, bias=to_dev(bias), residual=to_dev(res), act=1)
+    y_ref = fused_ref(x, d["w_hat"], bias, res, 1)
+    scale = np.max(np.abs(orc.gemm_ref(x, d["w_hat"])))
+    assert np.max(np.abs(y.float().cpu().numpy() - y_ref)) <= TOL * scale
