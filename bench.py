@@ -299,7 +299,19 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
             del wd
     tf = flops_total / time_total / 1e6
     tfd = flops_total / dense_time_total / 1e6
-    return {"m": m, "tflops": round(tf, 1), "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
+    # the other two token counts of the same configuration, aggregate only
+    other = {}
+    with torch.cuda.stream(stream):
+        for m2 in (512, 4096):
+            fl2, t2 = 0.0, 0.0
+            for (w, zs), (name, n, k) in list(zip(layer, shapes))[3:]:
+                x = torch.randn((m2, k), device=dev, generator=gen).half()
+                y = torch.empty((m2, n), dtype=torch.float16, device=dev)
+                t2 += timed(lambda: capi.gemm(x, w, zs, n, k, g, out=y, stream=stream))
+                fl2 += 2.0 * m2 * n * k
+            other["m%d" % m2] = {"tflops": round(fl2 / t2 / 1e6, 1),
+                                 "frac_of_fp16_mfma_peak": round(fl2 / t2 / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)}
+    return {"m": m, "other_token_counts": other, "tflops": round(tf, 1), "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
             "dense_fp16_library_tflops": round(tfd, 1), "vs_dense_fp16_library": round(tf / tfd, 3),
             "nominal_shader_mhz": 2400, "per_linear": res}
 

@@ -90,7 +90,7 @@ std::pair<at::Tensor, at::Tensor> l1_view_of_l2(const at::Tensor& W, const at::T
     return {w1, zs1};
 }
 
-// Workspace of the split-K kernel (5..128 tokens, in blocks of at most 32): one zero-initialised buffer per
+// Workspace of the split-K kernels (5..1024 tokens): one zero-initialised buffer per
 // (device, stream), grown on demand and kept for the life of the process.  Calls on one
 // stream are ordered, which is what sharing a workspace requires.  Under HIP graph capture
 // the buffer must already exist (run the call once on the capturing stream beforehand).
@@ -170,7 +170,7 @@ at::Tensor gemm_impl(const at::Tensor& I, const at::Tensor& W, const at::Tensor&
     void* ws_ptr = nullptr;
     size_t ws_bytes = 0;
     at::Tensor ws;
-    if (M > 4 && M <= 128 && ((algo & 0xFF) == SQ_ALGO_AUTO || (algo & 0xFF) == SQ_ALGO_SKINNY_WS)) {
+    if (M > 4 && M <= 1024 && ((algo & 0xFF) == SQ_ALGO_AUTO || (algo & 0xFF) == SQ_ALGO_SKINNY_WS)) {
         ws = workspace_for(I, stream, sq_w4a16_workspace_bytes((int)M, N, (int)K));
         ws_ptr = ws.data_ptr();
         ws_bytes = (size_t)ws.numel();

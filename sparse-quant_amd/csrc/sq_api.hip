@@ -96,7 +96,8 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
                 return SQ_ERR_WORKSPACE;
             return launch_code(sq::launch_skinny2_tuned(x, w, zs, y, workspace, M, N, K, group_size, tune, epi, st));
         case SQ_ALGO_GEMM:
-            return launch_code(sq::launch_gemm_tuned(x, w, zs, y, M, N, K, group_size, tune, epi, st));
+            return launch_code(sq::launch_gemm_tuned(x, w, zs, y, aligned16(workspace) ? workspace : nullptr,
+                                                     workspace_bytes, M, N, K, group_size, tune, epi, st));
         default:
             return SQ_ERR_BAD_ALGO;
     }
@@ -131,7 +132,9 @@ int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y, int 
 
 size_t sq_w4a16_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
-    return sq::skinny2_workspace_bytes(M > 32 ? 32 : M, N, K);
+    const size_t a = sq::skinny2_workspace_bytes(M > 32 ? 32 : M, N, K);
+    const size_t b = M > 32 ? sq::gemm_workspace_bytes(M, N, K) : 0;
+    return a > b ? a : b;
 }
 
 int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,

@@ -125,4 +125,29 @@ __device__ __forceinline__ half_t epilogue(float v, int m, int n, int N, const E
     return (half_t)v;
 }
 
+// 128-bit global accesses at the device-coherent level (cache policy sc1, what agent-scope
+// relaxed atomics use), for data exchanged between workgroups inside one kernel.  The eight
+// loads and the wait for them are one asm statement, so the compiler never sees a register
+// whose data is still in flight.
+__device__ __forceinline__ void store_coherent_x4(float* p, float4_t v) {
+    // The trailing s_nop covers the hazard between a wide store and a later overwrite of its
+    // data registers, which the compiler cannot see through inline asm.
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 3" : : "v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void load8_coherent_x4(const float* const (&p)[8], float4_t (&v)[8]) {
+    asm volatile(
+        "global_load_dwordx4 %0, %8, off sc1\n\t"
+        "global_load_dwordx4 %1, %9, off sc1\n\t"
+        "global_load_dwordx4 %2, %10, off sc1\n\t"
+        "global_load_dwordx4 %3, %11, off sc1\n\t"
+        "global_load_dwordx4 %4, %12, off sc1\n\t"
+        "global_load_dwordx4 %5, %13, off sc1\n\t"
+        "global_load_dwordx4 %6, %14, off sc1\n\t"
+        "global_load_dwordx4 %7, %15, off sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7])
+        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
+        : "memory");
+}
+
 }  // namespace sq

@@ -38,7 +38,8 @@ __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1
 template <int MI>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_kernel(const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS,
                                                    const half_t* __restrict__ X, half_t* __restrict__ Y, int M,
-                                                   int N, int K, int gshift, Epilogue epi) {
+                                                   int N, int K, int gshift, Epilogue epi, float* part,
+                                                   unsigned* counters) {
     constexpr int BM = 32 * MI;
     // Activation tile, two stages, row pitch 128 B (64 halves, no padding); the eight
     // 16-byte chunks of row R are stored at chunk position c ^ swz(R); 8 consecutive
@@ -56,6 +57,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     const int n0 = blockIdx.x * GEMM_BN + 64 * wave;
     const int groups = K >> gshift;
     const int nit = (K + GEMM_BK - 1) / GEMM_BK;
+    // K split over gridDim.z workgroups (1 = no split): this one runs steps it0 .. it1-1.
+    const int ksplit = gridDim.z;
+    const int spz = (nit + ksplit - 1) / ksplit;
+    const int it0 = blockIdx.z * spz;
+    const int it1 = imin(it0 + spz, nit);
 
     // Global -> registers -> LDS staging of the activation tile.  Pass p of wave w moves
     // rows 32*p + 8*w .. +7; lane l = 8*r + c' fetches the chunk that belongs at
@@ -138,7 +144,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         load_w(it + GEMM_STAGES - 1, w[cf]);
         __builtin_amdgcn_sched_barrier(0);
         half8_t bf[2][4];
-        const bool kin = it * GEMM_BK + 32 * lc < K;  // false only past K: scale 0 -> W_hat 0
+        const bool kin = it < it1 && it * GEMM_BK + 32 * lc < K;  // false past the range: scale 0 -> W_hat 0
 #pragma unroll
         for (int ni = 0; ni < 2; ni++) {
             const half_t sv = kin ? w[c].zs[ni].y : (half_t)0.f;
@@ -165,8 +171,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 
 #pragma unroll
     for (int s0 = 0; s0 < GEMM_STAGES - 1; s0++) {
-        load_x(s0, xr[s0]);
-        load_w(s0, w[s0]);
+        load_x(it0 + s0, xr[s0]);
+        load_w(it0 + s0, w[s0]);
     }
     store_x(0, xr[0]);
     __syncthreads();
@@ -174,8 +180,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     // with steps whose scale is 0 everywhere and whose loads are clamped.
     constexpr int TRIP = 2 * GEMM_STAGES;
     static_assert(GEMM_STAGES == 3, "the trip below is written for three register stages");
-    const int nitp = (nit + TRIP - 1) / TRIP * TRIP;
-    for (int it = 0; it < nitp; it += TRIP) {
+    const int nitp = (it1 - it0 + TRIP - 1) / TRIP * TRIP;
+    for (int it = it0; it < it0 + nitp; it += TRIP) {
         // LDS buffer = step parity, register stage = step % GEMM_STAGES: unroll over
         // their common period.
         step(it, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
@@ -184,6 +190,56 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         step(it + 3, std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
         step(it + 4, std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
         step(it + 5, std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
+    }
+
+    if (ksplit > 1) {
+        // Partial tiles meet in the workspace: 128-bit stores at the device-coherent cache level,
+        // one counter per output tile; the workgroup that arrives last adds the partials in a
+        // fixed order (bit-reproducible), stores the tile and resets the counter.
+        __shared__ unsigned last_flag;
+        constexpr int SLOTS = MI * 2 * 4;  // float4 per thread
+        const long tile = (long)blockIdx.y * gridDim.x + blockIdx.x;
+        const long ntile = (long)gridDim.x * gridDim.y;
+        float* mine = part + ((long)blockIdx.z * ntile + tile) * (SLOTS * 256 * 4);
+#pragma unroll
+        for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float4_t v4 = {acc[mi][ni][4 * q], acc[mi][ni][4 * q + 1], acc[mi][ni][4 * q + 2],
+                                         acc[mi][ni][4 * q + 3]};
+                    store_coherent_x4(mine + (((mi * 2 + ni) * 4 + q) * 256 + tid) * 4, v4);
+                }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned old = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_flag = (old == (unsigned)(ksplit - 1)) ? 1u : 0u;
+        }
+        __syncthreads();
+        if (!last_flag) return;
+#pragma unroll
+        for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float* src[8];
+#pragma unroll
+                    for (int z = 0; z < 8; z++)
+                        src[z] = part + ((long)(z < ksplit ? z : 0) * ntile + tile) * (SLOTS * 256 * 4) +
+                                 (((mi * 2 + ni) * 4 + q) * 256 + tid) * 4;
+                    float4_t pv[8];
+                    load8_coherent_x4(src, pv);
+                    float4_t sum = pv[0];
+#pragma unroll
+                    for (int z = 1; z < 8; z++)
+                        if (z < ksplit) sum += pv[z];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[mi][ni][4 * q + e] = sum[e];
+                }
+        if (tid == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // Epilogue: fp32 -> fp16, 32 consecutive columns per half-wave.
@@ -200,50 +256,95 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         }
 }
 
+constexpr int GEMM_COUNTER_BYTES = 65536;  // start of the workspace: one uint32 per output tile
+
 template <int MI>
 static hipError_t launch_mi(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int gshift,
-                            Epilogue epi, hipStream_t st) {
-    const dim3 grid((N + GEMM_BN - 1) / GEMM_BN, (M + 32 * MI - 1) / (32 * MI));
+                            Epilogue epi, void* ws, int ksplit, hipStream_t st) {
+    const dim3 grid((N + GEMM_BN - 1) / GEMM_BN, (M + 32 * MI - 1) / (32 * MI), ksplit);
+    unsigned* counters = (unsigned*)ws;
+    float* part = ws ? (float*)((char*)ws + GEMM_COUNTER_BYTES) : nullptr;
     hipLaunchKernelGGL((gemm_kernel<MI>), grid, dim3(256), 0, st, (const uint8_t*)w, (const half2_t*)zs,
-                       (const half_t*)x, (half_t*)y, M, N, K, gshift, epi);
+                       (const half_t*)x, (half_t*)y, M, N, K, gshift, epi, part, counters);
     return hipGetLastError();
 }
 
-// tune = 0 for the heuristic, else the number of 32-row tiles per workgroup (1, 2 or 4), or 8 / 9 / 10 for
-// the software-pipelined kernel (128 rows at two waves per SIMD, 128 rows at one, 256 rows at one).
-hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                             int tune, Epilogue epi, hipStream_t st) {
+// Tile height and K split for a shape (shared by the launcher and the workspace query): the
+// tallest tile that still gives about 160 workgroups, and when even 32-row tiles give fewer
+// than 128 a split of K that brings the grid to about 256 workgroups (each range at least 16
+// steps of 64 long).  `pipe` receives the pipelined variant to use instead (-1 = none).
+struct GemmPlan {
+    int mi, ksplit, pipe;
+};
+static GemmPlan plan_gemm(int M, int N, int K, bool have_ws) {
+    GemmPlan p = {1, 1, -1};
+    const long ncol = (N + 255) / 256;
+    auto ntiles = [&](int rows) { return ncol * ((M + rows - 1) / rows); };
+    const long t256 = ntiles(256);
+    const long rounds = (t256 + 255) / 256;
+    if (M > 64 && t256 * 10 >= rounds * 256 * 8) {
+        p.pipe = 2;
+    } else if (M > 64 && ntiles(128) >= 160) {
+        if (K >= 8192) p.pipe = 1;
+        p.mi = 4;
+    } else if (M > 32 && ntiles(64) >= 160) {
+        p.mi = 2;
+    } else {
+        p.mi = 1;
+        if (have_ws && M > 32) {
+            // few tiles: taller tiles and a K split instead (the partial tiles cost 4 bytes per
+            // output element and split, so the split stays at the minimum that fills the chip)
+            const int nit = (K + GEMM_BK - 1) / GEMM_BK;
+            for (int mi = 4; mi >= 1; mi >>= 1) {
+                const long t = ntiles(32 * mi);
+                if (t > 16384) continue;
+                int ks = 1;
+                while (ks < 8 && t * ks * 2 <= 256 && nit / (ks * 2) >= 16) ks *= 2;
+                if (t * ks >= 128 || mi == 1) {
+                    p.mi = mi;
+                    p.ksplit = ks;
+                    break;
+                }
+            }
+        }
+    }
+    return p;
+}
+
+size_t gemm_workspace_bytes(int M, int N, int K) {
+    const GemmPlan p = plan_gemm(M, N, K, true);
+    if (p.ksplit == 1) return 0;
+    const long tiles = (long)((N + 255) / 256) * ((M + 32 * p.mi - 1) / (32 * p.mi));
+    return (size_t)GEMM_COUNTER_BYTES + (size_t)p.ksplit * tiles * (32 * p.mi) * 256 * sizeof(float);
+}
+
+// tune = 0 for the heuristic, else the number of 32-row tiles per workgroup (1, 2 or 4) | ksplit << 8
+// (needs ws), or 8 / 9 / 10 for the software-pipelined kernel (128 rows at two waves per SIMD, 128 rows
+// at one, 256 rows at one).  ws = null or too small: K is never split.
+hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, size_t ws_bytes, int M,
+                             int N, int K, int g, int tune, Epilogue epi, hipStream_t st) {
     int gshift = 0;
     while ((1 << gshift) < g) gshift++;
     int mi = tune & 0xFF;
+    int ksplit = (tune >> 8) & 0xFF;
     if (mi >= 8 && mi <= 10) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, mi - 8, epi, st);
     if (mi != 1 && mi != 2 && mi != 4) {
-        // Measured on MI355X.  Large M (the chip runs these kernels at a power-limited clock, so
-        // fewer instructions per flop is what counts): the 256-row tile halves the unpack work
-        // per flop and wins whenever its grid fills the 256 CUs evenly; otherwise 128-row tiles,
-        // pipelined variant for long K.  Smaller M: filling the CUs matters more than the tile's
-        // efficiency, so the tallest tile that still gives about 160 workgroups is taken
-        // (4096 x 4096 at M = 512: 46 us with 32-row tiles, 71 us with 128-row tiles).
-        const long ncol = (N + 255) / 256;
-        auto ntiles = [&](int rows) { return ncol * ((M + rows - 1) / rows); };
-        const long t256 = ntiles(256);
-        const long rounds = (t256 + 255) / 256;
-        if (M > 64 && t256 * 10 >= rounds * 256 * 8) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, 2, epi, st);
-        if (M > 64 && ntiles(128) >= 160) {
-            if (K >= 8192) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, 1, epi, st);
-            mi = 4;
-        } else if (M > 32 && ntiles(64) >= 160) {
-            mi = 2;
-        } else {
-            mi = 1;
-        }
+        const bool have_ws = ws != nullptr && ws_bytes >= gemm_workspace_bytes(M, N, K);
+        const GemmPlan p = plan_gemm(M, N, K, have_ws);
+        if (p.pipe >= 0) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, p.pipe, epi, st);
+        mi = p.mi;
+        ksplit = p.ksplit;
+    } else {
+        if (ksplit != 2 && ksplit != 4 && ksplit != 8) ksplit = 1;
+        const long tiles = (long)((N + 255) / 256) * ((M + 32 * mi - 1) / (32 * mi));
+        const size_t need = (size_t)GEMM_COUNTER_BYTES + (size_t)ksplit * tiles * (32 * mi) * 256 * sizeof(float);
+        if (ksplit > 1 && (!ws || ws_bytes < need || tiles > 16384)) ksplit = 1;
     }
     switch (mi) {
-        case 1: return launch_mi<1>(x, w, zs, y, M, N, K, gshift, epi, st);
-        case 2: return launch_mi<2>(x, w, zs, y, M, N, K, gshift, epi, st);
-        default: return launch_mi<4>(x, w, zs, y, M, N, K, gshift, epi, st);
+        case 1: return launch_mi<1>(x, w, zs, y, M, N, K, gshift, epi, ws, ksplit, st);
+        case 2: return launch_mi<2>(x, w, zs, y, M, N, K, gshift, epi, ws, ksplit, st);
+        default: return launch_mi<4>(x, w, zs, y, M, N, K, gshift, epi, ws, ksplit, st);
     }
 }
-
 
 }  // namespace sq

@@ -38,9 +38,10 @@ hipError_t launch_skinny_tuned(const void* x, const void* w, const void* zs, voi
 size_t skinny2_workspace_bytes(int M, int N, int K);
 hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                                 int g, int tune, Epilogue epi, hipStream_t st);
-// sq_gemm.hip: any M.  tune = 32-row tiles per workgroup (1,2,4).
-hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                             int tune, Epilogue epi, hipStream_t st);
+// sq_gemm.hip: any M.  tune = 32-row tiles per workgroup (1,2,4) | ksplit << 8; ws may be null.
+size_t gemm_workspace_bytes(int M, int N, int K);
+hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, size_t ws_bytes, int M,
+                             int N, int K, int g, int tune, Epilogue epi, hipStream_t st);
 
 // sq_gemm2.hip: software-pipelined 128 x 256 tile variant for M > 64.
 hipError_t launch_gemm_pipe(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,

@@ -129,7 +129,7 @@ def gemm_fused(x, w, zs, n, k, group_size, bias=None, residual=None, act=SQ_ACT_
     m = x.numel() // k
     if out is None:
         out = torch.empty((m, n), dtype=torch.float16, device=x.device)
-    if ws is None and use_workspace and 4 < m <= 128:
+    if ws is None and use_workspace and 4 < m <= 1024:
         ws = workspace(m, n, k, x.device, stream)
     _check(lib().sq_w4a16_gemm_fused(_ptr(x), _ptr(w), _ptr(zs), _ptr(bias), _ptr(residual), _ptr(out), m, n, k,
                                      group_size, SQ_LAYOUT_L1, act, algo, _ptr(ws), 0 if ws is None else ws.numel(),

@@ -594,3 +594,20 @@ def test_mid_size_batch_fused_epilogue_blocks(capi):
     y_ref = fused_ref(x, d["w_hat"], bias, res, 1)
     scale = np.max(np.abs(orc.gemm_ref(x, d["w_hat"])))
     assert np.max(np.abs(y.float().cpu().numpy() - y_ref)) <= TOL * scale
+
+
+@pytest.mark.parametrize("mi", [1, 2, 4])
+@pytest.mark.parametrize("ksplit", [2, 4, 8])
+def test_gemm_split_k_every_tile_height(capi, mi, ksplit):
+    # K split over workgroups in the tiled GEMM (partial tiles through the workspace), incl. ragged N, M and
+    # K ranges that do not divide evenly; bit-reproducible across calls on one workspace
+    for (m, n, k, g) in [(70, 264, 2112, 64), (200, 520, 4096, 128), (129, 4096, 4096, 128)]:
+        algo = capi.SQ_ALGO_GEMM | ((mi | (ksplit << 8)) << 8)
+        d = linear(n, k, g, seed=61)
+        x = to_dev(orc.synth_x(m, k, seed=62))
+        ws = torch.zeros(64 * 1024 * 1024, dtype=torch.uint8, device=DEV)
+        y1 = capi.gemm_ws(x, d["w_dev"], d["zs_dev"], n, k, g, algo=algo, ws=ws)
+        y_ref = orc.gemm_ref(x.cpu().numpy(), d["w_hat"])
+        assert np.max(np.abs(y1.float().cpu().numpy() - y_ref)) <= TOL * np.max(np.abs(y_ref))
+        assert torch.count_nonzero(ws[:65536]).item() == 0
+        assert torch.equal(y1, capi.gemm_ws(x, d["w_dev"], d["zs_dev"], n, k, g, algo=algo, ws=ws))
