@@ -291,7 +291,9 @@ static GemmPlan plan_gemm(int M, int N, int K, bool have_ws) {
         p.mi = 2;
     } else {
         p.mi = 1;
-        if (have_ws && M > 32) {
+        // (measured: with K = 4096 the exchange only pays off below about 64 tiles; with
+        // K >= 8192 it pays off up to a full grid of 32-row tiles)
+        if (have_ws && M > 32 && (ntiles(32) <= 64 || (K >= 8192 && ntiles(32) <= 256))) {
             // few tiles: taller tiles and a K split instead (the partial tiles cost 4 bytes per
             // output element and split, so the split stays at the minimum that fills the chip)
             const int nit = (K + GEMM_BK - 1) / GEMM_BK;
