@@ -72,22 +72,26 @@ int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y,
                      int M, int N, int K, int group_size, int layout, int algo,
                      void* stream);
 
-/* Same product with a caller-owned device workspace, which lets the 5 <= M <= 32
- * range split K over workgroups (fp32 partial tiles, summed in a fixed order by the
- * workgroup that finishes last, so results are bit-reproducible).  No counterpart
- * in the reference.  The workspace must hold at least
- * sq_w4a16_workspace_bytes(M, N, K) bytes, be 16-byte aligned, and have its first
- * 64 KiB zeroed before the first call (every call leaves them zero); calls that
- * share a workspace must not overlap in time.  With SQ_ALGO_AUTO the split-K kernel
- * is taken where it is the fastest (5..32 tokens on weights of 2^25 elements or more
- * or with K > 8192, 17..32 tokens on any weight; 33..64 tokens on such weights and up to
- * 128 tokens with K > 8192 run as blocks of 32 tokens); everywhere else, and with an explicit other
- * algo, the call behaves like sq_w4a16_gemm_ex and ignores the workspace. */
+/* Same product with a caller-owned device workspace, which lets the kernels split K
+ * over workgroups where a single pass cannot fill the chip (fp32 partial tiles, summed
+ * in a fixed order by the workgroup that finishes last, so results are
+ * bit-reproducible).  No counterpart in the reference.  The workspace must hold at
+ * least sq_w4a16_workspace_bytes(M, N, K) bytes, be 16-byte aligned, and have its
+ * first 64 KiB zeroed before the first call (every call leaves them zero); calls that
+ * share a workspace must not overlap in time.  With SQ_ALGO_AUTO the split is taken
+ * where it is the fastest: the split-K decode kernel for 5..32 tokens on weights of
+ * 2^25 elements or more or with K > 8192 and for 17..32 tokens on any weight, the same
+ * kernel in blocks of 32 tokens for 33..64 tokens on such weights and up to 128 tokens
+ * with K > 8192, and a K split of the tiled GEMM for larger M whose grid would leave
+ * most CUs idle.  A workspace that is NULL, misaligned or too small is ignored under
+ * SQ_ALGO_AUTO (the workspace-free kernels run); an explicit SQ_ALGO_SKINNY_WS then
+ * returns SQ_ERR_WORKSPACE. */
 int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y,
                      int M, int N, int K, int group_size, int layout, int algo,
                      void* workspace, size_t workspace_bytes, void* stream);
 
-/* Bytes sq_w4a16_gemm_ws needs for this shape (grows with N; M is capped at 32). */
+/* Bytes sq_w4a16_gemm_ws / sq_w4a16_gemm_fused can use for this shape (8.06 MiB for
+ * every decode batch with N <= 16384; up to tens of MiB for the GEMM split). */
 size_t sq_w4a16_workspace_bytes(int M, int N, int K);
 
 /* The same product with the element-wise tail of the linear folded into the kernel's
