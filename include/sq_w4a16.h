@@ -81,9 +81,8 @@ int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y,
  * share a workspace must not overlap in time.  With SQ_ALGO_AUTO the split is taken
  * where it is the fastest: the split-K decode kernel for 5..32 tokens on weights of
  * 2^25 elements or more or with K > 8192 and for 17..32 tokens on any weight, the same
- * kernel in blocks of 32 tokens for 33..64 tokens on such weights and up to 128 tokens
- * with K > 8192, and a K split of the tiled GEMM for larger M whose grid would leave
- * most CUs idle.  A workspace that is NULL, misaligned or too small is ignored under
+ * kernel in two blocks for 33..48 tokens on such weights, and a K split of the tiled
+ * GEMM for larger M whose grid would leave most CUs idle.  A workspace that is NULL, misaligned or too small is ignored under
  * SQ_ALGO_AUTO (the workspace-free kernels run); an explicit SQ_ALGO_SKINNY_WS then
  * returns SQ_ERR_WORKSPACE. */
 int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y,

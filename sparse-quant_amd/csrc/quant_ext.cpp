@@ -96,6 +96,7 @@ std::pair<at::Tensor, at::Tensor> l1_view_of_l2(const at::Tensor& W, const at::T
 // the buffer must already exist (run the call once on the capturing stream beforehand).
 std::mutex g_ws_mutex;
 std::map<std::pair<int, void*>, at::Tensor> g_workspaces;
+std::vector<at::Tensor> g_retired;
 
 at::Tensor workspace_for(const at::Tensor& like, void* stream, size_t bytes) {
     std::lock_guard<std::mutex> lock(g_ws_mutex);
@@ -104,6 +105,8 @@ at::Tensor workspace_for(const at::Tensor& like, void* stream, size_t bytes) {
     if (it != g_workspaces.end() && (size_t)it->second.numel() >= bytes) return it->second;
     const int64_t want = (int64_t)std::max<size_t>(bytes, (size_t)1 << 20);
     at::Tensor ws = torch::zeros({want}, like.options().dtype(at::kByte));
+    // A captured HIP graph may still hold the address of the smaller buffer: keep it alive.
+    if (it != g_workspaces.end()) g_retired.push_back(it->second);
     g_workspaces[key] = ws;
     return ws;
 }

@@ -53,12 +53,14 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
         const bool ws_ok = workspace && aligned16(workspace) &&
                            workspace_bytes >= sq::skinny2_workspace_bytes(M > 32 ? 32 : M, N, K) &&
                            (N + 63) / 64 <= 16384;
+        const bool gemm_ws = workspace && aligned16(workspace) && M > 32 &&
+                             workspace_bytes >= sq::gemm_workspace_bytes(M, N, K);
         if (ws_ok && M > 4 && M <= 32 && (large || M > 16 || K > 8192)) {
             kernel = SQ_ALGO_SKINNY_WS;
-        } else if (ws_ok && M > 32 && ((M <= 64 && large) || (M <= 128 && K > 8192))) {
-            // 33..128 tokens on a large weight: the tiled GEMM would run on a handful of
-            // workgroups (its grid is N/256 x M/32..128); blocks of 32 tokens through the split-K
-            // kernel are 2-4 times faster there (fc2 at M = 64: 43 us against 170 us).
+        } else if (ws_ok && M > 32 && M <= 48 && (large || K > 8192)) {
+            // 33..48 tokens on a large weight: two blocks through the split-K decode kernel are
+            // still a little faster than the tiled GEMM with K split (fc1: 30 us against 31 us,
+            // fc2: 35 us against 37 us); beyond that the GEMM takes over.
             for (int m0 = 0; m0 < M; m0 += 32) {
                 const int mb = M - m0 < 32 ? M - m0 : 32;
                 sq::Epilogue e = epi;
@@ -71,7 +73,10 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
             return SQ_OK;
         } else if (M <= 4 || (M <= 8 && K <= 8192)) {
             kernel = SQ_ALGO_GEMV_FIXUP;
-        } else if (M <= 32 || (M <= 64 && (!large || K > 8192))) {
+        } else if (M <= 32 || (M <= 64 && ((!large && K <= 8192) || (!gemm_ws && K > 8192)))) {
+            // 33..64 tokens: the 16-column kernel on small weights (4096 x 4096: 21 us against
+            // 19 us for the GEMM with K split, 46 us without), and on long K when no workspace
+            // allows the GEMM to split K (4096 x 16384: 70 us against 170 us unsplit).
             kernel = SQ_ALGO_SKINNY;
         } else {
             kernel = SQ_ALGO_GEMM;

@@ -269,10 +269,12 @@ static hipError_t launch_mi(const void* x, const void* w, const void* zs, void* 
     return hipGetLastError();
 }
 
-// Tile height and K split for a shape (shared by the launcher and the workspace query): the
-// tallest tile that still gives about 160 workgroups, and when even 32-row tiles give fewer
-// than 128 a split of K that brings the grid to about 256 workgroups (each range at least 16
-// steps of 64 long).  `pipe` receives the pipelined variant to use instead (-1 = none).
+// Tile height and K split for a shape (shared by the launcher and the workspace query).
+// Measured on MI355X: large M wants the tallest tile whose grid fills the 256 CUs (fewer
+// unpack instructions per flop); when even 64-row tiles give fewer than 256 workgroups and a
+// workspace is at hand, 64-row tiles (32-row when those are too few) with K split so that
+// the grid reaches about 256 workgroups (4096 x 16384 at M = 128: 47 us against 163 us
+// unsplit).  `pipe` receives the pipelined variant to use instead (-1 = none).
 struct GemmPlan {
     int mi, ksplit, pipe;
 };
@@ -282,33 +284,25 @@ static GemmPlan plan_gemm(int M, int N, int K, bool have_ws) {
     auto ntiles = [&](int rows) { return ncol * ((M + rows - 1) / rows); };
     const long t256 = ntiles(256);
     const long rounds = (t256 + 255) / 256;
-    if (M > 64 && t256 * 10 >= rounds * 256 * 8) {
-        p.pipe = 2;
+    const int nit = (K + GEMM_BK - 1) / GEMM_BK;
+    if (M > 64 && t256 * 10 >= rounds * 256 * 6) {
+        p.pipe = 2;  // 256 x 256 tiles pay from about 60 % of the CUs (5120 x 13696 at M = 2048: 338 us against 390 us)
     } else if (M > 64 && ntiles(128) >= 160) {
         if (K >= 8192) p.pipe = 1;
         p.mi = 4;
+    } else if (have_ws && M > 32 && ntiles(64) < 256 && ntiles(32) <= 16384) {
+        p.mi = (ntiles(64) * 8 < 256 || (ntiles(64) * 8 == 256 && K <= 8192)) ? 1 : 2;
+        const long t = ntiles(32 * p.mi);
+        while (p.ksplit < 8 && t * p.ksplit * 2 <= 256 && nit / (p.ksplit * 2) >= 8) p.ksplit *= 2;
+        if (p.ksplit == 1 && K >= 12288 && ntiles(128) * 4 <= 512) p = {4, 4, -1};
+    } else if (have_ws && M > 64 && K >= 12288 && ntiles(128) * 4 <= 512) {
+        // Long K with a grid between one and two rounds of 64-row tiles: 128-row tiles with K
+        // split four ways even out the rounds (4096 x 16384 at M = 1024: 185 us against 207 us).
+        p = {4, 4, -1};
     } else if (M > 32 && ntiles(64) >= 160) {
         p.mi = 2;
     } else {
         p.mi = 1;
-        // (measured: with K = 4096 the exchange only pays off below about 64 tiles; with
-        // K >= 8192 it pays off up to a full grid of 32-row tiles)
-        if (have_ws && M > 32 && (ntiles(32) <= 64 || (K >= 8192 && ntiles(32) <= 256))) {
-            // few tiles: taller tiles and a K split instead (the partial tiles cost 4 bytes per
-            // output element and split, so the split stays at the minimum that fills the chip)
-            const int nit = (K + GEMM_BK - 1) / GEMM_BK;
-            for (int mi = 4; mi >= 1; mi >>= 1) {
-                const long t = ntiles(32 * mi);
-                if (t > 16384) continue;
-                int ks = 1;
-                while (ks < 8 && t * ks * 2 <= 256 && nit / (ks * 2) >= 16) ks *= 2;
-                if (t * ks >= 128 || mi == 1) {
-                    p.mi = mi;
-                    p.ksplit = ks;
-                    break;
-                }
-            }
-        }
     }
     return p;
 }
