@@ -161,6 +161,33 @@ int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out,
                          int lut_elem_bytes, int Z, int H, int S, int D, int nnz, float sm_scale, int causal,
                          void* stream);
 
+/* Dense decode attention, one query token per sequence (q_len == 1 < kv_len):
+ *   out[b,h,:] = sum_j P[j] v[b,h,j,:],  P = fp16(softmax_j(q[b,h,:] . k[b,h,j,:] * sm_scale + mask[b,j]))
+ * over the first L rows of an fp16 key/value cache, softmax in fp32, probabilities rounded
+ * to fp16 before they meet v, fp32 accumulation.  Replaces the decode branch of
+ * sparse_attention (reference: sparse-attention/nvidia/playground/kernels/
+ * block_sparse_attention_lut.py:272-300), which runs two torch.matmul and a softmax.
+ *   q          fp16, element (b,h,d) at q[b*q_bstride + h*q_hstride + d]
+ *   k_cache, v_cache  fp16, row j of (b,h) at cache[b*cache_bstride + h*cache_hstride + j*D],
+ *              room for Lmax rows per (b,h) (cache_hstride >= Lmax*D)
+ *   k_new, v_new  both NULL, or the step's new key/value rows, element (b,h,d) at
+ *              new[b*new_bstride + h*new_hstride + d]: they are stored to cache row
+ *              cache_len and take part in the attention (L = cache_len + 1); without them
+ *              L = cache_len.  (Extension over the reference, which appends with torch.cat
+ *              before the call; it saves two copy launches per layer.)
+ *   mask       NULL or fp16 additive mask, element (b,j) at mask[b*mask_bstride + j], j < L
+ *              (the reference's attention_mask [bsz,1,1,kv_len])
+ *   out        fp16 [B, H, D] contiguous (= [B, 1, H*D], the layout the output projection reads)
+ *   cache_len  rows already valid; cache_len_dev, if not NULL, points to that number on the
+ *              device (int64) and overrides cache_len -- read by the kernel, so a captured HIP
+ *              graph follows a growing cache; the kernel clamps it to the cache size.
+ * D in {64, 128}; all strides in elements and multiples of 8; pointers 16-byte aligned; Lmax up to
+ * about 38000 rows (scores are held in LDS).  A fully masked row gives NaN, as in the reference. */
+int sq_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                        const void* mask, void* out, int B, int H, int D, int Lmax, long q_bstride, long q_hstride,
+                        long new_bstride, long new_hstride, long cache_bstride, long cache_hstride, long mask_bstride,
+                        int cache_len, const long long* cache_len_dev, float sm_scale, void* stream);
+
 /* Diagnostic, no counterpart in the reference: a single wave spins for `spins`
  * (1 .. 2^26) dependent multiply-adds and writes three uint64 to out: shader-clock
  * ticks elapsed, ticks of the constant 100 MHz counter elapsed, and a dummy.  Run on

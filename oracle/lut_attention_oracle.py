@@ -13,6 +13,11 @@ Pinning (tests/test_attention_oracle.py): hand-written LUT known answer; a two-k
 softmax with weights known in closed form; single-visible-key rows return that V
 row exactly; constant V returns the constant; an all-blocks LUT equals unmasked
 softmax attention computed with a different formulation (per-row loops).
+decode_attention_ref restates the decode branch of the same entry point (:272-300): dense
+attention of one query row over the whole cache, softmax in fp32, probabilities cast to fp16
+before the product with v.  Pinning: equal keys give the mean of v; a dominating key returns
+its v row; -inf mask entries equal attention over the remaining rows; a per-element Python
+loop formulation on a small case; the two-key closed form.
 No function here is "parity unpinned".
 """
 import numpy as np
@@ -91,3 +96,21 @@ def attention_ref(q, k, v, lut, sm_scale, causal):
         p /= p.sum(axis=-1, keepdims=True)
         out[b] = np.einsum("hmn,hnd->hmd", p, v[b])
     return out
+
+
+def decode_attention_ref(q, k, v, sm_scale, mask=None):
+    """q float [B,H,D]; k, v float [B,H,L,D]; mask None or additive float [B,L] -> float64 [B,H,D].
+
+    Follows block_sparse_attention_lut.py:279-298: weights = q k^T * sm_scale (+ mask), softmax,
+    cast of the probabilities to fp16, product with v."""
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    w = np.einsum("bhd,bhld->bhl", q, k) * sm_scale
+    if mask is not None:
+        w = w + np.asarray(mask, dtype=np.float64)[:, None, :]
+    w = w - w.max(axis=-1, keepdims=True)
+    p = np.exp(w)
+    p /= p.sum(axis=-1, keepdims=True)
+    p = p.astype(np.float16).astype(np.float64)
+    return np.einsum("bhl,bhld->bhd", p, v)

@@ -226,6 +226,33 @@ int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out,
                                                 static_cast<hipStream_t>(stream)));
 }
 
+int sq_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                        const void* mask, void* out, int B, int H, int D, int Lmax, long q_bstride, long q_hstride,
+                        long new_bstride, long new_hstride, long cache_bstride, long cache_hstride, long mask_bstride,
+                        int cache_len, const long long* cache_len_dev, float sm_scale, void* stream) {
+    if (B <= 0 || H <= 0 || Lmax <= 0 || (D != 64 && D != 128)) return SQ_ERR_BAD_SHAPE;
+    if ((long)B * H > (1L << 24)) return SQ_ERR_BAD_SHAPE;
+    if (sq::decode_attention_lds_bytes(Lmax, D) > sq::DECODE_ATTN_MAX_LDS) return SQ_ERR_BAD_SHAPE;
+    if (!q || !k_cache || !v_cache || !out) return SQ_ERR_NULL_POINTER;
+    if ((k_new == nullptr) != (v_new == nullptr)) return SQ_ERR_NULL_POINTER;
+    const bool append = k_new != nullptr;
+    if (!cache_len_dev) {  // a length on the device is clamped to the cache by the kernel
+        if (cache_len < 0 || cache_len + (append ? 1 : 0) > Lmax || cache_len + (append ? 1 : 0) < 1)
+            return SQ_ERR_BAD_SHAPE;
+    }
+    if (!aligned16(q) || !aligned16(k_cache) || !aligned16(v_cache) || (append && (!aligned16(k_new) || !aligned16(v_new))))
+        return SQ_ERR_MISALIGNED;
+    if ((q_bstride | q_hstride | cache_bstride | cache_hstride) % 8 != 0) return SQ_ERR_MISALIGNED;
+    if (append && (new_bstride | new_hstride) % 8 != 0) return SQ_ERR_MISALIGNED;
+    if (q_bstride < 0 || q_hstride < 0 || cache_bstride < 0 || cache_hstride < (long)Lmax * D || mask_bstride < 0 ||
+        (append && (new_bstride < 0 || new_hstride < 0)))
+        return SQ_ERR_BAD_SHAPE;
+    return launch_code(sq::launch_decode_attention(q, k_new, v_new, k_cache, v_cache, mask, out, B, H, D, Lmax,
+                                                   q_bstride, q_hstride, new_bstride, new_hstride, cache_bstride,
+                                                   cache_hstride, mask_bstride, cache_len, cache_len_dev, sm_scale,
+                                                   static_cast<hipStream_t>(stream)));
+}
+
 int sq_clock_probe(void* out, int spins, void* stream) {
     if (!out) return SQ_ERR_NULL_POINTER;
     if (spins <= 0 || spins > (1 << 26)) return SQ_ERR_BAD_SHAPE;

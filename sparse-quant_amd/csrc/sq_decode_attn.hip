@@ -1,0 +1,244 @@
+// Dense decode attention: one query token per sequence against an fp16 key/value cache,
+// optionally appending the step's new key/value row to the cache in the same launch.
+//
+// out[b,h,:] = sum_j P[j] * V[b,h,j,:],  P = fp16(softmax_j(q[b,h,:] . K[b,h,j,:] * sm_scale + mask[b,j]))
+// over the rows j < L of the cache, softmax in fp32, P rounded to fp16 before it meets V,
+// fp32 accumulation, fp16 output -- the decode branch of the reference's sparse_attention
+// (reference: sparse-attention/nvidia/playground/kernels/block_sparse_attention_lut.py:272-300).
+//
+// The work is a pure stream over the cache (2 * L * D * 2 bytes per head, two flops per
+// byte), so the kernel is laid out for the memory system and nothing else:
+//   * one workgroup of eight waves per (batch, head); a wave's 128-bit load covers 64/(D/8)
+//     consecutive cache rows = 1 KiB of contiguous memory (eight whole 128-byte lines), four
+//     such loads are in flight per wave while the previous four are consumed;
+//   * pass 1 streams K and leaves the scaled scores in LDS; the block then takes max and sum
+//     (fp32) once; pass 2 streams V with the normalised fp16 probabilities.  The first V rows
+//     are requested before the softmax reduction so that the reduction hides their latency;
+//   * the row that is being appended is taken from the new-row pointers, never read back from
+//     the cache, and stored to the cache by the lanes that hold it.
+// The number of valid rows may live on the device (HIP-graph replay with a growing cache).
+#include "sq_common.h"
+#include "sq_kernels.h"
+
+namespace sq {
+
+namespace {
+
+constexpr int DA_WAVES = 8;
+constexpr int DA_U = 4;  // 128-bit loads in flight per wave
+
+struct DecodeAttnArgs {
+    const half_t* q;
+    const half_t* kn;
+    const half_t* vn;
+    half_t* kc;
+    half_t* vc;
+    const half_t* mask;
+    half_t* o;
+    long q_bs, q_hs;  // element strides of q over batch / head
+    long n_bs, n_hs;  // ... of the new key and value rows
+    long c_bs, c_hs;  // ... of both caches (row stride is D)
+    long m_bs;        // ... of the additive mask over batch
+    int H, Lmax, cache_len;
+    const long long* cache_len_dev;
+    float scale;
+};
+
+__device__ __forceinline__ float xor_sum(float v, int m) { return v + __shfl_xor(v, m, 64); }
+
+template <int D>
+__global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnArgs a) {
+    constexpr int LPR = D / 8;    // lanes per cache row
+    constexpr int RPI = 64 / LPR; // rows per load instruction
+    constexpr int STEP = DA_WAVES * RPI * DA_U;
+    extern __shared__ float smem[];
+    float* sc = smem;                       // [Lmax rounded up to 4] scores, then exp(score - max)
+    float* red = smem + ((a.Lmax + 3) & ~3);  // [2 * DA_WAVES] block reductions
+    float* ored = red + 2 * DA_WAVES;       // [DA_WAVES][D] per-wave output partials
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int c = lane % LPR;
+    const int r = lane / LPR;
+    const int b = blockIdx.x / a.H;
+    const int h = blockIdx.x % a.H;
+    const bool append = a.kn != nullptr;
+
+    int n0 = a.cache_len_dev ? (int)*a.cache_len_dev : a.cache_len;
+    const int n0max = a.Lmax - (append ? 1 : 0);
+    n0 = n0 < 0 ? 0 : (n0 > n0max ? n0max : n0);
+    const int L = n0 + (append ? 1 : 0);  // rows attended; the appended row is row n0
+
+    half_t* kbase = a.kc + (long)b * a.c_bs + (long)h * a.c_hs + 8 * c;
+    half_t* vbase = a.vc + (long)b * a.c_bs + (long)h * a.c_hs + 8 * c;
+    const half_t* knrow = append ? a.kn + (long)b * a.n_bs + (long)h * a.n_hs + 8 * c : nullptr;
+    const half_t* vnrow = append ? a.vn + (long)b * a.n_bs + (long)h * a.n_hs + 8 * c : nullptr;
+    const half8_t qv = *(const half8_t*)(a.q + (long)b * a.q_bs + (long)h * a.q_hs + 8 * c);
+    const half2_t q01 = {qv[0], qv[1]}, q23 = {qv[2], qv[3]}, q45 = {qv[4], qv[5]}, q67 = {qv[6], qv[7]};
+
+    // Row j of a four-load batch that starts at `base`: base + u * RPI + r.
+    auto load_rows = [&](const half_t* cache, const half_t* fresh, int base, u32x4_t (&dst)[DA_U]) {
+#pragma unroll
+        for (int u = 0; u < DA_U; u++) {
+            const int j = imin(base + u * RPI + r, L - 1);
+            const half_t* src = (append && j == n0) ? fresh : cache + (long)j * D;
+            dst[u] = *(const u32x4_t*)src;
+        }
+    };
+    auto store_fresh = [&](half_t* cache, int base, const u32x4_t (&src)[DA_U]) {
+        if (!append) return;
+#pragma unroll
+        for (int u = 0; u < DA_U; u++)
+            if (base + u * RPI + r == n0) *(u32x4_t*)(cache + (long)n0 * D) = src[u];
+    };
+
+    // ---- pass 1: scores ----
+    if (L > 0) {
+        u32x4_t cur[DA_U], nxt[DA_U];
+        int base = wave * RPI * DA_U;
+        if (base < L) load_rows(kbase, knrow, base, cur);
+        for (; base < L; base += STEP) {
+            const bool more = base + STEP < L;
+            if (more) load_rows(kbase, knrow, base + STEP, nxt);
+            store_fresh(kbase, base, cur);
+#pragma unroll
+            for (int u = 0; u < DA_U; u++) {
+                const half8_t kv = bit_cast<half8_t>(cur[u]);
+                float s = __builtin_amdgcn_fdot2((half2_t){kv[0], kv[1]}, q01, 0.f, false);
+                s = __builtin_amdgcn_fdot2((half2_t){kv[2], kv[3]}, q23, s, false);
+                s = __builtin_amdgcn_fdot2((half2_t){kv[4], kv[5]}, q45, s, false);
+                s = __builtin_amdgcn_fdot2((half2_t){kv[6], kv[7]}, q67, s, false);
+                s = quad_sum(s);
+                s = xor_sum(s, 4);
+                if (LPR == 16) s = xor_sum(s, 8);
+                const int j = base + u * RPI + r;
+                if (c == 0 && j < L) {
+                    s *= a.scale;
+                    if (a.mask) s += (float)a.mask[(long)b * a.m_bs + j];
+                    sc[j] = s;
+                }
+            }
+            if (more) {
+#pragma unroll
+                for (int u = 0; u < DA_U; u++) cur[u] = nxt[u];
+            }
+        }
+    }
+
+    // First V rows on their way while the block reduces.
+    u32x4_t vcur[DA_U], vnxt[DA_U];
+    const int vbase0 = wave * RPI * DA_U;
+    if (vbase0 < L) load_rows(vbase, vnrow, vbase0, vcur);
+    __syncthreads();
+
+    // ---- softmax over sc[0..L) in fp32 ----
+    float mx = -INFINITY;
+    for (int j = tid; j < L; j += 64 * DA_WAVES) mx = fmaxf(mx, sc[j]);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < DA_WAVES; w++) mx = fmaxf(mx, red[w]);
+    float sum = 0.f;
+    for (int j = tid; j < L; j += 64 * DA_WAVES) {
+        const float e = __expf(sc[j] - mx);
+        sc[j] = e;
+        sum += e;
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) sum = xor_sum(sum, m);
+    if (lane == 0) red[DA_WAVES + wave] = sum;
+    __syncthreads();
+    sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < DA_WAVES; w++) sum += red[DA_WAVES + w];
+    const float inv = 1.f / sum;
+
+    // ---- pass 2: probabilities times V ----
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.f;
+    for (int base = vbase0; base < L; base += STEP) {
+        const bool more = base + STEP < L;
+        if (more) load_rows(vbase, vnrow, base + STEP, vnxt);
+        store_fresh(vbase, base, vcur);
+#pragma unroll
+        for (int u = 0; u < DA_U; u++) {
+            const int j = base + u * RPI + r;
+            const float p = j < L ? (float)(half_t)(sc[j] * inv) : 0.f;
+            const half8_t vv = bit_cast<half8_t>(vcur[u]);
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[i] += p * (float)vv[i];
+        }
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < DA_U; u++) vcur[u] = vnxt[u];
+        }
+    }
+    // Sum the row slots of a wave (lanes with equal c), then the waves.
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+#pragma unroll
+        for (int m = LPR; m < 64; m <<= 1) acc[i] = xor_sum(acc[i], m);
+    }
+    if (r == 0) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) ored[wave * D + 8 * c + i] = acc[i];
+    }
+    __syncthreads();
+    if (tid < D) {
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < DA_WAVES; w++) o += ored[w * D + tid];
+        a.o[(long)blockIdx.x * D + tid] = (half_t)o;
+    }
+}
+
+template <int D>
+hipError_t launch_d(const DecodeAttnArgs& a, int B, size_t lds, hipStream_t st) {
+    if (lds > 64 * 1024) {  // beyond the default limit of dynamic LDS per workgroup
+        const hipError_t e = hipFuncSetAttribute((const void*)decode_attn_kernel<D>,
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((decode_attn_kernel<D>), dim3(B * a.H), dim3(64 * DA_WAVES), lds, st, a);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+size_t decode_attention_lds_bytes(int Lmax, int D) {
+    return ((size_t)((Lmax + 3) & ~3) + 2 * DA_WAVES + (size_t)DA_WAVES * D) * sizeof(float);
+}
+
+hipError_t launch_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
+                                   const void* mask, void* out, int B, int H, int D, int Lmax, long q_bs, long q_hs,
+                                   long n_bs, long n_hs, long c_bs, long c_hs, long m_bs, int cache_len,
+                                   const long long* cache_len_dev, float sm_scale, hipStream_t st) {
+    DecodeAttnArgs a;
+    a.q = (const half_t*)q;
+    a.kn = (const half_t*)k_new;
+    a.vn = (const half_t*)v_new;
+    a.kc = (half_t*)k_cache;
+    a.vc = (half_t*)v_cache;
+    a.mask = (const half_t*)mask;
+    a.o = (half_t*)out;
+    a.q_bs = q_bs;
+    a.q_hs = q_hs;
+    a.n_bs = n_bs;
+    a.n_hs = n_hs;
+    a.c_bs = c_bs;
+    a.c_hs = c_hs;
+    a.m_bs = m_bs;
+    a.H = H;
+    a.Lmax = Lmax;
+    a.cache_len = cache_len;
+    a.cache_len_dev = cache_len_dev;
+    a.scale = sm_scale;
+    const size_t lds = decode_attention_lds_bytes(Lmax, D);
+    return D == 64 ? launch_d<64>(a, B, lds, st) : launch_d<128>(a, B, lds, st);
+}
+
+}  // namespace sq

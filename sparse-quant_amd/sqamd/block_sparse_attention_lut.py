@@ -5,10 +5,10 @@ sparse-attention/nvidia/playground/kernels/block_sparse_attention_lut.py:246-309
 (`sparse_attention(q, k, v, sm_scale, lut, LT, BLOCK_M, BLOCK_N, attention_mask,
 attention_dropout)`): prefill (q_len == kv_len) runs the HIP kernel behind
 sq_lut_attention_fwd; decode (q_len < kv_len, q_len == 1) is dense attention over
-the whole KV cache in torch, exactly as the reference does it.
+the whole KV cache, the same quantity the reference computes with two matmuls and a softmax,
+here in one kernel behind sq_decode_attention.
 """
 import torch
-from torch import nn
 
 from . import capi
 
@@ -31,15 +31,19 @@ def sparse_attention(q, k, v, sm_scale, lut, LT=True, BLOCK_M=64, BLOCK_N=64, at
                      attention_dropout=0.0):
     bsz, num_heads, q_len, _ = q.shape
     kv_len = k.size(2)
-    if q_len < kv_len:  # decode: dense over the cache
+    if q_len < kv_len:  # decode: dense over the cache, one kernel
         assert q_len == 1
-        w = torch.matmul(q, k.transpose(2, 3)) * sm_scale
+        if attention_mask is not None and attention_mask.size() != (bsz, 1, q_len, kv_len):
+            raise ValueError("Attention mask should be of size %s, but is %s"
+                             % ((bsz, 1, q_len, kv_len), tuple(attention_mask.size())))
+        if attention_dropout != 0.0:
+            raise ValueError("decode attention is inference only (the reference applies dropout with training=False)")
+        if not q.is_cuda:
+            raise RuntimeError("sparse_attention needs device tensors; there is no host path")
+        if k.stride(-1) != 1 or k.stride(2) != k.size(3) or v.stride() != k.stride():
+            k, v = k.contiguous(), v.contiguous()
         if attention_mask is not None:
-            if attention_mask.size() != (bsz, 1, q_len, kv_len):
-                raise ValueError("Attention mask should be of size %s, but is %s"
-                                 % ((bsz, 1, q_len, kv_len), tuple(attention_mask.size())))
-            w = w + attention_mask
-        w = nn.functional.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
-        w = nn.functional.dropout(w, p=attention_dropout, training=False)
-        return torch.matmul(w, v)
+            attention_mask = attention_mask.to(torch.float16).contiguous()
+        out = capi.decode_attention(q.contiguous(), k, v, kv_len, sm_scale, mask=attention_mask)
+        return out.view(bsz, num_heads, 1, -1)
     return sparse_attention_prefill(q, k, v, sm_scale, lut, LT, BLOCK_M, BLOCK_N)

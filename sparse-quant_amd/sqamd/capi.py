@@ -36,6 +36,7 @@ SIGNATURES = {
     "sq_repack_l2_to_l1": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "sq_convert_2bit_to_4bit": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_clock_probe": (_i, [_vp, _i, _vp]),
+    "sq_decode_attention": (_i, [_vp] * 7 + [_i] * 4 + [ctypes.c_long] * 7 + [_i, _vp, ctypes.c_float, _vp]),
     "sq_lut_attention_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, ctypes.c_float, _i, _vp]),
 }
 
@@ -188,6 +189,50 @@ def lut_attention(q, k, v, lut, sm_scale, causal, stream=None):
     _check(lib().sq_lut_attention_fwd(_ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lut), lut.element_size(), z, h, s, d,
                                       lut.shape[-1], float(sm_scale), int(bool(causal)), _stream(stream)),
            "sq_lut_attention_fwd")
+    return out
+
+
+def decode_attention(q, k_cache, v_cache, cache_len, sm_scale, k_new=None, v_new=None, mask=None, out=None,
+                     stream=None):
+    """Dense decode attention over an fp16 KV cache, optionally appending the new row.
+
+    q [B,H,1,D] or [B,H,D] (any batch/head strides, D contiguous); k_cache, v_cache [B,H,Lmax,D] with
+    contiguous rows (a slice cache[:, :, :L] of a bigger buffer is fine); k_new, v_new like q or None;
+    cache_len: int, or an int64 device tensor of one element (read by the kernel); mask None or fp16
+    [B,1,1,L] / [B,L] additive.  Returns out fp16 [B, 1, H*D]."""
+    b, h = q.shape[0], q.shape[1]
+    d = q.shape[-1]
+    q3 = q.reshape(b, h, d) if q.dim() == 4 else q
+    if q3.stride(-1) != 1 or k_cache.stride(-1) != 1 or k_cache.stride(2) != d or v_cache.stride() != k_cache.stride():
+        raise ValueError("decode_attention needs D-contiguous q and caches with contiguous rows")
+    lmax = k_cache.shape[2]
+    kn = vn = None
+    n_bs = n_hs = 0
+    if k_new is not None:
+        kn = k_new.reshape(b, h, d) if k_new.dim() == 4 else k_new
+        vn = v_new.reshape(b, h, d) if v_new.dim() == 4 else v_new
+        if kn.stride(-1) != 1 or vn.stride() != kn.stride():
+            raise ValueError("k_new and v_new must be D-contiguous with equal strides")
+        n_bs, n_hs = kn.stride(0), kn.stride(1)
+    m_bs = 0
+    if mask is not None:
+        mask = mask.reshape(b, -1)
+        if mask.dtype != torch.float16 or mask.stride(-1) != 1:
+            raise ValueError("mask must be fp16 with contiguous rows")
+        m_bs = mask.stride(0)
+    if out is None:
+        out = torch.empty((b, 1, h * d), dtype=torch.float16, device=q.device)
+    if torch.is_tensor(cache_len):
+        if cache_len.dtype != torch.int64 or not cache_len.is_cuda:
+            raise TypeError("a device-side cache_len must be an int64 device tensor")
+        len_host, len_dev = 0, _ptr(cache_len)
+    else:
+        len_host, len_dev = int(cache_len), None
+    _check(lib().sq_decode_attention(_ptr(q3), _ptr(kn) if kn is not None else None,
+                                     _ptr(vn) if vn is not None else None, _ptr(k_cache), _ptr(v_cache),
+                                     _ptr(mask) if mask is not None else None, _ptr(out), b, h, d, lmax,
+                                     q3.stride(0), q3.stride(1), n_bs, n_hs, k_cache.stride(0), k_cache.stride(1), m_bs,
+                                     len_host, len_dev, float(sm_scale), _stream(stream)), "sq_decode_attention")
     return out
 
 

@@ -7,8 +7,9 @@ are `WALinear` modules (layout L1, group 128) with random packed weights -- the 
 six linears per layer, in the same order and with the same [1, tokens, K] call shape
 the reference feeds to gemm_awq_ut (test/nvidia/module/opt/modeling_opt_ours.py:
 158-164, 505-506, 598-611).  Attention is dense (the reference's decode path is dense
-too); the KV cache is fp16 and preallocated so that a decode step is a fixed kernel
-sequence that can be captured in a HIP graph.
+too): the decode step appends to the preallocated fp16 KV cache and attends in one kernel
+(sq_decode_attention) that reads the position from the device, so the step is a fixed
+kernel sequence that can be captured in a HIP graph.
 """
 import math
 import time
@@ -16,6 +17,7 @@ import time
 import torch
 from torch import nn
 
+from . import capi
 from .qlinear import WALinear
 
 
@@ -43,7 +45,7 @@ class DecoderLayer(nn.Module):
         self.fc2 = _random_walinear(ffn, hidden, g, dev, gen)
         self.qkv_proj = None
 
-    def forward(self, x, kc, vc, pos0, mask):
+    def forward(self, x, kc, vc, pos0):
         """x [B, T, H]; kc, vc [B, heads, Lmax, hd]; writes cache rows pos0 .. pos0+T-1."""
         b, t, hdim = x.shape
         h = self.ln1(x)
@@ -60,11 +62,11 @@ class DecoderLayer(nn.Module):
             vc[:, :, pos0:pos0 + t] = v
             a = nn.functional.scaled_dot_product_attention(q, kc[:, :, :pos0 + t], vc[:, :, :pos0 + t],
                                                            is_causal=(t > 1))
-        else:  # graph-captured decode step: position lives in a device tensor, the mask hides unused rows
-            kc.index_copy_(2, pos0, k)
-            vc.index_copy_(2, pos0, v)
-            a = nn.functional.scaled_dot_product_attention(q, kc, vc, attn_mask=mask)
-        a = a.transpose(1, 2).reshape(1, b * t, hdim)
+            a = a.transpose(1, 2).reshape(1, b * t, hdim)
+        else:
+            # graph-captured decode step: the position lives in a device tensor; one kernel appends the
+            # new key/value rows to the cache and attends over rows 0 .. pos0, output already [b, 1, hidden]
+            a = capi.decode_attention(q, kc, vc, pos0, 1.0 / math.sqrt(self.hd), k_new=k, v_new=v).view(1, b * t, hdim)
         # bias, ReLU and the two residual adds ride in the kernels' stores
         x = self.out_proj(a, residual=x.reshape(1, b * t, hdim)).view(b, t, hdim)
         h = self.ln2(x).reshape(1, b * t, hdim)
@@ -105,13 +107,13 @@ class OPTDecoder(nn.Module):
                 for _ in self.layers]
 
     @torch.no_grad()
-    def forward(self, ids, cache, pos0, pos_ids=None, mask=None):
+    def forward(self, ids, cache, pos0, pos_ids=None):
         b, t = ids.shape
         if pos_ids is None:
             pos_ids = torch.arange(pos0, pos0 + t, device=ids.device) + 2
         x = self.embed[ids] + self.pos[pos_ids]
         for layer, (kc, vc) in zip(self.layers, cache):
-            x = layer(x, kc, vc, pos0, mask)
+            x = layer(x, kc, vc, pos0)
         x = self.final_ln(x[:, -1:])
         return torch.matmul(x, self.lm_head.t())  # [B, 1, vocab]
 
@@ -139,21 +141,15 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
 
     # One decode step with device-side position so that it can be replayed as a graph.
     pos_t = torch.tensor([prompt], device=dev, dtype=torch.long)
-    mask = torch.zeros((1, 1, 1, max_len), device=dev, dtype=torch.float16)
     tok = nxt.clone()
     out_tok = torch.empty_like(tok)
 
-    def set_mask():
-        mask.fill_(float("-inf"))
-        mask[..., :int(pos_t.item()) + 1] = 0
-
     def step():
-        lg = model(tok, cache, pos_t, pos_ids=pos_t + 2, mask=mask)
+        lg = model(tok, cache, pos_t, pos_ids=pos_t + 2)
         out_tok.copy_(lg.argmax(-1))
 
     graph = None
     if use_graph:
-        set_mask()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -164,13 +160,9 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
         with torch.cuda.graph(graph, stream=side):  # same stream as the warm-up: per-stream workspaces exist
             step()
     generated = [tok.clone()]
-    mask.fill_(float("-inf"))
-    mask[..., :prompt] = 0
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(new_tokens - 1):
-        # the key/value row written by this step becomes visible to it
-        mask[..., prompt + i] = 0
         if graph is not None:
             graph.replay()
         else:

@@ -83,3 +83,64 @@ def test_single_visible_key_returns_its_value_row():
     lut = att.layout_to_lut(att.synth_layout(2, 2, 1.0, causal=True))
     out = att.attention_ref(q, k, v, lut, 1.0, causal=True)
     assert np.array_equal(out[0, :, 0], v[0, :, 0])
+
+
+# ---- decode branch ----
+
+def test_decode_equal_keys_give_mean_of_values():
+    rng = np.random.default_rng(0)
+    b, h, l, d = 2, 3, 8, 16  # 1/8 is exact in fp16
+    q = rng.normal(size=(b, h, d))
+    k = np.broadcast_to(rng.normal(size=(b, h, 1, d)), (b, h, l, d))
+    v = rng.normal(size=(b, h, l, d))
+    out = att.decode_attention_ref(q, k, v, 0.3)
+    assert np.allclose(out, v.mean(axis=2), rtol=0, atol=1e-12)
+
+
+def test_decode_dominating_key_returns_its_value_row():
+    rng = np.random.default_rng(1)
+    b, h, l, d = 1, 2, 37, 8
+    q = np.zeros((b, h, d)); q[..., 0] = 1.0
+    k = np.zeros((b, h, l, d)); k[:, :, 5, 0] = 60.0   # score gap 60 -> all other probabilities round to 0
+    v = rng.normal(size=(b, h, l, d))
+    out = att.decode_attention_ref(q, k, v, 1.0)
+    assert np.array_equal(out, v[:, :, 5])
+
+
+def test_decode_two_key_closed_form():
+    # scores (a, 0): p0 = 1/(1+e^-a); P is rounded to fp16 before it meets v
+    a = 0.75
+    q = np.array([[[1.0, 0.0]]]); k = np.array([[[[a, 0.0], [0.0, 0.0]]]])
+    v = np.array([[[[1.0, 0.0], [0.0, 1.0]]]])
+    out = att.decode_attention_ref(q, k, v, 1.0)
+    p0 = 1.0 / (1.0 + np.exp(-a))
+    want = np.array([np.float16(p0), np.float16(1 - p0)], dtype=np.float64)
+    assert np.array_equal(out[0, 0], want)
+
+
+def test_decode_minus_inf_mask_equals_attention_over_remaining_rows():
+    rng = np.random.default_rng(2)
+    b, h, l, d = 2, 2, 21, 8
+    q = rng.normal(size=(b, h, d)); k = rng.normal(size=(b, h, l, d)); v = rng.normal(size=(b, h, l, d))
+    keep = np.array([0, 3, 4, 9, 20])
+    mask = np.full((b, l), -np.inf); mask[:, keep] = 0.0
+    got = att.decode_attention_ref(q, k, v, 0.35, mask)
+    want = att.decode_attention_ref(q, k[:, :, keep], v[:, :, keep], 0.35)
+    assert np.allclose(got, want, rtol=0, atol=1e-12)
+
+
+def test_decode_against_elementwise_loops():
+    import math
+    rng = np.random.default_rng(3)
+    b, h, l, d = 1, 2, 5, 4
+    q = rng.normal(size=(b, h, d)); k = rng.normal(size=(b, h, l, d)); v = rng.normal(size=(b, h, l, d))
+    mask = rng.normal(size=(b, l))
+    got = att.decode_attention_ref(q, k, v, 0.5, mask)
+    for hh in range(h):
+        s = [sum(q[0, hh, t] * k[0, hh, j, t] for t in range(d)) * 0.5 + mask[0, j] for j in range(l)]
+        m = max(s)
+        e = [math.exp(x - m) for x in s]
+        tot = sum(e)
+        p = [float(np.float16(x / tot)) for x in e]
+        for t in range(d):
+            assert abs(got[0, hh, t] - sum(p[j] * v[0, hh, j, t] for j in range(l))) < 1e-12
