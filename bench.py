@@ -233,6 +233,7 @@ def main():
             out["decode_batch"] = decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream)
             out["fused_qkv"] = fused_qkv_leg(torch, capi, m, g, dev, gen, stream, args.layers, bytes_per_step)
             out["attention"] = attention_leg(torch, capi, dev)
+            out["decode_attention"] = decode_attention_leg(torch, capi, dev)
             from sqamd import opt_decode
             out["e2e_opt67"] = opt_decode.run_e2e(batch=8, prompt=512, new_tokens=128)
         except Exception as exc:  # an extra leg must never hide the headline line
@@ -388,13 +389,13 @@ def fused_qkv_leg(torch, capi, m, g, dev, gen, stream, layers, bytes_per_step):
 def attention_leg(torch, capi, dev):
     """LUT block-sparse attention (BASELINE configs[3]): batch 8, 16 heads, head dim 64, 64x64 blocks,
     ~25 % density with the diagonal block kept, non-causal; flops = 4 * kept blocks * 64 * 64 * D."""
-    import lut_attention_oracle as att
+    from sqamd.lut_layout import layout2lut_single_density, synth_layout
     res = {}
     for s in (512, 4096):
         z, h, d = 8, 16, 64
-        lay = att.synth_layout(h, s // 64, 0.25, False, seed=1)
-        lut = torch.from_numpy(att.layout_to_lut(lay)).to(dev)
-        kept = int(lay.sum()) * z
+        lay = synth_layout(h, s // 64, 0.25, False, seed=1)
+        lut = layout2lut_single_density(lay[None])[0].to(dev)
+        kept = int(lay.sum().item()) * z
         q = torch.randn((z, h, s, d), device=dev).half()
         k = torch.randn_like(q)
         v = torch.randn_like(q)
@@ -411,6 +412,51 @@ def attention_leg(torch, capi, dev):
         tf = 4.0 * kept * 64 * 64 * d / us / 1e6
         res["seq%d" % s] = {"us": round(us, 1), "tflops": round(tf, 1),
                             "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4)}
+    return res
+
+
+def decode_attention_leg(torch, capi, dev, pool=8, reps=20):
+    """Dense decode attention of the end-to-end configuration: batch 8, 32 heads, head dim 128, 640 cache
+    rows (639 valid + the appended one), fp16; algorithmic bytes = K and V rows read once; caches rotate
+    through a pool larger than the last-level cache; HIP-graph replay.  torch's SDPA on the same tensors
+    (which also needs two copy launches for the append, not timed) is shown beside it."""
+    b, h, d, rows = 8, 32, 128, 640
+    qs = [torch.randn((b, h, 1, d), device=dev).half() for _ in range(pool)]
+    kcs = [torch.randn((b, h, rows, d), device=dev).half() for _ in range(pool)]
+    vcs = [torch.randn((b, h, rows, d), device=dev).half() for _ in range(pool)]
+    pos = torch.tensor([rows - 1], device=dev)
+    scale = d ** -0.5
+
+    def ours():
+        for i in range(pool):
+            capi.decode_attention(qs[i], kcs[i], vcs[i], pos, scale, k_new=qs[i], v_new=qs[i])
+
+    def sdpa():
+        for i in range(pool):
+            torch.nn.functional.scaled_dot_product_attention(qs[i], kcs[i], vcs[i])
+
+    res = {"shape": "B=8 H=32 D=128 rows=640", "bytes": 2 * b * h * rows * d * 2}
+    for name, fn in (("kernel", ours), ("torch_sdpa", sdpa)):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                fn()
+        graph.replay()
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * pool)
+        res[name] = {"us": round(us, 2), "gbs": round(res["bytes"] / us / 1e3, 1),
+                     "frac_of_hbm_peak": round(res["bytes"] / us / 1e3 / HBM_PEAK_GBS, 4)}
     return res
 
 

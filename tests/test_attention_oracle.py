@@ -144,3 +144,15 @@ def test_decode_against_elementwise_loops():
         p = [float(np.float16(x / tot)) for x in e]
         for t in range(d):
             assert abs(got[0, hh, t] - sum(p[j] * v[0, hh, j, t] for j in range(l))) < 1e-12
+
+
+def test_package_lut_builder_agrees_with_the_oracle():
+    import torch
+    from sqamd.lut_layout import layout2lut_single_density, synth_layout
+    for causal in (False, True):
+        lay = synth_layout(3, 9, 0.4, causal, seed=5)
+        assert bool(lay.diagonal(dim1=1, dim2=2).all())
+        if causal:
+            assert not bool(torch.triu(lay, diagonal=1).any())
+        lut = layout2lut_single_density(lay[None])[0]
+        assert np.array_equal(lut.numpy(), att.layout_to_lut(lay.numpy()))
