@@ -188,6 +188,14 @@ int sq_decode_attention(const void* q, const void* k_new, const void* v_new, voi
                         long new_bstride, long new_hstride, long cache_bstride, long cache_hstride, long mask_bstride,
                         int cache_len, const long long* cache_len_dev, float sm_scale, void* stream);
 
+/* LayerNorm over the last dimension: y[r,:] = (x[r,:] - mean) * rsqrt(var + eps) * gamma + beta,
+ * biased variance, statistics and arithmetic in fp32, x and y fp16 [rows, cols] contiguous (y may
+ * be x), gamma / beta fp16 [cols] or NULL; cols a multiple of 8, at most 16384.  Feeds the q/k/v and
+ * fc1 linears of a decoder layer, where torch's nn.LayerNorm costs as much as a decode GEMV
+ * (reference: test/nvidia/module/opt/modeling_opt_ours.py:500-507,561-562,603-604). */
+int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, int rows, int cols, float eps,
+                 void* stream);
+
 /* Diagnostic, no counterpart in the reference: a single wave spins for `spins`
  * (1 .. 2^26) dependent multiply-adds and writes three uint64 to out: shader-clock
  * ticks elapsed, ticks of the constant 100 MHz counter elapsed, and a dummy.  Run on

@@ -319,3 +319,19 @@ def synth_linear(n, k, g, seed=0):
 def synth_x(m, k, seed=1):
     rng = np.random.default_rng(seed)
     return rng.normal(0.0, 1.0, size=(m, k)).astype(np.float16)
+
+
+def layernorm_ref(x, gamma=None, beta=None, eps=1e-5):
+    """LayerNorm over the last axis in float64: (x - mean) / sqrt(biased var + eps) * gamma + beta,
+    what nn.LayerNorm computes at the call sites test/nvidia/module/opt/modeling_opt_ours.py:561-562,
+    603-604.  Pinned by closed forms in tests/test_oracle.py (constant rows, +-1 rows, shift
+    invariance, a row whose statistics are known by hand)."""
+    x = np.asarray(x, dtype=np.float64)
+    mean = x.mean(axis=-1, keepdims=True)
+    var = ((x - mean) ** 2).mean(axis=-1, keepdims=True)
+    y = (x - mean) / np.sqrt(var + eps)
+    if gamma is not None:
+        y = y * np.asarray(gamma, dtype=np.float64)
+    if beta is not None:
+        y = y + np.asarray(beta, dtype=np.float64)
+    return y

@@ -253,6 +253,16 @@ int sq_decode_attention(const void* q, const void* k_new, const void* v_new, voi
                                                    static_cast<hipStream_t>(stream)));
 }
 
+int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, int rows, int cols, float eps,
+                 void* stream) {
+    if (rows < 0 || cols <= 0 || cols % 8 != 0 || cols > 16384) return SQ_ERR_BAD_SHAPE;
+    if (rows == 0) return SQ_OK;
+    if (!x || !y) return SQ_ERR_NULL_POINTER;
+    if (!aligned16(x) || !aligned16(y) || (gamma && !aligned16(gamma)) || (beta && !aligned16(beta)))
+        return SQ_ERR_MISALIGNED;
+    return launch_code(sq::launch_layernorm(x, gamma, beta, y, rows, cols, eps, static_cast<hipStream_t>(stream)));
+}
+
 int sq_clock_probe(void* out, int spins, void* stream) {
     if (!out) return SQ_ERR_NULL_POINTER;
     if (spins <= 0 || spins > (1 << 26)) return SQ_ERR_BAD_SHAPE;

@@ -61,4 +61,9 @@ hipError_t launch_decode_attention(const void* q, const void* k_new, const void*
                                    long n_bs, long n_hs, long c_bs, long c_hs, long m_bs, int cache_len,
                                    const long long* cache_len_dev, float sm_scale, hipStream_t st);
 
+// sq_layernorm.hip: LayerNorm over the last dimension, fp16 in/out, fp32 statistics; cols % 8 == 0,
+// cols <= 16384.
+hipError_t launch_layernorm(const void* x, const void* gamma, const void* beta, void* y, int rows, int cols, float eps,
+                            hipStream_t st);
+
 }  // namespace sq

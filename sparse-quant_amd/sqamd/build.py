@@ -24,7 +24,7 @@ EXT_PATH = os.path.join(PKG_ROOT, "quant" + sysconfig.get_config_var("EXT_SUFFIX
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 HIP_SOURCES = ["sq_api.hip", "sq_dequant.hip", "sq_repack.hip", "sq_gemv.hip", "sq_gemv2.hip", "sq_skinny.hip", "sq_skinny2.hip", "sq_gemm.hip", "sq_gemm2.hip",
-               "sq_attn.hip", "sq_decode_attn.hip"]
+               "sq_attn.hip", "sq_decode_attn.hip", "sq_layernorm.hip"]
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
              # keep the compiler from forming packed-fp32 instructions
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

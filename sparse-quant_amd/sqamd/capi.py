@@ -37,6 +37,7 @@ SIGNATURES = {
     "sq_convert_2bit_to_4bit": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_clock_probe": (_i, [_vp, _i, _vp]),
     "sq_decode_attention": (_i, [_vp] * 7 + [_i] * 4 + [ctypes.c_long] * 7 + [_i, _vp, ctypes.c_float, _vp]),
+    "sq_layernorm": (_i, [_vp, _vp, _vp, _vp, _i, _i, ctypes.c_float, _vp]),
     "sq_lut_attention_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, ctypes.c_float, _i, _vp]),
 }
 
@@ -233,6 +234,16 @@ def decode_attention(q, k_cache, v_cache, cache_len, sm_scale, k_new=None, v_new
                                      _ptr(mask) if mask is not None else None, _ptr(out), b, h, d, lmax,
                                      q3.stride(0), q3.stride(1), n_bs, n_hs, k_cache.stride(0), k_cache.stride(1), m_bs,
                                      len_host, len_dev, float(sm_scale), _stream(stream)), "sq_decode_attention")
+    return out
+
+
+def layernorm(x, gamma, beta, eps=1e-5, out=None, stream=None):
+    """LayerNorm over the last dimension of a contiguous fp16 tensor; gamma / beta fp16 [cols] or None."""
+    cols = x.shape[-1]
+    if out is None:
+        out = torch.empty_like(x)
+    _check(lib().sq_layernorm(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(out), x.numel() // cols, cols, float(eps),
+                              _stream(stream)), "sq_layernorm")
     return out
 
 

@@ -211,3 +211,32 @@ def test_decoder_step_with_the_kernel_matches_the_torch_attention_path(capi):
             assert torch.equal(ka, kb) and torch.equal(va, vb)
         tok = want.argmax(-1)
         pos += 1
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 8), (8, 4096), (3, 5120), (5, 1000), (2, 8192), (4, 16384), (4096, 4096)])
+def test_layernorm_parity(capi, rows, cols):
+    import w4a16_oracle as orc
+    rng = np.random.default_rng(rows + cols)
+    x = (rng.normal(size=(rows, cols)) * 2 + 0.5).astype(np.float16)
+    gamma = rng.normal(size=cols).astype(np.float16)
+    beta = rng.normal(size=cols).astype(np.float16)
+    ref = orc.layernorm_ref(x, gamma, beta, 1e-5)
+    xt = torch.from_numpy(x).cuda()
+    out = capi.layernorm(xt, torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda(), 1e-5)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy().astype(np.float64)
+    # one rounding to fp16 at the end: half an ulp of the result, plus fp32 arithmetic noise
+    tol = np.abs(ref) * 2.0 ** -11 + 1e-3
+    assert np.all(np.abs(got - ref) <= tol), np.max(np.abs(got - ref))
+    # without affine parameters, and in place
+    ref0 = orc.layernorm_ref(x, None, None, 1e-5)
+    capi.layernorm(xt, None, None, 1e-5, out=xt)
+    got0 = xt.float().cpu().numpy().astype(np.float64)
+    assert np.all(np.abs(got0 - ref0) <= np.abs(ref0) * 2.0 ** -11 + 1e-3)
+
+
+def test_layernorm_rejections(capi):
+    x = torch.zeros((2, 12), dtype=torch.float16, device="cuda")
+    with pytest.raises(capi.SqError) as ei:
+        capi.layernorm(x, None, None)
+    assert ei.value.code == capi.SQ_ERR_BAD_SHAPE

@@ -257,3 +257,24 @@ def test_two_bit_kat_and_exhaustive():
     for v in range(256):
         a, bb, c, d = (v >> 4) & 3, (v >> 6) & 3, v & 3, (v >> 2) & 3
         assert out[v, 0] == (a | (bb << 4)) and out[v, 1] == (c | (d << 4))
+
+
+# ---- LayerNorm restatement ----
+
+def test_layernorm_closed_forms():
+    rng = np.random.default_rng(0)
+    gamma = rng.normal(size=16)
+    beta = rng.normal(size=16)
+    # a constant row has zero deviation: the output is beta
+    assert np.allclose(orc.layernorm_ref(np.full((2, 16), 3.25), gamma, beta), np.broadcast_to(beta, (2, 16)), atol=1e-12)
+    # +-1 alternating: mean 0, variance 1
+    x = np.tile([1.0, -1.0], 8)[None]
+    assert np.allclose(orc.layernorm_ref(x, gamma, beta, eps=1e-5), x / np.sqrt(1 + 1e-5) * gamma + beta, atol=1e-12)
+    # statistics by hand: [0, 0, 0, 4] has mean 1 and biased variance 3
+    y = orc.layernorm_ref(np.array([[0.0, 0.0, 0.0, 4.0]]), eps=0.0)
+    assert np.allclose(y, np.array([[-1.0, -1.0, -1.0, 3.0]]) / np.sqrt(3.0), atol=1e-12)
+    # shift invariance, and unit variance / zero mean of the normalised row
+    x = rng.normal(size=(3, 64))
+    assert np.allclose(orc.layernorm_ref(x + 7.5, eps=1e-5), orc.layernorm_ref(x, eps=1e-5), atol=1e-9)
+    y = orc.layernorm_ref(x, eps=0.0)
+    assert np.allclose(y.mean(axis=-1), 0, atol=1e-12) and np.allclose((y ** 2).mean(axis=-1), 1, atol=1e-12)
