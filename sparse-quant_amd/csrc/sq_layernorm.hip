@@ -5,7 +5,7 @@
 // nn.LayerNorm there); at that size the work is one launch latency, so the kernel is a single
 // pass: one workgroup per row, the row held in registers between the two reductions (mean
 // first, then the variance around it, as torch computes it), one 128-bit load and store per
-// eight elements.
+// eight elements, gamma and beta fetched before the reductions.
 #include "sq_common.h"
 #include "sq_kernels.h"
 
@@ -34,13 +34,26 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_kernel(const half_t* __r
     __shared__ float red[4];
     const long row = blockIdx.x;
     const int nvec = cols >> 3;
-    half8_t v[VPT];
+    half8_t v[VPT], g[VPT], b[VPT];
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < VPT; i++) {
         const int j = threadIdx.x + i * LN_THREADS;
+        if (j < nvec) v[i] = *(const half8_t*)(X + row * cols + 8 * j);
+    }
+    // gamma and beta are requested now so that their latency hides behind the two reductions
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int j = threadIdx.x + i * LN_THREADS;
         if (j < nvec) {
-            v[i] = *(const half8_t*)(X + row * cols + 8 * j);
+            if (gamma) g[i] = *(const half8_t*)(gamma + 8 * j);
+            if (beta) b[i] = *(const half8_t*)(beta + 8 * j);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; i++) {
+        const int j = threadIdx.x + i * LN_THREADS;
+        if (j < nvec) {
 #pragma unroll
             for (int e = 0; e < 8; e++) sum += (float)v[i][e];
         }
@@ -63,14 +76,12 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_kernel(const half_t* __r
     for (int i = 0; i < VPT; i++) {
         const int j = threadIdx.x + i * LN_THREADS;
         if (j < nvec) {
-            half8_t g, b, o;
-            if (gamma) g = *(const half8_t*)(gamma + 8 * j);
-            if (beta) b = *(const half8_t*)(beta + 8 * j);
+            half8_t o;
 #pragma unroll
             for (int e = 0; e < 8; e++) {
                 float t = ((float)v[i][e] - mean) * rstd;
-                if (gamma) t *= (float)g[e];
-                if (beta) t += (float)b[e];
+                if (gamma) t *= (float)g[i][e];
+                if (beta) t += (float)b[i][e];
                 o[e] = (half_t)t;
             }
             *(half8_t*)(Y + row * cols + 8 * j) = o;
