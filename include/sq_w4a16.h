@@ -163,8 +163,9 @@ int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out,
 
 /* Dense decode attention, one query token per sequence (q_len == 1 < kv_len):
  *   out[b,h,:] = sum_j P[j] v[b,h,j,:],  P = fp16(softmax_j(q[b,h,:] . k[b,h,j,:] * sm_scale + mask[b,j]))
- * over the first L rows of an fp16 key/value cache, softmax in fp32, probabilities rounded
- * to fp16 before they meet v, fp32 accumulation.  Replaces the decode branch of
+ * over the first L rows of an fp16 key/value cache, softmax and accumulation in fp32 (one
+ * streaming pass with an online softmax; the reference's rounding of P to fp16 is not
+ * reproduced, the result is within that rounding of it).  Replaces the decode branch of
  * sparse_attention (reference: sparse-attention/nvidia/playground/kernels/
  * block_sparse_attention_lut.py:272-300), which runs two torch.matmul and a softmax.
  *   q          fp16, element (b,h,d) at q[b*q_bstride + h*q_hstride + d]
@@ -181,8 +182,8 @@ int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out,
  *   cache_len  rows already valid; cache_len_dev, if not NULL, points to that number on the
  *              device (int64) and overrides cache_len -- read by the kernel, so a captured HIP
  *              graph follows a growing cache; the kernel clamps it to the cache size.
- * D in {64, 128}; all strides in elements and multiples of 8; pointers 16-byte aligned; Lmax up to
- * about 38000 rows (scores are held in LDS).  A fully masked row gives NaN, as in the reference. */
+ * D in {64, 128}; all strides in elements and multiples of 8; pointers 16-byte aligned.  A fully
+ * masked row gives NaN, as in the reference. */
 int sq_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
                         const void* mask, void* out, int B, int H, int D, int Lmax, long q_bstride, long q_hstride,
                         long new_bstride, long new_hstride, long cache_bstride, long cache_hstride, long mask_bstride,

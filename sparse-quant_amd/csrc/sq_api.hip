@@ -232,7 +232,6 @@ int sq_decode_attention(const void* q, const void* k_new, const void* v_new, voi
                         int cache_len, const long long* cache_len_dev, float sm_scale, void* stream) {
     if (B <= 0 || H <= 0 || Lmax <= 0 || (D != 64 && D != 128)) return SQ_ERR_BAD_SHAPE;
     if ((long)B * H > (1L << 24)) return SQ_ERR_BAD_SHAPE;
-    if (sq::decode_attention_lds_bytes(Lmax, D) > sq::DECODE_ATTN_MAX_LDS) return SQ_ERR_BAD_SHAPE;
     if (!q || !k_cache || !v_cache || !out) return SQ_ERR_NULL_POINTER;
     if ((k_new == nullptr) != (v_new == nullptr)) return SQ_ERR_NULL_POINTER;
     const bool append = k_new != nullptr;

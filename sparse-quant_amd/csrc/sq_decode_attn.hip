@@ -9,11 +9,14 @@
 // The work is a pure stream over the cache (2 * L * D * 2 bytes per head, two flops per
 // byte), so the kernel is laid out for the memory system and nothing else:
 //   * one workgroup of eight waves per (batch, head); a wave's 128-bit load covers 64/(D/8)
-//     consecutive cache rows = 1 KiB of contiguous memory (eight whole 128-byte lines), four
-//     such loads are in flight per wave while the previous four are consumed;
-//   * pass 1 streams K and leaves the scaled scores in LDS; the block then takes max and sum
-//     (fp32) once; pass 2 streams V with the normalised fp16 probabilities.  The first V rows
-//     are requested before the softmax reduction so that the reduction hides their latency;
+//     consecutive cache rows = 1 KiB of contiguous memory (eight whole 128-byte lines); the K
+//     and V rows of a batch of rows are requested together, the next batch while the current
+//     one is consumed;
+//   * one pass: every 16-lane (D = 128) or 8-lane (D = 64) row slot of every wave runs its own
+//     online softmax (running maximum, sum and 8 output columns per lane, all fp32) over the
+//     rows it is dealt; no barrier and no LDS inside the stream; the 32 or 64 partial states
+//     of a head are merged once at the end.  The probabilities meet V unrounded (the reference
+//     rounds the normalised ones to fp16 first; the difference is below its own rounding);
 //   * the row that is being appended is taken from the new-row pointers, never read back from
 //     the cache, and stored to the cache by the lanes that hold it.
 // The number of valid rows may live on the device (HIP-graph replay with a growing cache).
@@ -51,10 +54,9 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
     constexpr int LPR = D / 8;    // lanes per cache row
     constexpr int RPI = 64 / LPR; // rows per load instruction
     constexpr int STEP = DA_WAVES * RPI * DA_U;
-    extern __shared__ float smem[];
-    float* sc = smem;                       // [Lmax rounded up to 4] scores, then exp(score - max)
-    float* red = smem + ((a.Lmax + 3) & ~3);  // [2 * DA_WAVES] block reductions
-    float* ored = red + 2 * DA_WAVES;       // [DA_WAVES][D] per-wave output partials
+    __shared__ float mred[DA_WAVES];
+    __shared__ float lred[DA_WAVES];
+    __shared__ float ored[DA_WAVES][D];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -74,10 +76,12 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
     half_t* vbase = a.vc + (long)b * a.c_bs + (long)h * a.c_hs + 8 * c;
     const half_t* knrow = append ? a.kn + (long)b * a.n_bs + (long)h * a.n_hs + 8 * c : nullptr;
     const half_t* vnrow = append ? a.vn + (long)b * a.n_bs + (long)h * a.n_hs + 8 * c : nullptr;
+    const half_t* mrow = a.mask ? a.mask + (long)b * a.m_bs : nullptr;
     const half8_t qv = *(const half8_t*)(a.q + (long)b * a.q_bs + (long)h * a.q_hs + 8 * c);
     const half2_t q01 = {qv[0], qv[1]}, q23 = {qv[2], qv[3]}, q45 = {qv[4], qv[5]}, q67 = {qv[6], qv[7]};
 
-    // Row j of a four-load batch that starts at `base`: base + u * RPI + r.
+    // Row j of a batch that starts at `base`: base + u * RPI + r (clamped for the loads; rows past
+    // the end get probability zero).
     auto load_rows = [&](const half_t* cache, const half_t* fresh, int base, u32x4_t (&dst)[DA_U]) {
 #pragma unroll
         for (int u = 0; u < DA_U; u++) {
@@ -93,125 +97,112 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
             if (base + u * RPI + r == n0) *(u32x4_t*)(cache + (long)n0 * D) = src[u];
     };
 
-    // ---- pass 1: scores ----
-    if (L > 0) {
-        u32x4_t cur[DA_U], nxt[DA_U];
-        int base = wave * RPI * DA_U;
-        if (base < L) load_rows(kbase, knrow, base, cur);
-        for (; base < L; base += STEP) {
-            const bool more = base + STEP < L;
-            if (more) load_rows(kbase, knrow, base + STEP, nxt);
-            store_fresh(kbase, base, cur);
-#pragma unroll
-            for (int u = 0; u < DA_U; u++) {
-                const half8_t kv = bit_cast<half8_t>(cur[u]);
-                float s = __builtin_amdgcn_fdot2((half2_t){kv[0], kv[1]}, q01, 0.f, false);
-                s = __builtin_amdgcn_fdot2((half2_t){kv[2], kv[3]}, q23, s, false);
-                s = __builtin_amdgcn_fdot2((half2_t){kv[4], kv[5]}, q45, s, false);
-                s = __builtin_amdgcn_fdot2((half2_t){kv[6], kv[7]}, q67, s, false);
-                s = quad_sum(s);
-                s = xor_sum(s, 4);
-                if (LPR == 16) s = xor_sum(s, 8);
-                const int j = base + u * RPI + r;
-                if (c == 0 && j < L) {
-                    s *= a.scale;
-                    if (a.mask) s += (float)a.mask[(long)b * a.m_bs + j];
-                    sc[j] = s;
-                }
-            }
-            if (more) {
-#pragma unroll
-                for (int u = 0; u < DA_U; u++) cur[u] = nxt[u];
-            }
-        }
-    }
-
-    // First V rows on their way while the block reduces.
-    u32x4_t vcur[DA_U], vnxt[DA_U];
-    const int vbase0 = wave * RPI * DA_U;
-    if (vbase0 < L) load_rows(vbase, vnrow, vbase0, vcur);
-    __syncthreads();
-
-    // ---- softmax over sc[0..L) in fp32 ----
-    float mx = -INFINITY;
-    for (int j = tid; j < L; j += 64 * DA_WAVES) mx = fmaxf(mx, sc[j]);
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) mx = fmaxf(mx, __shfl_xor(mx, m, 64));
-    if (lane == 0) red[wave] = mx;
-    __syncthreads();
-#pragma unroll
-    for (int w = 0; w < DA_WAVES; w++) mx = fmaxf(mx, red[w]);
-    float sum = 0.f;
-    for (int j = tid; j < L; j += 64 * DA_WAVES) {
-        const float e = __expf(sc[j] - mx);
-        sc[j] = e;
-        sum += e;
-    }
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) sum = xor_sum(sum, m);
-    if (lane == 0) red[DA_WAVES + wave] = sum;
-    __syncthreads();
-    sum = 0.f;
-#pragma unroll
-    for (int w = 0; w < DA_WAVES; w++) sum += red[DA_WAVES + w];
-    const float inv = 1.f / sum;
-
-    // ---- pass 2: probabilities times V ----
+    // Online softmax state of this lane's row slot (the LPR lanes of a slot hold the same m and l).
+    float m = -INFINITY, l = 0.f;
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.f;
-    for (int base = vbase0; base < L; base += STEP) {
+
+    u32x4_t kcur[DA_U], vcur[DA_U], knxt[DA_U], vnxt[DA_U];
+    int base = wave * RPI * DA_U;
+    if (base < L) {
+        load_rows(kbase, knrow, base, kcur);
+        load_rows(vbase, vnrow, base, vcur);
+    }
+    for (; base < L; base += STEP) {
         const bool more = base + STEP < L;
-        if (more) load_rows(vbase, vnrow, base + STEP, vnxt);
+        if (more) {
+            load_rows(kbase, knrow, base + STEP, knxt);
+            load_rows(vbase, vnrow, base + STEP, vnxt);
+        }
+        store_fresh(kbase, base, kcur);
         store_fresh(vbase, base, vcur);
+        float sc[DA_U];
+        float mx = m;
 #pragma unroll
         for (int u = 0; u < DA_U; u++) {
+            const half8_t kv = bit_cast<half8_t>(kcur[u]);
+            float s = __builtin_amdgcn_fdot2((half2_t){kv[0], kv[1]}, q01, 0.f, false);
+            s = __builtin_amdgcn_fdot2((half2_t){kv[2], kv[3]}, q23, s, false);
+            s = __builtin_amdgcn_fdot2((half2_t){kv[4], kv[5]}, q45, s, false);
+            s = __builtin_amdgcn_fdot2((half2_t){kv[6], kv[7]}, q67, s, false);
+            s = quad_sum(s);
+            s = xor_sum(s, 4);
+            if (LPR == 16) s = xor_sum(s, 8);
             const int j = base + u * RPI + r;
-            const float p = j < L ? (float)(half_t)(sc[j] * inv) : 0.f;
+            s *= a.scale;
+            if (mrow && j < L) s += (float)mrow[j];
+            sc[u] = j < L ? s : -INFINITY;
+            mx = fmaxf(mx, sc[u]);
+        }
+        // exp(-inf - -inf) is kept out: a slot that has seen only masked rows stays at (m, l) = (-inf, 0)
+        const float rescale = (m == -INFINITY) ? 0.f : __expf(m - mx);
+        l *= rescale;
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] *= rescale;
+#pragma unroll
+        for (int u = 0; u < DA_U; u++) {
+            const float p = (sc[u] == -INFINITY) ? 0.f : __expf(sc[u] - mx);
+            l += p;
             const half8_t vv = bit_cast<half8_t>(vcur[u]);
 #pragma unroll
             for (int i = 0; i < 8; i++) acc[i] += p * (float)vv[i];
         }
+        m = mx;
         if (more) {
 #pragma unroll
-            for (int u = 0; u < DA_U; u++) vcur[u] = vnxt[u];
+            for (int u = 0; u < DA_U; u++) {
+                kcur[u] = knxt[u];
+                vcur[u] = vnxt[u];
+            }
         }
     }
-    // Sum the row slots of a wave (lanes with equal c), then the waves.
+
+    // Merge the row slots of a wave (lanes with equal c), then the waves.
+    float mw = m;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
+    for (int x = LPR; x < 64; x <<= 1) mw = fmaxf(mw, __shfl_xor(mw, x, 64));
+    const float sw = (m == -INFINITY) ? 0.f : __expf(m - mw);
+    l *= sw;
 #pragma unroll
-        for (int m = LPR; m < 64; m <<= 1) acc[i] = xor_sum(acc[i], m);
+    for (int i = 0; i < 8; i++) acc[i] *= sw;
+#pragma unroll
+    for (int x = LPR; x < 64; x <<= 1) {
+        l = xor_sum(l, x);
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] = xor_sum(acc[i], x);
+    }
+    if (lane == 0) {
+        mred[wave] = mw;
+        lred[wave] = l;
     }
     if (r == 0) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) ored[wave * D + 8 * c + i] = acc[i];
+        for (int i = 0; i < 8; i++) ored[wave][8 * c + i] = acc[i];
     }
     __syncthreads();
     if (tid < D) {
-        float o = 0.f;
+        float mb = mred[0];
 #pragma unroll
-        for (int w = 0; w < DA_WAVES; w++) o += ored[w * D + tid];
-        a.o[(long)blockIdx.x * D + tid] = (half_t)o;
+        for (int w = 1; w < DA_WAVES; w++) mb = fmaxf(mb, mred[w]);
+        float lsum = 0.f, o = 0.f;
+#pragma unroll
+        for (int w = 0; w < DA_WAVES; w++) {
+            const float f = (mred[w] == -INFINITY) ? 0.f : __expf(mred[w] - mb);
+            lsum += lred[w] * f;
+            o += ored[w][tid] * f;
+        }
+        a.o[(long)blockIdx.x * D + tid] = (half_t)(o / lsum);  // nothing visible: 0 / 0 = NaN, as the reference
     }
 }
 
 template <int D>
-hipError_t launch_d(const DecodeAttnArgs& a, int B, size_t lds, hipStream_t st) {
-    if (lds > 64 * 1024) {  // beyond the default limit of dynamic LDS per workgroup
-        const hipError_t e = hipFuncSetAttribute((const void*)decode_attn_kernel<D>,
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-    }
-    hipLaunchKernelGGL((decode_attn_kernel<D>), dim3(B * a.H), dim3(64 * DA_WAVES), lds, st, a);
+hipError_t launch_d(const DecodeAttnArgs& a, int B, hipStream_t st) {
+    hipLaunchKernelGGL((decode_attn_kernel<D>), dim3(B * a.H), dim3(64 * DA_WAVES), 0, st, a);
     return hipGetLastError();
 }
 
 }  // namespace
-
-size_t decode_attention_lds_bytes(int Lmax, int D) {
-    return ((size_t)((Lmax + 3) & ~3) + 2 * DA_WAVES + (size_t)DA_WAVES * D) * sizeof(float);
-}
 
 hipError_t launch_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
                                    const void* mask, void* out, int B, int H, int D, int Lmax, long q_bs, long q_hs,
@@ -237,8 +228,7 @@ hipError_t launch_decode_attention(const void* q, const void* k_new, const void*
     a.cache_len = cache_len;
     a.cache_len_dev = cache_len_dev;
     a.scale = sm_scale;
-    const size_t lds = decode_attention_lds_bytes(Lmax, D);
-    return D == 64 ? launch_d<64>(a, B, lds, st) : launch_d<128>(a, B, lds, st);
+    return D == 64 ? launch_d<64>(a, B, st) : launch_d<128>(a, B, st);
 }
 
 }  // namespace sq

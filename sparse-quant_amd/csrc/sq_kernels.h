@@ -53,9 +53,7 @@ hipError_t launch_lut_attention(const void* q, const void* k, const void* v, voi
                                 hipStream_t st);
 
 // sq_decode_attn.hip: dense decode attention over an fp16 KV cache (one query row per sequence),
-// optionally appending the new key/value row.  Strides in elements; LDS need grows with Lmax.
-constexpr size_t DECODE_ATTN_MAX_LDS = 160 * 1024;
-size_t decode_attention_lds_bytes(int Lmax, int D);
+// optionally appending the new key/value row.  Strides in elements.
 hipError_t launch_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
                                    const void* mask, void* out, int B, int H, int D, int Lmax, long q_bs, long q_hs,
                                    long n_bs, long n_hs, long c_bs, long c_hs, long m_bs, int cache_len,
