@@ -162,7 +162,7 @@ int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out,
                          void* stream);
 
 /* Dense decode attention, one query token per sequence (q_len == 1 < kv_len):
- *   out[b,h,:] = sum_j P[j] v[b,h,j,:],  P = fp16(softmax_j(q[b,h,:] . k[b,h,j,:] * sm_scale + mask[b,j]))
+ *   out[b,h,:] = sum_j P[j] v[b,h,j,:],  P = softmax_j(q[b,h,:] . k[b,h,j,:] * sm_scale + mask[b,j])
  * over the first L rows of an fp16 key/value cache, softmax and accumulation in fp32 (one
  * streaming pass with an online softmax; the reference's rounding of P to fp16 is not
  * reproduced, the result is within that rounding of it).  Replaces the decode branch of

@@ -1,9 +1,9 @@
 // Dense decode attention: one query token per sequence against an fp16 key/value cache,
 // optionally appending the step's new key/value row to the cache in the same launch.
 //
-// out[b,h,:] = sum_j P[j] * V[b,h,j,:],  P = fp16(softmax_j(q[b,h,:] . K[b,h,j,:] * sm_scale + mask[b,j]))
-// over the rows j < L of the cache, softmax in fp32, P rounded to fp16 before it meets V,
-// fp32 accumulation, fp16 output -- the decode branch of the reference's sparse_attention
+// out[b,h,:] = sum_j P[j] * V[b,h,j,:],  P = softmax_j(q[b,h,:] . K[b,h,j,:] * sm_scale + mask[b,j])
+// over the rows j < L of the cache, fp32 softmax and accumulation, fp16 output -- the decode
+// branch of the reference's sparse_attention
 // (reference: sparse-attention/nvidia/playground/kernels/block_sparse_attention_lut.py:272-300).
 //
 // The work is a pure stream over the cache (2 * L * D * 2 bytes per head, two flops per

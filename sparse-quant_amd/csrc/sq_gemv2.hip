@@ -259,7 +259,7 @@ hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void
         ks = nsteps > 16 ? 4 : (((long)N * K >= (1L << 25) && nsteps >= 8) ? 2 : 1);
         if (M >= 3 && M <= 4 && ks == 1 && nsteps >= 8) ks = 2;  // 4096 x 4096 with 3..4 tokens: 4.5 vs 5.6 us
     }
-    if (nr != 2 && nr != 4 && nr != 8) nr = ks == 4 ? 2 : 4;
+    if (nr != 2 && nr != 4 && nr != 8) nr = (ks == 4 && M <= 1) ? 2 : 4;  // 4096 x 16384 at M = 4: 12.8 vs 13.7 us
     const int spw = (nsteps + ks - 1) / ks;
     if (M <= 1) return launch_rows<1>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
     if (M <= 2) return launch_rows<2>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, epi, st);

@@ -240,3 +240,12 @@ def test_layernorm_rejections(capi):
     with pytest.raises(capi.SqError) as ei:
         capi.layernorm(x, None, None)
     assert ei.value.code == capi.SQ_ERR_BAD_SHAPE
+
+
+def test_decode_long_cache(capi):
+    # 40000 rows: far beyond what a score buffer in LDS could hold
+    b, h, l, d = 1, 2, 40000, 64
+    q, k, v = make(b, h, l, d, seed=51)
+    ref = att.decode_attention_ref(q, k, v, 0.125)
+    out = capi.decode_attention(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(), l, 0.125)
+    check(out, ref, "long cache")
