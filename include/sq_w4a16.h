@@ -182,12 +182,20 @@ int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out,
  *   cache_len  rows already valid; cache_len_dev, if not NULL, points to that number on the
  *              device (int64) and overrides cache_len -- read by the kernel, so a captured HIP
  *              graph follows a growing cache; the kernel clamps it to the cache size.
+ *   workspace  NULL, or sq_decode_attention_workspace_bytes(B, H, D) bytes, 16-byte aligned, its
+ *              first B*H*4 bytes zero before the first call (every call leaves them zero).  The kernel
+ *              runs one workgroup per (batch, head); with fewer than 256 of them and a workspace
+ *              the cache rows of a head are shared among up to 16 workgroups whose partial
+ *              softmax states meet in the workspace (batch 1, 32 heads, 640 rows: 4 workgroups
+ *              per head).  Calls that share a workspace must be ordered (same stream).
  * D in {64, 128}; all strides in elements and multiples of 8; pointers 16-byte aligned.  A fully
  * masked row gives NaN, as in the reference. */
 int sq_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
                         const void* mask, void* out, int B, int H, int D, int Lmax, long q_bstride, long q_hstride,
                         long new_bstride, long new_hstride, long cache_bstride, long cache_hstride, long mask_bstride,
-                        int cache_len, const long long* cache_len_dev, float sm_scale, void* stream);
+                        int cache_len, const long long* cache_len_dev, float sm_scale, void* workspace,
+                        size_t workspace_bytes, void* stream);
+size_t sq_decode_attention_workspace_bytes(int B, int H, int D);
 
 /* LayerNorm over the last dimension: y[r,:] = (x[r,:] - mean) * rsqrt(var + eps) * gamma + beta,
  * biased variance, statistics and arithmetic in fp32, x and y fp16 [rows, cols] contiguous (y may

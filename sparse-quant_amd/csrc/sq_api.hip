@@ -229,7 +229,8 @@ int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out,
 int sq_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
                         const void* mask, void* out, int B, int H, int D, int Lmax, long q_bstride, long q_hstride,
                         long new_bstride, long new_hstride, long cache_bstride, long cache_hstride, long mask_bstride,
-                        int cache_len, const long long* cache_len_dev, float sm_scale, void* stream) {
+                        int cache_len, const long long* cache_len_dev, float sm_scale, void* workspace,
+                        size_t workspace_bytes, void* stream) {
     if (B <= 0 || H <= 0 || Lmax <= 0 || (D != 64 && D != 128)) return SQ_ERR_BAD_SHAPE;
     if ((long)B * H > (1L << 24)) return SQ_ERR_BAD_SHAPE;
     if (!q || !k_cache || !v_cache || !out) return SQ_ERR_NULL_POINTER;
@@ -249,7 +250,13 @@ int sq_decode_attention(const void* q, const void* k_new, const void* v_new, voi
     return launch_code(sq::launch_decode_attention(q, k_new, v_new, k_cache, v_cache, mask, out, B, H, D, Lmax,
                                                    q_bstride, q_hstride, new_bstride, new_hstride, cache_bstride,
                                                    cache_hstride, mask_bstride, cache_len, cache_len_dev, sm_scale,
+                                                   aligned16(workspace) ? workspace : nullptr, workspace_bytes,
                                                    static_cast<hipStream_t>(stream)));
+}
+
+size_t sq_decode_attention_workspace_bytes(int B, int H, int D) {
+    if (B <= 0 || H <= 0 || (D != 64 && D != 128)) return 0;
+    return sq::decode_attention_workspace_bytes(B, H, D);
 }
 
 int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, int rows, int cols, float eps,

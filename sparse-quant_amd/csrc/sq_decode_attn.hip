@@ -45,6 +45,11 @@ struct DecodeAttnArgs {
     int H, Lmax, cache_len;
     const long long* cache_len_dev;
     float scale;
+    // Split of the cache rows over gridDim.y workgroups per (batch, head), for launches with too few
+    // heads to fill the chip: partial softmax states (m, l, D outputs) meet in `part`, one counter
+    // per head in `counters` (zero between calls), the last arriver merges.
+    float* part;
+    unsigned* counters;
 };
 
 __device__ __forceinline__ float xor_sum(float v, int m) { return v + __shfl_xor(v, m, 64); }
@@ -57,6 +62,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
     __shared__ float mred[DA_WAVES];
     __shared__ float lred[DA_WAVES];
     __shared__ float ored[DA_WAVES][D];
+    __shared__ unsigned last_flag;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -71,6 +77,11 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
     const int n0max = a.Lmax - (append ? 1 : 0);
     n0 = n0 < 0 ? 0 : (n0 > n0max ? n0max : n0);
     const int L = n0 + (append ? 1 : 0);  // rows attended; the appended row is row n0
+    // This workgroup's share of the rows: [r0, r1).
+    const int nsplit = gridDim.y;
+    const int rows_per = (L + nsplit - 1) / nsplit;
+    const int r0 = imin(blockIdx.y * rows_per, L);
+    const int r1 = imin(r0 + rows_per, L);
 
     half_t* kbase = a.kc + (long)b * a.c_bs + (long)h * a.c_hs + 8 * c;
     half_t* vbase = a.vc + (long)b * a.c_bs + (long)h * a.c_hs + 8 * c;
@@ -85,7 +96,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
     auto load_rows = [&](const half_t* cache, const half_t* fresh, int base, u32x4_t (&dst)[DA_U]) {
 #pragma unroll
         for (int u = 0; u < DA_U; u++) {
-            const int j = imin(base + u * RPI + r, L - 1);
+            const int j = imin(base + u * RPI + r, r1 - 1);
             const half_t* src = (append && j == n0) ? fresh : cache + (long)j * D;
             dst[u] = *(const u32x4_t*)src;
         }
@@ -94,7 +105,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
         if (!append) return;
 #pragma unroll
         for (int u = 0; u < DA_U; u++)
-            if (base + u * RPI + r == n0) *(u32x4_t*)(cache + (long)n0 * D) = src[u];
+            if (base + u * RPI + r == n0 && n0 < r1) *(u32x4_t*)(cache + (long)n0 * D) = src[u];
     };
 
     // Online softmax state of this lane's row slot (the LPR lanes of a slot hold the same m and l).
@@ -104,13 +115,13 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
     for (int i = 0; i < 8; i++) acc[i] = 0.f;
 
     u32x4_t kcur[DA_U], vcur[DA_U], knxt[DA_U], vnxt[DA_U];
-    int base = wave * RPI * DA_U;
-    if (base < L) {
+    int base = r0 + wave * RPI * DA_U;
+    if (base < r1) {
         load_rows(kbase, knrow, base, kcur);
         load_rows(vbase, vnrow, base, vcur);
     }
-    for (; base < L; base += STEP) {
-        const bool more = base + STEP < L;
+    for (; base < r1; base += STEP) {
+        const bool more = base + STEP < r1;
         if (more) {
             load_rows(kbase, knrow, base + STEP, knxt);
             load_rows(vbase, vnrow, base + STEP, vnxt);
@@ -131,8 +142,8 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
             if (LPR == 16) s = xor_sum(s, 8);
             const int j = base + u * RPI + r;
             s *= a.scale;
-            if (mrow && j < L) s += (float)mrow[j];
-            sc[u] = j < L ? s : -INFINITY;
+            if (mrow && j < r1) s += (float)mrow[j];
+            sc[u] = j < r1 ? s : -INFINITY;
             mx = fmaxf(mx, sc[u]);
         }
         // exp(-inf - -inf) is kept out: a slot that has seen only masked rows stays at (m, l) = (-inf, 0)
@@ -181,33 +192,83 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
         for (int i = 0; i < 8; i++) ored[wave][8 * c + i] = acc[i];
     }
     __syncthreads();
-    if (tid < D) {
-        float mb = mred[0];
+    float mb = mred[0];
 #pragma unroll
-        for (int w = 1; w < DA_WAVES; w++) mb = fmaxf(mb, mred[w]);
-        float lsum = 0.f, o = 0.f;
+    for (int w = 1; w < DA_WAVES; w++) mb = fmaxf(mb, mred[w]);
+    float lsum = 0.f, o = 0.f;
+    if (tid < D) {
 #pragma unroll
         for (int w = 0; w < DA_WAVES; w++) {
             const float f = (mred[w] == -INFINITY) ? 0.f : __expf(mred[w] - mb);
             lsum += lred[w] * f;
             o += ored[w][tid] * f;
         }
-        a.o[(long)blockIdx.x * D + tid] = (half_t)(o / lsum);  // nothing visible: 0 / 0 = NaN, as the reference
     }
+    if (nsplit == 1) {
+        if (tid < D) a.o[(long)blockIdx.x * D + tid] = (half_t)(o / lsum);  // nothing visible: 0 / 0 = NaN, as the reference
+        return;
+    }
+    // Partial state of this share: [m, l, o[0..D)], exchanged at the device-coherent level (relaxed
+    // agent-scope accesses, ordered by the wait below and the counter; no device-wide fence).
+    float* mine = a.part + ((long)blockIdx.x * nsplit + blockIdx.y) * (D + 2);
+    if (tid < D) __hip_atomic_store(mine + 2 + tid, o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) {
+        __hip_atomic_store(mine, mb, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(mine + 1, lsum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned old = __hip_atomic_fetch_add(&a.counters[blockIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last_flag = (old == (unsigned)(nsplit - 1)) ? 1u : 0u;
+    }
+    __syncthreads();
+    if (!last_flag) return;
+    if (tid < D) {
+        const float* all = a.part + (long)blockIdx.x * nsplit * (D + 2);
+        float mg = -INFINITY;
+        for (int sp = 0; sp < nsplit; sp++)
+            mg = fmaxf(mg, __hip_atomic_load(all + sp * (D + 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        float lg = 0.f, og = 0.f;
+        for (int sp = 0; sp < nsplit; sp++) {  // fixed order: bit-reproducible
+            const float ms = __hip_atomic_load(all + sp * (D + 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const float f = (ms == -INFINITY) ? 0.f : __expf(ms - mg);
+            lg += __hip_atomic_load(all + sp * (D + 2) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+            og += __hip_atomic_load(all + sp * (D + 2) + 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+        }
+        a.o[(long)blockIdx.x * D + tid] = (half_t)(og / lg);
+    }
+    if (tid == 0) __hip_atomic_store(&a.counters[blockIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <int D>
-hipError_t launch_d(const DecodeAttnArgs& a, int B, hipStream_t st) {
-    hipLaunchKernelGGL((decode_attn_kernel<D>), dim3(B * a.H), dim3(64 * DA_WAVES), 0, st, a);
+hipError_t launch_d(const DecodeAttnArgs& a, int B, int nsplit, hipStream_t st) {
+    hipLaunchKernelGGL((decode_attn_kernel<D>), dim3(B * a.H, nsplit), dim3(64 * DA_WAVES), 0, st, a);
     return hipGetLastError();
 }
 
 }  // namespace
 
+static size_t decode_attention_counter_bytes(int B, int H) { return (((size_t)B * H * 4) + 255) & ~(size_t)255; }
+
+size_t decode_attention_workspace_bytes(int B, int H, int D) {
+    return decode_attention_counter_bytes(B, H) + (size_t)B * H * DECODE_ATTN_MAX_SPLIT * (D + 2) * sizeof(float);
+}
+
 hipError_t launch_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
                                    const void* mask, void* out, int B, int H, int D, int Lmax, long q_bs, long q_hs,
                                    long n_bs, long n_hs, long c_bs, long c_hs, long m_bs, int cache_len,
-                                   const long long* cache_len_dev, float sm_scale, hipStream_t st) {
+                                   const long long* cache_len_dev, float sm_scale, void* workspace,
+                                   size_t workspace_bytes, hipStream_t st) {
+    // Shares per head: enough workgroups for the 256 CUs, at least 128 rows each (what one pass of
+    // the eight waves covers), only with a workspace that holds the partial states.
+    int nsplit = 1;
+    const long heads = (long)B * H;
+    if (workspace && heads < 256) {
+        const int rows = cache_len_dev ? Lmax : cache_len + (k_new ? 1 : 0);
+        while (nsplit < DECODE_ATTN_MAX_SPLIT && heads * nsplit * 2 <= 256 && rows / (nsplit * 2) >= 128) nsplit *= 2;
+        if (workspace_bytes < decode_attention_workspace_bytes(B, H, D)) nsplit = 1;
+    }
     DecodeAttnArgs a;
     a.q = (const half_t*)q;
     a.kn = (const half_t*)k_new;
@@ -228,7 +289,9 @@ hipError_t launch_decode_attention(const void* q, const void* k_new, const void*
     a.cache_len = cache_len;
     a.cache_len_dev = cache_len_dev;
     a.scale = sm_scale;
-    return D == 64 ? launch_d<64>(a, B, st) : launch_d<128>(a, B, st);
+    a.counters = (unsigned*)workspace;
+    a.part = workspace ? (float*)((char*)workspace + decode_attention_counter_bytes(B, H)) : nullptr;
+    return D == 64 ? launch_d<64>(a, B, nsplit, st) : launch_d<128>(a, B, nsplit, st);
 }
 
 }  // namespace sq

@@ -57,7 +57,10 @@ hipError_t launch_lut_attention(const void* q, const void* k, const void* v, voi
 hipError_t launch_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
                                    const void* mask, void* out, int B, int H, int D, int Lmax, long q_bs, long q_hs,
                                    long n_bs, long n_hs, long c_bs, long c_hs, long m_bs, int cache_len,
-                                   const long long* cache_len_dev, float sm_scale, hipStream_t st);
+                                   const long long* cache_len_dev, float sm_scale, void* workspace,
+                                   size_t workspace_bytes, hipStream_t st);
+constexpr int DECODE_ATTN_MAX_SPLIT = 16;
+size_t decode_attention_workspace_bytes(int B, int H, int D);
 
 // sq_layernorm.hip: LayerNorm over the last dimension, fp16 in/out, fp32 statistics; cols % 8 == 0,
 // cols <= 16384.

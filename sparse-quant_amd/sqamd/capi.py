@@ -36,7 +36,9 @@ SIGNATURES = {
     "sq_repack_l2_to_l1": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "sq_convert_2bit_to_4bit": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_clock_probe": (_i, [_vp, _i, _vp]),
-    "sq_decode_attention": (_i, [_vp] * 7 + [_i] * 4 + [ctypes.c_long] * 7 + [_i, _vp, ctypes.c_float, _vp]),
+    "sq_decode_attention": (_i, [_vp] * 7 + [_i] * 4 + [ctypes.c_long] * 7 + [_i, _vp, ctypes.c_float, _vp, ctypes.c_size_t,
+                                 _vp]),
+    "sq_decode_attention_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
     "sq_layernorm": (_i, [_vp, _vp, _vp, _vp, _i, _i, ctypes.c_float, _vp]),
     "sq_lut_attention_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, ctypes.c_float, _i, _vp]),
 }
@@ -194,13 +196,15 @@ def lut_attention(q, k, v, lut, sm_scale, causal, stream=None):
 
 
 def decode_attention(q, k_cache, v_cache, cache_len, sm_scale, k_new=None, v_new=None, mask=None, out=None,
-                     stream=None):
+                     stream=None, ws=None, use_workspace=True):
     """Dense decode attention over an fp16 KV cache, optionally appending the new row.
 
     q [B,H,1,D] or [B,H,D] (any batch/head strides, D contiguous); k_cache, v_cache [B,H,Lmax,D] with
     contiguous rows (a slice cache[:, :, :L] of a bigger buffer is fine); k_new, v_new like q or None;
     cache_len: int, or an int64 device tensor of one element (read by the kernel); mask None or fp16
-    [B,1,1,L] / [B,L] additive.  Returns out fp16 [B, 1, H*D]."""
+    [B,1,1,L] / [B,L] additive.  With fewer than 256 (batch, head) pairs a zeroed workspace (cached per
+    device and stream unless `ws` is given) lets several workgroups share a head.  Returns out fp16
+    [B, 1, H*D]."""
     b, h = q.shape[0], q.shape[1]
     d = q.shape[-1]
     q3 = q.reshape(b, h, d) if q.dim() == 4 else q
@@ -229,11 +233,19 @@ def decode_attention(q, k_cache, v_cache, cache_len, sm_scale, k_new=None, v_new
         len_host, len_dev = 0, _ptr(cache_len)
     else:
         len_host, len_dev = int(cache_len), None
+    if ws is None and use_workspace and b * h < 256:
+        need = lib().sq_decode_attention_workspace_bytes(b, h, d)
+        key = ("attn", str(q.device), (stream or torch.cuda.current_stream()).cuda_stream)
+        ws = _workspaces.get(key)
+        if ws is None or ws.numel() < need:
+            ws = torch.zeros(need, dtype=torch.uint8, device=q.device)
+            _workspaces[key] = ws
     _check(lib().sq_decode_attention(_ptr(q3), _ptr(kn) if kn is not None else None,
                                      _ptr(vn) if vn is not None else None, _ptr(k_cache), _ptr(v_cache),
                                      _ptr(mask) if mask is not None else None, _ptr(out), b, h, d, lmax,
                                      q3.stride(0), q3.stride(1), n_bs, n_hs, k_cache.stride(0), k_cache.stride(1), m_bs,
-                                     len_host, len_dev, float(sm_scale), _stream(stream)), "sq_decode_attention")
+                                     len_host, len_dev, float(sm_scale), _ptr(ws), 0 if ws is None else ws.numel(),
+                                     _stream(stream)), "sq_decode_attention")
     return out
 
 

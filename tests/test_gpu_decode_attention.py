@@ -168,7 +168,7 @@ def test_decode_rejections(capi):
     with pytest.raises(capi.SqError):
         capi.decode_attention(q96, kc96, kc96.clone(), 64, 1.0)  # head dim
     assert L.sq_decode_attention(None, None, None, None, None, None, None, 1, 1, 128, 64, 0, 0, 0, 0, 0, 8192, 0, 1, None,
-                                 1.0, None) == capi.SQ_ERR_NULL_POINTER
+                                 1.0, None, 0, None) == capi.SQ_ERR_NULL_POINTER
 
 
 def test_sparse_attention_entry_point_decode_branch(capi):
@@ -249,3 +249,39 @@ def test_decode_long_cache(capi):
     ref = att.decode_attention_ref(q, k, v, 0.125)
     out = capi.decode_attention(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(), l, 0.125)
     check(out, ref, "long cache")
+
+
+@pytest.mark.parametrize("b,h,d,l", [(1, 32, 128, 640), (1, 4, 64, 5000), (2, 16, 128, 300), (1, 1, 128, 2049), (3, 5, 64, 129)])
+def test_decode_split_over_cache_rows(capi, b, h, d, l):
+    """Few heads: several workgroups share a head through the workspace; same result as one workgroup per
+    head, bit-reproducible, the workspace counters back at zero, append still lands in the cache."""
+    lmax = l + 3
+    q, k, v = make(b, h, l, d, seed=l + h, lmax=lmax)
+    scale = 1.0 / np.sqrt(d)
+    rng = np.random.default_rng(l)
+    kn = rng.normal(size=(b, h, d)).astype(np.float16)
+    vn = rng.normal(size=(b, h, d)).astype(np.float16)
+    k_full, v_full = k.copy(), v.copy()
+    k_full[:, :, l] = kn
+    v_full[:, :, l] = vn
+    ref = att.decode_attention_ref(q, k_full[:, :, :l + 1], v_full[:, :, :l + 1], scale)
+    qt = torch.from_numpy(q).cuda()
+    need = capi.lib().sq_decode_attention_workspace_bytes(b, h, d)
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    outs = []
+    for length in (l, torch.tensor([l], device="cuda")):   # host length: shares sized by l; device length: by Lmax
+        kc, vc = torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda()
+        out = capi.decode_attention(qt, kc, vc, length, scale, k_new=torch.from_numpy(kn).cuda(),
+                                    v_new=torch.from_numpy(vn).cuda(), ws=ws)
+        torch.cuda.synchronize()
+        check(out, ref, "split b=%d h=%d l=%d" % (b, h, l))
+        assert np.array_equal(kc.cpu().numpy(), k_full) and np.array_equal(vc.cpu().numpy(), v_full)
+        assert torch.count_nonzero(ws[:b * h * 4]).item() == 0
+        again = capi.decode_attention(qt, kc, vc, l + 1, scale, ws=ws)
+        assert torch.equal(again, capi.decode_attention(qt, kc, vc, l + 1, scale, ws=ws))
+        outs.append(again)
+    single = capi.decode_attention(qt, torch.from_numpy(k_full).cuda(), torch.from_numpy(v_full).cuda(), l + 1, scale,
+                                   use_workspace=False)
+    check(single, ref, "one workgroup per head")
+    for o in outs:
+        assert (o.float() - single.float()).abs().max().item() <= 2e-3
