@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the W4A16 linear hot path on one MI355X.
 
-Workload (BASELINE.json configs[1], decode regime): the six W4A16 linears of one
+Workload (the headline decode configuration): the six W4A16 linears of one
 OPT-6.7B decoder layer -- q/k/v/out 4096x4096, fc1 4096->16384, fc2 16384->4096 --
 int4 weights in layout L1, group size 128, fp16 activations, M = 1 token.  One
 "step" is one pass over the six linears of one layer, launched back to back on one
@@ -244,7 +244,7 @@ def main():
 
 
 def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10):
-    """TFLOP/s of the M=2048 linears of the same layer (BASELINE.json configs[2]).
+    """TFLOP/s of the M=2048 linears of the same layer (the prefill configuration).
 
     Reported beside each figure: the library's dense fp16 GEMM (torch.matmul, no int4 work at all) on
     the same shape in the same run, and the shader clock the chip sustains while the kernel runs
@@ -319,7 +319,7 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
 
 
 def decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream):
-    """GB/s of the same six linears at decode batches M = 4, 8, 16, 32 (BASELINE.json configs[1]), through
+    """GB/s of the same six linears at decode batches M = 4, 8, 16, 32 (the other batch sizes of the decode configuration), through
     the product dispatch with its workspace (sq_w4a16_gemm_ws), HIP-graph replay over the rotating pool."""
     res = {}
     for m in (4, 8, 16, 32):
@@ -388,7 +388,7 @@ def fused_qkv_leg(torch, capi, m, g, dev, gen, stream, layers, bytes_per_step):
 
 
 def attention_leg(torch, capi, dev):
-    """LUT block-sparse attention (BASELINE configs[3]): batch 8, 16 heads, head dim 64, 64x64 blocks,
+    """LUT block-sparse attention at the BERT-large shape: batch 8, 16 heads, head dim 64, 64x64 blocks,
     ~25 % density with the diagonal block kept, non-causal; flops = 4 * kept blocks * 64 * 64 * D."""
     from sqamd.lut_layout import layout2lut_single_density, synth_layout
     res = {}

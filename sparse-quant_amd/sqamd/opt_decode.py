@@ -1,6 +1,6 @@
 """Random-init OPT-6.7B-shaped decoder with W4A16 linears: the end-to-end harness.
 
-This is the shape generator of BASELINE configuration 5, not a model port: 32
+This is the shape generator of the end-to-end benchmark configuration, not a model port: 32
 pre-LN decoder layers, hidden 4096, 32 heads (head dim 128), FFN 16384 with ReLU,
 vocab 50272, learned positions with OPT's +2 offset, fp16 lm_head; q/k/v/out/fc1/fc2
 are `WALinear` modules (layout L1, group 128) with random packed weights -- the same

@@ -45,7 +45,7 @@ def test_attention_parity(capi, d, causal, s, density):
 
 
 def test_attention_bert_large_shape(capi):
-    # batch 8 x 16 heads x 512 x 64, ~25 % density, non-causal (BASELINE configuration 4)
+    # batch 8 x 16 heads x 512 x 64, ~25 % density, non-causal (the benchmark's BERT-large configuration)
     run_case(capi, 8, 16, 512, 64, 0.25, False, seed=5)
 
 

@@ -117,7 +117,7 @@ def test_gemm_every_tile_height_is_correct(capi, mi):
         check_gemm(capi, m, 264, 704, 64, capi.SQ_ALGO_GEMM | (mi << 8))
 
 
-# BASELINE configuration 1 and 2 shapes (decode) and configuration 3 (prefill).
+# The benchmark's decode shapes (OPT-6.7B linears) and prefill shapes (plus the Llama-2-7B MLP).
 @pytest.mark.parametrize("n,k,g", [(4096, 4096, 64), (4096, 4096, 128), (16384, 4096, 128), (4096, 16384, 128)])
 @pytest.mark.parametrize("m", [1, 4, 8, 16, 32])
 def test_decode_shapes_auto_dispatch(capi, n, k, g, m):
