@@ -285,3 +285,17 @@ def test_decode_split_over_cache_rows(capi, b, h, d, l):
     check(single, ref, "one workgroup per head")
     for o in outs:
         assert (o.float() - single.float()).abs().max().item() <= 2e-3
+
+
+def test_decode_split_with_mask_and_fully_masked_share(capi):
+    # batch 1 x 8 heads, 1024 rows: 8 shares of 128 rows; the mask hides the whole of shares 2 and 5
+    b, h, l, d = 1, 8, 1024, 128
+    q, k, v = make(b, h, l, d, seed=61)
+    mask = np.zeros((b, l), dtype=np.float16)
+    mask[:, 256:384] = -np.inf
+    mask[:, 640:768] = -np.inf
+    mask[:, 5] = -1.5
+    ref = att.decode_attention_ref(q, k, v, 0.09, mask.astype(np.float64))
+    out = capi.decode_attention(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(), l, 0.09,
+                                mask=torch.from_numpy(mask).cuda())
+    check(out, ref, "masked shares")
