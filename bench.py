@@ -313,9 +313,24 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
                 fl2 += 2.0 * m2 * n * k
             other["m%d" % m2] = {"tflops": round(fl2 / t2 / 1e6, 1),
                                  "frac_of_fp16_mfma_peak": round(fl2 / t2 / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)}
+    # What the matrix pipes sustain under the power limit: a loop of nothing but independent
+    # v_mfma_f32_32x32x16_f16 on all CUs (one wave per SIMD), on N(0,1) operands and on zeros.
+    roof = {}
+    with torch.cuda.stream(stream):
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        iters = 20000
+        for name, data in (("normal_operands", torch.randn(5120, device=dev, generator=gen).half()),
+                           ("zero_operands", torch.zeros(5120, device=dev, dtype=torch.float16))):
+            us = timed(lambda: capi.mfma_probe(data, cus, iters, stream=stream))
+            ticks = capi.mfma_probe(data, cus, iters, stream=stream)
+            torch.cuda.synchronize()
+            roof[name] = {"tflops": round(cus * 4 * iters * 16 * 32768.0 / us / 1e6, 1),
+                          "shader_mhz": round(float(ticks.double().median().item()) / us),
+                          "cycles_per_mfma": round(float(ticks.double().median().item()) / (iters * 16), 2)}
     return {"m": m, "other_token_counts": other, "tflops": round(tf, 1), "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
             "dense_fp16_library_tflops": round(tfd, 1), "vs_dense_fp16_library": round(tf / tfd, 3),
-            "nominal_shader_mhz": 2400, "per_linear": res}
+            "nominal_shader_mhz": 2400, "mfma_only_loop": roof,
+            "frac_of_mfma_only_loop": round(tf / roof["normal_operands"]["tflops"], 4), "per_linear": res}
 
 
 def decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream):

@@ -205,6 +205,15 @@ size_t sq_decode_attention_workspace_bytes(int B, int H, int D);
 int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, int rows, int cols, float eps,
                  void* stream);
 
+/* Diagnostic, no counterpart in the reference: `workgroups` workgroups of four waves (one per SIMD)
+ * issue nothing but independent v_mfma_f32_32x32x16_f16, 16 * iters each, on operands taken from
+ * data (5120 fp16 values, 16-byte aligned: the power drawn and so the sustained clock depend on
+ * the operand bits).  out receives one uint64 per workgroup (shader-clock ticks spent in the loop)
+ * followed by 4 scratch bytes, i.e. workgroups * 8 + 4 bytes.  Timed by the caller it gives the
+ * fp16 matrix throughput the part sustains under its power limit (used by bench.py beside the
+ * prefill figures). */
+int sq_mfma_probe(const void* data, void* out, int workgroups, int iters, void* stream);
+
 /* Diagnostic, no counterpart in the reference: a single wave spins for `spins`
  * (1 .. 2^26) dependent multiply-adds and writes three uint64 to out: shader-clock
  * ticks elapsed, ticks of the constant 100 MHz counter elapsed, and a dummy.  Run on

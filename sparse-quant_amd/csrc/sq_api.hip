@@ -269,6 +269,13 @@ int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, in
     return launch_code(sq::launch_layernorm(x, gamma, beta, y, rows, cols, eps, static_cast<hipStream_t>(stream)));
 }
 
+int sq_mfma_probe(const void* data, void* out, int workgroups, int iters, void* stream) {
+    if (!data || !out) return SQ_ERR_NULL_POINTER;
+    if (workgroups <= 0 || workgroups > 65536 || iters <= 0 || iters > (1 << 22)) return SQ_ERR_BAD_SHAPE;
+    if (!aligned16(data)) return SQ_ERR_MISALIGNED;
+    return launch_code(sq::launch_mfma_probe(data, out, workgroups, iters, static_cast<hipStream_t>(stream)));
+}
+
 int sq_clock_probe(void* out, int spins, void* stream) {
     if (!out) return SQ_ERR_NULL_POINTER;
     if (spins <= 0 || spins > (1 << 26)) return SQ_ERR_BAD_SHAPE;

@@ -52,6 +52,9 @@ hipError_t launch_lut_attention(const void* q, const void* k, const void* v, voi
                                 int lut_elem_bytes, int Z, int H, int S, int D, int nnz, float sm_scale, int causal,
                                 hipStream_t st);
 
+// sq_repack.hip: diagnostic loop of independent matrix instructions (see sq_mfma_probe).
+hipError_t launch_mfma_probe(const void* data, void* out, int workgroups, int iters, hipStream_t st);
+
 // sq_decode_attn.hip: dense decode attention over an fp16 KV cache (one query row per sequence),
 // optionally appending the new key/value row.  Strides in elements.
 hipError_t launch_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,

@@ -184,6 +184,52 @@ __global__ void clock_probe_kernel(unsigned long long* out, int spins) {
     }
 }
 
+// Diagnostic: nothing but independent v_mfma_f32_32x32x16_f16, one wave per SIMD (256 threads per
+// workgroup, `workgroups` of them), operands taken from `data` (64 * 80 fp16 values of the caller's
+// choosing: the power the matrix pipes draw, and with it the clock the chip sustains, depends on the
+// operand bits).  out[w] = shader-clock ticks wave 0 of workgroup w spent in the loop.  The caller
+// times the launch: workgroups * 4 * iters * 16 matrix instructions of 32768 flop each.
+__global__ __launch_bounds__(256) void mfma_probe_kernel(const half_t* __restrict__ data, unsigned long long* out,
+                                                         float* sink, int iters) {
+    const int lane = threadIdx.x & 63;
+    half8_t a[8], b[2];
+#pragma unroll
+    for (int i = 0; i < 8; i++) a[i] = *(const half8_t*)(data + (lane * 10 + i) * 8);
+#pragma unroll
+    for (int i = 0; i < 2; i++) b[i] = *(const half8_t*)(data + (lane * 10 + 8 + i) * 8);
+    float16_t acc[8][2];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+    const unsigned long long c0 = __builtin_readcyclecounter();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    const unsigned long long c1 = __builtin_readcyclecounter();
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) s += acc[i][j][v];
+    if (s == 12345.678f) sink[0] = s;  // keeps the accumulators alive
+    if (threadIdx.x == 0) out[blockIdx.x] = c1 - c0;
+}
+
+hipError_t launch_mfma_probe(const void* data, void* out, int workgroups, int iters, hipStream_t st) {
+    float* sink = (float*)((unsigned long long*)out + workgroups);
+    hipLaunchKernelGGL(mfma_probe_kernel, dim3(workgroups), dim3(256), 0, st, (const half_t*)data,
+                       (unsigned long long*)out, sink, iters);
+    return hipGetLastError();
+}
+
 hipError_t launch_clock_probe(void* out, int spins, hipStream_t st) {
     hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, st, (unsigned long long*)out, spins);
     return hipGetLastError();

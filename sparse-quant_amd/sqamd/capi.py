@@ -36,6 +36,7 @@ SIGNATURES = {
     "sq_repack_l2_to_l1": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "sq_convert_2bit_to_4bit": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_clock_probe": (_i, [_vp, _i, _vp]),
+    "sq_mfma_probe": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_decode_attention": (_i, [_vp] * 7 + [_i] * 4 + [ctypes.c_long] * 7 + [_i, _vp, ctypes.c_float, _vp, ctypes.c_size_t,
                                  _vp]),
     "sq_decode_attention_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
@@ -257,6 +258,13 @@ def layernorm(x, gamma, beta, eps=1e-5, out=None, stream=None):
     _check(lib().sq_layernorm(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(out), x.numel() // cols, cols, float(eps),
                               _stream(stream)), "sq_layernorm")
     return out
+
+
+def mfma_probe(data, workgroups, iters, stream=None):
+    """Launch the matrix-instruction loop; returns the int64 tensor of per-workgroup shader ticks."""
+    out = torch.zeros(workgroups + 1, dtype=torch.int64, device=data.device)
+    _check(lib().sq_mfma_probe(_ptr(data), _ptr(out), int(workgroups), int(iters), _stream(stream)), "sq_mfma_probe")
+    return out[:workgroups]
 
 
 def clock_probe(spins=400000, stream=None):

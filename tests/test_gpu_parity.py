@@ -611,3 +611,13 @@ def test_gemm_split_k_every_tile_height(capi, mi, ksplit):
         assert np.max(np.abs(y1.float().cpu().numpy() - y_ref)) <= TOL * np.max(np.abs(y_ref))
         assert torch.count_nonzero(ws[:65536]).item() == 0
         assert torch.equal(y1, capi.gemm_ws(x, d["w_dev"], d["zs_dev"], n, k, g, algo=algo, ws=ws))
+
+
+def test_mfma_probe_reports_one_instruction_per_32_cycles(capi):
+    data = torch.randn(5120, device=DEV).half()
+    ticks = capi.mfma_probe(data, 4, 2000)
+    torch.cuda.synchronize()
+    per = ticks.double().median().item() / (2000 * 16)
+    assert 31.0 <= per <= 40.0, per
+    with pytest.raises(capi.SqError):
+        capi.mfma_probe(data, 0, 10)
