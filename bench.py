@@ -187,6 +187,36 @@ def main():
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         assert done == steps
+        # The same step with the arithmetic taken away: sq_read_probe streams each weight with the GEMV's
+        # own grid and access pattern and only folds the bits.  What it needs per step is the floor that
+        # six dependent launches of these sizes leave to any kernel on this part.
+        probe_out = torch.zeros(4096, dtype=torch.int32, device=dev)
+        probe = lib.sq_read_probe
+        floor_us = None
+        if m == 1 and not args.no_graph:
+            def probe_layer(i):
+                for a in calls[i % len(calls)]:
+                    rc = probe(a[1], a[2], vp(probe_out.data_ptr()), a[5], a[6], a[7], st)
+                    if rc != 0:
+                        raise RuntimeError("sq_read_probe failed: " + capi.strerror(rc))
+            for i in range(len(calls)):
+                probe_layer(i)
+            stream.synchronize()
+            pgraph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(pgraph, stream=stream):
+                for i in range(len(calls)):
+                    probe_layer(i)
+            reps = max(1, steps // per_replay)
+            for _ in range(max(1, reps // 10)):
+                pgraph.replay()
+            p0 = torch.cuda.Event(enable_timing=True)
+            p1 = torch.cuda.Event(enable_timing=True)
+            p0.record(stream)
+            for _ in range(reps):
+                pgraph.replay()
+            p1.record(stream)
+            stream.synchronize()
+            floor_us = p0.elapsed_time(p1) * 1e3 / (reps * per_replay)
     wall_ms = (t1 - t0) * 1e3
     gpu_ms = e0.elapsed_time(e1)
     ms_per_step = wall_ms / steps
@@ -216,6 +246,14 @@ def main():
                      "kernel": "sq::gemv2_kernel (decode GEMV)", "avg_launch_us": round(launch_us, 3),
                      "bytes_per_launch": bytes_per_step // launches_per_step},
     }
+
+    if floor_us is not None:
+        out["read_only_floor"] = {
+            "what": "the same six launches per step through sq_read_probe (weights and zeros_scales streamed with "
+                    "the GEMV's grid and access pattern, no arithmetic, no activations, no output)",
+            "us_per_step": round(floor_us, 2), "gbs": round(bytes_per_step / floor_us / 1e3, 1),
+            "frac_of_hbm_peak": round(bytes_per_step / floor_us / 1e3 / HBM_PEAK_GBS, 4),
+            "value_over_floor": round(floor_us / (ms_per_step * 1e3), 4)}
 
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)

@@ -205,6 +205,13 @@ size_t sq_decode_attention_workspace_bytes(int B, int H, int D);
 int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, int rows, int cols, float eps,
                  void* stream);
 
+/* Diagnostic, no counterpart in the reference: reads an L1 weight and its zeros_scales exactly as the
+ * single-token GEMV does (same grid, lane -> address mapping and loads in flight) and does nothing
+ * else; its duration is what the memory system charges for the weight stream of one launch.  out:
+ * at least ceil(N / 8) uint32 (practically never written).  Used by bench.py to report the read-only
+ * floor of the decode step beside the measured figure. */
+int sq_read_probe(const void* w, const void* zs, void* out, int N, int K, int group_size, void* stream);
+
 /* Diagnostic, no counterpart in the reference: `workgroups` workgroups of four waves (one per SIMD)
  * issue nothing but independent v_mfma_f32_32x32x16_f16, 16 * iters each, on operands taken from
  * data (5120 fp16 values, 16-byte aligned: the power drawn and so the sustained clock depend on

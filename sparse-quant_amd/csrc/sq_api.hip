@@ -269,6 +269,14 @@ int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, in
     return launch_code(sq::launch_layernorm(x, gamma, beta, y, rows, cols, eps, static_cast<hipStream_t>(stream)));
 }
 
+int sq_read_probe(const void* w, const void* zs, void* out, int N, int K, int group_size, void* stream) {
+    const int rc = check_weight(N, K, group_size, SQ_LAYOUT_L1);
+    if (rc != SQ_OK) return rc;
+    if (!w || !zs || !out) return SQ_ERR_NULL_POINTER;
+    if (!aligned16(w) || !aligned16(zs)) return SQ_ERR_MISALIGNED;
+    return launch_code(sq::launch_read_probe(w, zs, out, N, K, group_size, static_cast<hipStream_t>(stream)));
+}
+
 int sq_mfma_probe(const void* data, void* out, int workgroups, int iters, void* stream) {
     if (!data || !out) return SQ_ERR_NULL_POINTER;
     if (workgroups <= 0 || workgroups > 65536 || iters <= 0 || iters > (1 << 22)) return SQ_ERR_BAD_SHAPE;

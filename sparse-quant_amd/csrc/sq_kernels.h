@@ -52,6 +52,9 @@ hipError_t launch_lut_attention(const void* q, const void* k, const void* v, voi
                                 int lut_elem_bytes, int Z, int H, int S, int D, int nnz, float sm_scale, int causal,
                                 hipStream_t st);
 
+// sq_repack.hip: diagnostic read of an L1 weight with the GEMV's access pattern (see sq_read_probe).
+hipError_t launch_read_probe(const void* w, const void* zs, void* out, int N, int K, int g, hipStream_t st);
+
 // sq_repack.hip: diagnostic loop of independent matrix instructions (see sq_mfma_probe).
 hipError_t launch_mfma_probe(const void* data, void* out, int workgroups, int iters, hipStream_t st);
 

@@ -37,6 +37,7 @@ SIGNATURES = {
     "sq_convert_2bit_to_4bit": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_clock_probe": (_i, [_vp, _i, _vp]),
     "sq_mfma_probe": (_i, [_vp, _vp, _i, _i, _vp]),
+    "sq_read_probe": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sq_decode_attention": (_i, [_vp] * 7 + [_i] * 4 + [ctypes.c_long] * 7 + [_i, _vp, ctypes.c_float, _vp, ctypes.c_size_t,
                                  _vp]),
     "sq_decode_attention_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),

@@ -621,3 +621,15 @@ def test_mfma_probe_reports_one_instruction_per_32_cycles(capi):
     assert 31.0 <= per <= 40.0, per
     with pytest.raises(capi.SqError):
         capi.mfma_probe(data, 0, 10)
+
+
+def test_read_probe_runs_on_every_reference_shape(capi):
+    out = torch.zeros(4096, dtype=torch.int32, device=DEV)
+    for n, k in ((4096, 4096), (16384, 4096), (4096, 16384), (11008, 4096), (200, 1056)):
+        g = 128 if k % 128 == 0 else 32
+        w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=DEV)
+        zs = torch.zeros((n, 2 * (k // g)), dtype=torch.float16, device=DEV)
+        rc = capi.lib().sq_read_probe(w.data_ptr(), zs.data_ptr(), out.data_ptr(), n, k, g, None)
+        assert rc == 0
+    torch.cuda.synchronize()
+    assert capi.lib().sq_read_probe(None, None, out.data_ptr(), 4096, 4096, 128, None) == capi.SQ_ERR_NULL_POINTER
