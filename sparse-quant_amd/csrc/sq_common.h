@@ -109,6 +109,16 @@ __device__ __forceinline__ u32x4_t quad_bcast(u32x4_t v) {
     return r;
 }
 
+// Word -> 8 fp16 with mixed bias and no shift: 1024 + q at positions 0, 1, 4, 5 (the low nibbles
+// land in mantissa bits 0..3 of 0x6400 = 1024, where ulp = 1) and 64 + q at positions 2, 3, 6, 7.
+// Five operations instead of seven; the consumer removes the extra 960 on the low positions.
+__device__ __forceinline__ half8_t unpack8_mixed(uint32_t w, const NibbleMasks& nm) {
+    const uint32_t t = w >> 8;
+    u32x4_t r = {(w & nm.lo) | 0x64006400u, (w & nm.hi) | 0x54005400u, (t & nm.lo) | 0x64006400u,
+                 (t & nm.hi) | 0x54005400u};
+    return bit_cast<half8_t>(r);
+}
+
 __device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
 
 // What happens to an fp32 accumulator on its way to Y[m, n]: + bias[n], activation,

@@ -20,10 +20,13 @@
 //
 // Arithmetic modes (both accumulate in fp32):
 //   exact : B = fp16((q - z) * s), bit-identical to the reference's W_hat.
-//   fixup : B = 64 + q (bit pattern only); per run of 32 k the lane adds
-//           s * (sum x*(64+q) - (64+z) * sum x): zero and scale are applied once per
-//           run in fp32 instead of once per weight in fp16 (with more than 4 tokens the
-//           zero-point term comes from a second matrix instruction instead of staged sums).
+//   fixup : B = bias + q (bit pattern only); per run of 32 k the lane adds
+//           s * (sum x*(bias+q) - sum x*bias - z * sum x): zero and scale are applied once
+//           per run in fp32 instead of once per weight in fp16.  Up to 4 tokens: the unpack
+//           without shifts (bias 1024 on four of every eight positions, 64 on the others,
+//           5 operations per word instead of 7) with both sums staged beside the activations;
+//           more tokens: bias 64 everywhere and the zero-point term from a second matrix
+//           instruction.
 // (replaces w4a16_bs1_kernel / w4a16_bs2_kernel, reference:
 // quantization/muxi/backend/w4a16_gemm.cuh:14-151,153-326)
 #include "sq_common.h"
@@ -48,7 +51,8 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
     constexpr int STAGE_PER_THREAD = (STAGE_TOTAL + NT - 1) / NT;
 
     __shared__ __attribute__((aligned(16))) uint8_t xbuf[KS][MROWS * PITCH];
-    __shared__ __attribute__((aligned(16))) float xsum[KS][S * 16][MROWS];
+    // per run of 32 k and token: {sum of x, 960 * sum of x over the positions unpacked with bias 1024}
+    __shared__ __attribute__((aligned(16))) float xsum[KS][S * 16][MROWS][2];
     __shared__ float red[KS][NR][MROWS][4];
 
     const NibbleMasks nm = nibble_masks();
@@ -111,11 +115,14 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
             if (idx < STAGE_TOTAL) *(u32x4_t*)(&xbuf[q][m * PITCH + w8 * 16]) = xr[p];
             if (FIXUP && !ZMFMA) {
                 const half8_t h = bit_cast<half8_t>(xr[p]);
-                float sum = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; e++) sum += (float)h[e];
+                float lo = ((float)h[0] + (float)h[1]) + ((float)h[4] + (float)h[5]);
+                float sum = lo + (((float)h[2] + (float)h[3]) + ((float)h[6] + (float)h[7]));
                 sum = quad_sum(sum);
-                if ((tid & 3) == 0 && idx < STAGE_TOTAL) xsum[q][w8 >> 2][m] = sum;
+                lo = quad_sum(lo);
+                if ((tid & 3) == 0 && idx < STAGE_TOTAL) {
+                    xsum[q][w8 >> 2][m][0] = sum;
+                    xsum[q][w8 >> 2][m][1] = 960.f * lo;
+                }
             }
         }
         __syncthreads();
@@ -151,7 +158,7 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
                 const half4_t nzb = {nz, nz, nz, nz};
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    const half8_t wv = unpack8_raw(wq[s][t], nm);
+                    const half8_t wv = ZMFMA ? unpack8_raw(wq[s][t], nm) : unpack8_mixed(wq[s][t], nm);
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
                         tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, wv.lo, tmp[mt], 0, 0, 0);
@@ -164,13 +171,14 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
                 }
                 const float zf = (float)p.x;
                 const float sf = (float)p.y;
-                const float* xs = &xsum[wq_][16 * s + b][0];
+                const float* xs = &xsum[wq_][16 * s + b][0][0];
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++)
 #pragma unroll
                     for (int j = 0; j < 4; j++)
                         if (4 * mt + j < MROWS)
-                            acc[mt][j] += ZMFMA ? sf * tmp[mt][j] : sf * (tmp[mt][j] - zf * xs[4 * mt + j]);
+                            acc[mt][j] += ZMFMA ? sf * tmp[mt][j]
+                                                : sf * ((tmp[mt][j] - xs[2 * (4 * mt + j) + 1]) - zf * xs[2 * (4 * mt + j)]);
             }
         }
     }
