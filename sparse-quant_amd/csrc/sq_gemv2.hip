@@ -24,9 +24,9 @@
 //           s * (sum x*(bias+q) - sum x*bias - z * sum x): zero and scale are applied once
 //           per run in fp32 instead of once per weight in fp16.  Up to 4 tokens: the unpack
 //           without shifts (bias 1024 on four of every eight positions, 64 on the others,
-//           5 operations per word instead of 7) with both sums staged beside the activations;
-//           more tokens: bias 64 everywhere and the zero-point term from a second matrix
-//           instruction.
+//           5 operations per word instead of 7); the bias terms come from two sums staged
+//           beside the activations or, with more than 4 tokens, from a second matrix
+//           instruction whose B operand is -(bias + z).
 // (replaces w4a16_bs1_kernel / w4a16_bs2_kernel, reference:
 // quantization/muxi/backend/w4a16_gemm.cuh:14-151,153-326)
 #include "sq_common.h"
@@ -154,11 +154,14 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
                 float4_t tmp[MT];
 #pragma unroll
                 for (int mt = 0; mt < MT; mt++) tmp[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                // zero-point operand for the mixed-bias unpack: -(1024 + z) where the weight carries
+                // bias 1024 (positions 0, 1 of each four), -(64 + z) elsewhere; both exact in fp16
                 const half_t nz = -p.x;
-                const half4_t nzb = {nz, nz, nz, nz};
+                const half_t nz1024 = nz - (half_t)960.f;
+                const half4_t nzb = {nz1024, nz1024, nz, nz};
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    const half8_t wv = ZMFMA ? unpack8_raw(wq[s][t], nm) : unpack8_mixed(wq[s][t], nm);
+                    const half8_t wv = unpack8_mixed(wq[s][t], nm);
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
                         tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, wv.lo, tmp[mt], 0, 0, 0);
