@@ -191,7 +191,7 @@ def main():
         # own grid and access pattern and only folds the bits.  What it needs per step is the floor that
         # six dependent launches of these sizes leave to any kernel on this part.
         probe_out = torch.zeros(4096, dtype=torch.int32, device=dev)
-        probe = lib.sq_read_probe
+        probe = capi.probes().sq_read_probe
         floor_us = None
         if m == 1 and not args.no_graph:
             def probe_layer(i):

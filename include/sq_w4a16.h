@@ -153,8 +153,10 @@ int sq_convert_2bit_to_4bit(const void* src, void* dst, int N, int K, void* stre
  * blocks lut[h][m/64][0..nnz) of (q k^T * sm_scale) (optionally causal) times v.
  * q, k, v, out fp16 [Z, H, S, D] contiguous, D in {64, 128}; lut int32 or int64
  * (lut_elem_bytes 4 or 8) [H, ceil(S/64), nnz], key-block indices of 64 keys; an
- * entry equal to its predecessor in the row is padding; at most ceil(S/64) entries
- * of a row are visited.  Replaces sparse_attention_prefill (reference:
+ * entry equal to its predecessor in the row is padding (a block named again after a
+ * different one is attended, and weighted, again); at most ceil(S/64) entries of a row
+ * are visited; entries outside [0, ceil(S/64)) select nothing.  A query row without any
+ * visible key gives NaN, as in the reference.  Replaces sparse_attention_prefill (reference:
  * sparse-attention/nvidia/playground/kernels/block_sparse_attention_lut.py:22-243;
  * sparse-attention/muxi/playground/kernels/csrc/src/block_sparse_attention_lut.cu:49-55). */
 int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out, const void* lut,
@@ -183,7 +185,8 @@ int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out,
  *              device (int64) and overrides cache_len -- read by the kernel, so a captured HIP
  *              graph follows a growing cache; the kernel clamps it to the cache size.
  *   workspace  NULL, or sq_decode_attention_workspace_bytes(B, H, D) bytes, 16-byte aligned, its
- *              first B*H*4 bytes zero before the first call (every call leaves them zero).  The kernel
+ *              first 1024 bytes (256 counters, a fixed region whatever B*H is) zero before the first call
+ *              (every call leaves them zero), so one workspace serves calls with different B*H.  The kernel
  *              runs one workgroup per (batch, head); with fewer than 256 of them and a workspace
  *              the cache rows of a head are shared among up to 16 workgroups whose partial
  *              softmax states meet in the workspace (batch 1, 32 heads, 640 rows: 4 workgroups
@@ -204,30 +207,6 @@ size_t sq_decode_attention_workspace_bytes(int B, int H, int D);
  * (reference: test/nvidia/module/opt/modeling_opt_ours.py:500-507,561-562,603-604). */
 int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, int rows, int cols, float eps,
                  void* stream);
-
-/* Diagnostic, no counterpart in the reference: reads an L1 weight and its zeros_scales exactly as the
- * single-token GEMV does (same grid, lane -> address mapping and loads in flight) and does nothing
- * else; its duration is what the memory system charges for the weight stream of one launch.  out:
- * at least ceil(N / 8) uint32 (practically never written).  Used by bench.py to report the read-only
- * floor of the decode step beside the measured figure. */
-int sq_read_probe(const void* w, const void* zs, void* out, int N, int K, int group_size, void* stream);
-
-/* Diagnostic, no counterpart in the reference: `workgroups` workgroups of four waves (one per SIMD)
- * issue nothing but independent v_mfma_f32_32x32x16_f16, 16 * iters each, on operands taken from
- * data (5120 fp16 values, 16-byte aligned: the power drawn and so the sustained clock depend on
- * the operand bits).  out receives one uint64 per workgroup (shader-clock ticks spent in the loop)
- * followed by 4 scratch bytes, i.e. workgroups * 8 + 4 bytes.  Timed by the caller it gives the
- * fp16 matrix throughput the part sustains under its power limit (used by bench.py beside the
- * prefill figures). */
-int sq_mfma_probe(const void* data, void* out, int workgroups, int iters, void* stream);
-
-/* Diagnostic, no counterpart in the reference: a single wave spins for `spins`
- * (1 .. 2^26) dependent multiply-adds and writes three uint64 to out: shader-clock
- * ticks elapsed, ticks of the constant 100 MHz counter elapsed, and a dummy.  Run on
- * a second stream beside a kernel it gives the clock the chip sustains under that
- * kernel's load (matrix-heavy kernels run power-limited, well below the nominal
- * clock that published peak rates assume). */
-int sq_clock_probe(void* out, int spins, void* stream);
 
 #ifdef __cplusplus
 }

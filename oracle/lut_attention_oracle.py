@@ -12,7 +12,10 @@ detail; the oracle computes the same quantity in float64.
 Pinning (tests/test_attention_oracle.py): hand-written LUT known answer; a two-key
 softmax with weights known in closed form; single-visible-key rows return that V
 row exactly; constant V returns the constant; an all-blocks LUT equals unmasked
-softmax attention computed with a different formulation (per-row loops).
+softmax attention computed with a different formulation (per-row loops); a row that names
+a block again after a different one equals textbook attention over the concatenation of the
+visited blocks' keys and values (the block counted twice), while an immediate repeat counts once.
+A row without any visible key is 0/0 = NaN here; the reference's running sums give NaN as well.
 decode_attention_ref restates the decode branch of the same entry point (:272-300): dense
 attention of one query row over the whole cache, softmax in fp32, probabilities cast to fp16
 before the product with v.  Pinning: equal keys give the mean of v; a dominating key returns
@@ -46,18 +49,31 @@ def layout_to_lut(layout):
     return lut
 
 
-def lut_to_layout(lut, nb):
-    """int [H, nb, nnz] -> bool [H, nb, nb]; at most nb entries of a row are read."""
+def lut_to_counts(lut, nb):
+    """int [H, nb, nnz] -> int64 [H, nb, nb]: how often the kernel's loop visits key block j for
+    query block i.  At most nb entries of a row are read and an entry is skipped only when it
+    equals its predecessor in the row (block_sparse_attention_lut.py:96,134,163: last_nnz_id
+    starts at -1 and p is multiplied by last_nnz_id != present_nnz_id), so a block that shows up
+    again after a different one is visited, and weighted, again.  Entries outside [0, nb) select
+    keys beyond the sequence, which the kernel masks completely."""
     lut = np.asarray(lut)
     h = lut.shape[0]
-    layout = np.zeros((h, nb, nb), dtype=bool)
+    counts = np.zeros((h, nb, nb), dtype=np.int64)
     visit = min(lut.shape[-1], nb)
     for a in range(h):
         for i in range(nb):
+            last = -1
             for j in lut[a, i, :visit]:
-                if 0 <= j < nb:
-                    layout[a, i, j] = True
-    return layout
+                j = int(j)
+                if j != last and 0 <= j < nb:
+                    counts[a, i, j] += 1
+                last = j
+    return counts
+
+
+def lut_to_layout(lut, nb):
+    """int [H, nb, nnz] -> bool [H, nb, nb]: the key blocks a row visits at least once."""
+    return lut_to_counts(lut, nb) > 0
 
 
 def synth_layout(h, nb, density, causal, seed=0):
@@ -83,16 +99,17 @@ def attention_ref(q, k, v, lut, sm_scale, causal):
     v = np.asarray(v, dtype=np.float64)
     z, h, s, d = q.shape
     nb = (s + BLOCK - 1) // BLOCK
-    layout = lut_to_layout(lut, nb)
-    mask = np.repeat(np.repeat(layout, BLOCK, axis=1), BLOCK, axis=2)[:, :s, :s]
+    counts = lut_to_counts(lut, nb)
+    weight = np.repeat(np.repeat(counts, BLOCK, axis=1), BLOCK, axis=2)[:, :s, :s].astype(np.float64)
     if causal:
-        mask = mask & np.tril(np.ones((s, s), dtype=bool))[None]
+        weight = weight * np.tril(np.ones((s, s)))[None]
+    mask = weight > 0
     out = np.empty_like(q)
     for b in range(z):
         scores = np.einsum("hmd,hnd->hmn", q[b], k[b]) * sm_scale
         scores = np.where(mask, scores, -np.inf)
         scores -= scores.max(axis=-1, keepdims=True)
-        p = np.exp(scores)
+        p = np.exp(scores) * weight  # a key block visited c times enters the running sums c times
         p /= p.sum(axis=-1, keepdims=True)
         out[b] = np.einsum("hmn,hnd->hmd", p, v[b])
     return out

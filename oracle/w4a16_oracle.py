@@ -258,21 +258,24 @@ def gemm_l2(x, w, zs, g, in_features, out_features):
 # Either side of the path: quantizer and 2-bit expansion
 # ---------------------------------------------------------------------------
 
-def rtn_quantize(w, n_bit, g):
+def rtn_quantize(w, n_bit, g, dtype=np.float32):
     """Round-to-nearest asymmetric group quantization.
 
     Follows test/muxi/utils/quant_funcs.py:96-114: per group of g along the
     last axis, s = clamp(max - min, 1e-5) / (2^b - 1), z = clamp(-round(min /
     s), 0, 2^b - 1), q = clamp(round(w / s) + z, 0, 2^b - 1); rounding is
-    half-to-even.  Returns (q uint8 [N,K], s fp32 [N,K/g], z fp32 [N,K/g]).
+    half-to-even.  Every operation is rounded to `dtype`: the reference computes in
+    the dtype of the weight it is handed (np.float16 for the fp16 models it packs).
+    Returns (q uint8 [N,K], s [N,K/g], z [N,K/g]) with s, z in `dtype`.
     """
-    w = np.asarray(w, dtype=np.float32)
+    ft = np.dtype(dtype).type
+    w = np.asarray(w, dtype=dtype)
     n, k = w.shape
     wg = w.reshape(-1, g)
     hi = wg.max(axis=1, keepdims=True)
     lo = wg.min(axis=1, keepdims=True)
-    qmax = np.float32(2 ** n_bit - 1)
-    s = np.maximum(hi - lo, np.float32(1e-5)) / qmax
+    qmax = ft(2 ** n_bit - 1)
+    s = np.maximum(hi - lo, ft(1e-5)) / qmax
     z = np.clip(-np.rint(lo / s), 0, qmax)
     q = np.clip(np.rint(wg / s) + z, 0, qmax)
     return (q.reshape(n, k).astype(np.uint8), s.reshape(n, k // g), z.reshape(n, k // g))

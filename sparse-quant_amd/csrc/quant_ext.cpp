@@ -14,6 +14,7 @@
 
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
+#include <hip/hip_runtime_api.h>
 
 #include <map>
 #include <mutex>
@@ -51,41 +52,70 @@ int layout_of(const at::Tensor& W) {
     return 0;
 }
 
-// Layout-L2 weights are converted to L1 once and kept while the source tensor
-// lives.  The key is the source's data pointer; an entry is valid only while the
-// source storage is alive (weak reference) and unmodified (version counter).
+// Layout-L2 weights are converted to L1 once and kept while the source tensors
+// live.  The key is the weight's data pointer; an entry is valid only while the
+// storages of both sources (weight and zeros_scales) are alive (weak references),
+// unmodified (version counters) and the same zeros_scales tensor is passed again.
+// The conversion is enqueued on the stream of the first call; an event recorded
+// behind it orders a later call on another stream after it.
 struct RepackEntry {
-    c10::weak_intrusive_ptr<c10::StorageImpl> src_storage;
-    int64_t version;
+    c10::weak_intrusive_ptr<c10::StorageImpl> src_storage, zs_storage;
+    int64_t version, zs_version;
+    const void* zs_ptr;
+    void* stream;
+    hipEvent_t done;
     at::Tensor w_l1, zs_l1;
 };
 std::mutex g_cache_mutex;
 std::unordered_map<const void*, RepackEntry> g_repack_cache;
 
+void drop_entry(RepackEntry& e) {
+    if (e.done) (void)hipEventDestroy(e.done);
+    e.done = nullptr;
+}
+
 void sweep_cache_locked() {
     for (auto it = g_repack_cache.begin(); it != g_repack_cache.end();) {
-        if (it->second.src_storage.expired())
+        if (it->second.src_storage.expired() || it->second.zs_storage.expired()) {
+            drop_entry(it->second);
             it = g_repack_cache.erase(it);
-        else
+        } else {
             ++it;
+        }
     }
 }
 
 std::pair<at::Tensor, at::Tensor> l1_view_of_l2(const at::Tensor& W, const at::Tensor& ZS, int N, int K, int g) {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     const void* key = W.data_ptr();
+    void* stream = current_stream(W);
     auto it = g_repack_cache.find(key);
-    if (it != g_repack_cache.end() && !it->second.src_storage.expired() &&
-        it->second.version == W._version() && it->second.w_l1.size(0) == N && it->second.w_l1.size(1) == K / 2)
-        return {it->second.w_l1, it->second.zs_l1};
+    if (it != g_repack_cache.end()) {
+        RepackEntry& e = it->second;
+        if (!e.src_storage.expired() && !e.zs_storage.expired() && e.version == (int64_t)W._version() &&
+            e.zs_ptr == ZS.data_ptr() && e.zs_version == (int64_t)ZS._version() && e.w_l1.size(0) == N &&
+            e.w_l1.size(1) == K / 2 && e.zs_l1.size(1) == 2 * (K / g)) {
+            if (stream != e.stream && e.done) {
+                if (hipStreamWaitEvent(static_cast<hipStream_t>(stream), e.done, 0) != hipSuccess)
+                    throw std::runtime_error("repack: hipStreamWaitEvent failed");
+            }
+            return {e.w_l1, e.zs_l1};
+        }
+        drop_entry(e);
+        g_repack_cache.erase(it);
+    }
     sweep_cache_locked();
     at::Tensor w1 = torch::empty({N, K / 2}, W.options().dtype(at::kByte));
     at::Tensor zs1 = torch::empty({N, 2 * (K / g)}, ZS.options());
-    raise_if_error(sq_repack_l2_to_l1(W.data_ptr(), ZS.data_ptr(), w1.data_ptr(), zs1.data_ptr(), N, K, g,
-                                      current_stream(W)),
+    raise_if_error(sq_repack_l2_to_l1(W.data_ptr(), ZS.data_ptr(), w1.data_ptr(), zs1.data_ptr(), N, K, g, stream),
                    "repack");
-    RepackEntry e{c10::weak_intrusive_ptr<c10::StorageImpl>(W.storage().getWeakStorageImpl()), W._version(), w1, zs1};
-    g_repack_cache.erase(key);
+    hipEvent_t done = nullptr;
+    if (hipEventCreateWithFlags(&done, hipEventDisableTiming) != hipSuccess ||
+        hipEventRecord(done, static_cast<hipStream_t>(stream)) != hipSuccess)
+        throw std::runtime_error("repack: could not record the completion event");
+    RepackEntry e{c10::weak_intrusive_ptr<c10::StorageImpl>(W.storage().getWeakStorageImpl()),
+                  c10::weak_intrusive_ptr<c10::StorageImpl>(ZS.storage().getWeakStorageImpl()),
+                  (int64_t)W._version(), (int64_t)ZS._version(), ZS.data_ptr(), stream, done, w1, zs1};
     g_repack_cache.emplace(key, std::move(e));
     return {w1, zs1};
 }
@@ -313,6 +343,7 @@ at::Tensor convert_2bit_to_4bit(at::Tensor qweight_2bit) {
 
 void clear_repack_cache() {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
+    for (auto& kv : g_repack_cache) drop_entry(kv.second);
     g_repack_cache.clear();
 }
 

@@ -86,9 +86,6 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
         case SQ_ALGO_GEMV:
         case SQ_ALGO_GEMV_FIXUP:
             if (M > 8) return SQ_ERR_BAD_ALGO;
-            if (tune & 0x8000)
-                return launch_code(sq::launch_gemv_tuned(x, w, zs, y, M, N, K, group_size,
-                                                         kernel == SQ_ALGO_GEMV_FIXUP, tune & 0x7FFF, epi, st));
             return launch_code(sq::launch_gemv2_tuned(x, w, zs, y, M, N, K, group_size,
                                                       kernel == SQ_ALGO_GEMV_FIXUP, tune, epi, st));
         case SQ_ALGO_SKINNY:
@@ -267,27 +264,6 @@ int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, in
     if (!aligned16(x) || !aligned16(y) || (gamma && !aligned16(gamma)) || (beta && !aligned16(beta)))
         return SQ_ERR_MISALIGNED;
     return launch_code(sq::launch_layernorm(x, gamma, beta, y, rows, cols, eps, static_cast<hipStream_t>(stream)));
-}
-
-int sq_read_probe(const void* w, const void* zs, void* out, int N, int K, int group_size, void* stream) {
-    const int rc = check_weight(N, K, group_size, SQ_LAYOUT_L1);
-    if (rc != SQ_OK) return rc;
-    if (!w || !zs || !out) return SQ_ERR_NULL_POINTER;
-    if (!aligned16(w) || !aligned16(zs)) return SQ_ERR_MISALIGNED;
-    return launch_code(sq::launch_read_probe(w, zs, out, N, K, group_size, static_cast<hipStream_t>(stream)));
-}
-
-int sq_mfma_probe(const void* data, void* out, int workgroups, int iters, void* stream) {
-    if (!data || !out) return SQ_ERR_NULL_POINTER;
-    if (workgroups <= 0 || workgroups > 65536 || iters <= 0 || iters > (1 << 22)) return SQ_ERR_BAD_SHAPE;
-    if (!aligned16(data)) return SQ_ERR_MISALIGNED;
-    return launch_code(sq::launch_mfma_probe(data, out, workgroups, iters, static_cast<hipStream_t>(stream)));
-}
-
-int sq_clock_probe(void* out, int spins, void* stream) {
-    if (!out) return SQ_ERR_NULL_POINTER;
-    if (spins <= 0 || spins > (1 << 26)) return SQ_ERR_BAD_SHAPE;
-    return launch_code(sq::launch_clock_probe(out, spins, static_cast<hipStream_t>(stream)));
 }
 
 }  // extern "C"

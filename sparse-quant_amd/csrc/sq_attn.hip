@@ -243,7 +243,9 @@ __global__ __launch_bounds__(256 / QT) void lut_attn_kernel(const half_t* __rest
 #pragma unroll
     for (int qt = 0; qt < QT; qt++) {
         if (m[qt] < S) {
-            const float inv = l_i[qt] > 0.f ? 1.f / l_i[qt] : 0.f;
+            // A query row without any visible key has l = 0 and acc = 0: 0 * inf = NaN, which is
+            // also what the reference's running sums produce for such a row.
+            const float inv = 1.f / l_i[qt];
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
                 half4_t o;

@@ -249,10 +249,13 @@ hipError_t launch_d(const DecodeAttnArgs& a, int B, int nsplit, hipStream_t st) 
 
 }  // namespace
 
-static size_t decode_attention_counter_bytes(int B, int H) { return (((size_t)B * H * 4) + 255) & ~(size_t)255; }
+// Rows of a head are shared only with fewer than 256 (batch, head) pairs, so 256 counters are
+// always enough: the counter region has one fixed size and the partial states one fixed offset,
+// whatever B * H a workspace is used with next.
+constexpr size_t DECODE_ATTN_COUNTER_BYTES = 256 * sizeof(unsigned);
 
 size_t decode_attention_workspace_bytes(int B, int H, int D) {
-    return decode_attention_counter_bytes(B, H) + (size_t)B * H * DECODE_ATTN_MAX_SPLIT * (D + 2) * sizeof(float);
+    return DECODE_ATTN_COUNTER_BYTES + (size_t)B * H * DECODE_ATTN_MAX_SPLIT * (D + 2) * sizeof(float);
 }
 
 hipError_t launch_decode_attention(const void* q, const void* k_new, const void* v_new, void* k_cache, void* v_cache,
@@ -290,7 +293,7 @@ hipError_t launch_decode_attention(const void* q, const void* k_new, const void*
     a.cache_len_dev = cache_len_dev;
     a.scale = sm_scale;
     a.counters = (unsigned*)workspace;
-    a.part = workspace ? (float*)((char*)workspace + decode_attention_counter_bytes(B, H)) : nullptr;
+    a.part = workspace ? (float*)((char*)workspace + DECODE_ATTN_COUNTER_BYTES) : nullptr;
     return D == 64 ? launch_d<64>(a, B, nsplit, st) : launch_d<128>(a, B, nsplit, st);
 }
 

@@ -21,12 +21,8 @@ hipError_t launch_awq_to_lmdeploy(const void* src, void* dst, int K, int N, hipS
 hipError_t launch_l2_to_l1(const void* w_l2, const void* zs_l2, void* w_l1, void* zs_l1, int N, int K, int g,
                            hipStream_t st);
 hipError_t launch_2bit_to_4bit(const void* src, void* dst, int N, int K, hipStream_t st);
-hipError_t launch_clock_probe(void* out, int spins, hipStream_t st);
 
 // The *_tuned launchers take a kernel-specific tuning word (0 = built-in heuristic).
-// sq_gemv.hip: M <= 8.  tune = row steps per workgroup (1,2,4) | waves << 8.
-hipError_t launch_gemv_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
-                             bool fixup, int tune, Epilogue epi, hipStream_t st);
 // sq_gemv2.hip: M <= 8, streaming formulation.  tune = waves per workgroup (1,2,4,8).
 hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
                               bool fixup, int tune, Epilogue epi, hipStream_t st);
@@ -51,12 +47,6 @@ hipError_t launch_gemm_pipe(const void* x, const void* w, const void* zs, void* 
 hipError_t launch_lut_attention(const void* q, const void* k, const void* v, void* o, const void* lut,
                                 int lut_elem_bytes, int Z, int H, int S, int D, int nnz, float sm_scale, int causal,
                                 hipStream_t st);
-
-// sq_repack.hip: diagnostic read of an L1 weight with the GEMV's access pattern (see sq_read_probe).
-hipError_t launch_read_probe(const void* w, const void* zs, void* out, int N, int K, int g, hipStream_t st);
-
-// sq_repack.hip: diagnostic loop of independent matrix instructions (see sq_mfma_probe).
-hipError_t launch_mfma_probe(const void* data, void* out, int workgroups, int iters, hipStream_t st);
 
 // sq_decode_attn.hip: dense decode attention over an fp16 KV cache (one query row per sequence),
 // optionally appending the new key/value row.  Strides in elements.

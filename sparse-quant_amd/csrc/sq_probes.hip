@@ -1,0 +1,170 @@
+// Diagnostic kernels behind libsq_probes.so (include/sq_probes.h): a clock probe, the memory
+// side of the single-token GEMV without its arithmetic, and a loop of nothing but matrix
+// instructions.  They serve the benchmark's roofline context and are not part of the product
+// library.
+#include "../../include/sq_probes.h"
+
+#include "sq_common.h"
+
+namespace sq {
+
+// Diagnostic: one wave spins for `spins` dependent multiply-adds and reports how many
+// shader-clock ticks and how many ticks of the constant 100 MHz counter went by, so that a
+// caller running it beside a kernel on another stream can read the clock the chip sustains
+// under that kernel's load.
+__global__ void clock_probe_kernel(unsigned long long* out, int spins) {
+    const unsigned long long c0 = __builtin_readcyclecounter();
+    const unsigned long long r0 = wall_clock64();
+    float a = (float)threadIdx.x;
+    for (int i = 0; i < spins; i++) a = a * 1.0001f + 0.5f;
+    const unsigned long long c1 = __builtin_readcyclecounter();
+    const unsigned long long r1 = wall_clock64();
+    if (threadIdx.x == 0) {
+        out[0] = c1 - c0;
+        out[1] = r1 - r0;
+        out[2] = (unsigned long long)a;
+    }
+}
+
+// Diagnostic: the memory side of the single-token GEMV and nothing else.  Same grid, same lane ->
+// address mapping and the same number of loads in flight as gemv2_kernel at M = 1 (a wave-wide load
+// covers 4 rows x 256 contiguous bytes, all S loads of a round are issued before any is consumed, one
+// 32-bit zeros/scales word per load), but the data is only XOR-folded: the time of this kernel is what
+// the memory system charges for the weight stream of one launch.
+template <int NR, int KS, int S>
+__global__ __launch_bounds__(64 * NR * KS) void read_probe_kernel(const uint8_t* __restrict__ W,
+                                                                  const uint32_t* __restrict__ ZS,
+                                                                  uint32_t* __restrict__ out, int N, int K, int gshift) {
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int wr = wave % NR, wq_ = wave / NR;
+    const int i = lane & 3, b = lane >> 2;
+    const int row = imin(blockIdx.x * (4 * NR) + 4 * wr + i, N - 1);
+    const int nsteps = (K + 511) >> 9;
+    const int spw = (nsteps + KS - 1) / KS;
+    const int rounds = (spw + S - 1) / S;
+    const uint8_t* wrow = W + (long)row * (K >> 1);
+    const uint32_t* zrow = ZS + (long)row * (K >> gshift);
+    uint32_t fold = 0;
+    for (int rnd = 0; rnd < rounds; rnd++) {
+        u32x4_t wq[S];
+        uint32_t zq[S];
+#pragma unroll
+        for (int s = 0; s < S; s++) {
+            const int j = rnd * S + s;
+            const int kk = (wq_ * spw + j) * 512 + 32 * b;
+            const int kc = (j < spw && kk < K) ? kk : 0;
+            wq[s] = __builtin_nontemporal_load((const u32x4_t*)(wrow + (kc >> 1)));
+            zq[s] = zrow[kc >> gshift];
+        }
+#pragma unroll
+        for (int s = 0; s < S; s++) fold ^= wq[s].x ^ wq[s].y ^ wq[s].z ^ wq[s].w ^ zq[s];
+    }
+    if (fold == 0x9E3779B9u) out[blockIdx.x] = fold;  // practically never: keeps the loads alive
+}
+
+static hipError_t launch_read_probe(const void* w, const void* zs, void* out, int N, int K, int g, hipStream_t st) {
+    int gshift = 0;
+    while ((1 << gshift) < g) gshift++;
+    // the workgroup shapes the GEMV launcher picks at M = 1
+    const int nsteps = (K + 511) / 512;
+    const int ks = nsteps > 16 ? 4 : (((long)N * K >= (1L << 25) && nsteps >= 8) ? 2 : 1);
+    const int nr = ks == 4 ? 2 : 4;
+    const int spw = (nsteps + ks - 1) / ks;
+    const dim3 grid((N + 4 * nr - 1) / (4 * nr));
+#define SQ_RP(NR_, KS_, S_)                                                                                  \
+    hipLaunchKernelGGL((read_probe_kernel<NR_, KS_, S_>), grid, dim3(64 * NR_ * KS_), 0, st, (const uint8_t*)w, \
+                       (const uint32_t*)zs, (uint32_t*)out, N, K, gshift)
+    if (ks == 4) {
+        if (spw >= 8) SQ_RP(2, 4, 8); else SQ_RP(2, 4, 4);
+    } else if (ks == 2) {
+        if (spw >= 8) SQ_RP(4, 2, 8); else SQ_RP(4, 2, 4);
+    } else {
+        if (spw >= 8) SQ_RP(4, 1, 8); else SQ_RP(4, 1, 4);
+    }
+#undef SQ_RP
+    return hipGetLastError();
+}
+
+// Diagnostic: nothing but independent v_mfma_f32_32x32x16_f16, one wave per SIMD (256 threads per
+// workgroup, `workgroups` of them), operands taken from `data` (64 * 80 fp16 values of the caller's
+// choosing: the power the matrix pipes draw, and with it the clock the chip sustains, depends on the
+// operand bits).  out[w] = shader-clock ticks wave 0 of workgroup w spent in the loop.  The caller
+// times the launch: workgroups * 4 * iters * 16 matrix instructions of 32768 flop each.
+__global__ __launch_bounds__(256) void mfma_probe_kernel(const half_t* __restrict__ data, unsigned long long* out,
+                                                         float* sink, int iters) {
+    const int lane = threadIdx.x & 63;
+    half8_t a[8], b[2];
+#pragma unroll
+    for (int i = 0; i < 8; i++) a[i] = *(const half8_t*)(data + (lane * 10 + i) * 8);
+#pragma unroll
+    for (int i = 0; i < 2; i++) b[i] = *(const half8_t*)(data + (lane * 10 + 8 + i) * 8);
+    float16_t acc[8][2];
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+    const unsigned long long c0 = __builtin_readcyclecounter();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    const unsigned long long c1 = __builtin_readcyclecounter();
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) s += acc[i][j][v];
+    if (s == 12345.678f) sink[0] = s;  // keeps the accumulators alive
+    if (threadIdx.x == 0) out[blockIdx.x] = c1 - c0;
+}
+
+static hipError_t launch_mfma_probe(const void* data, void* out, int workgroups, int iters, hipStream_t st) {
+    float* sink = (float*)((unsigned long long*)out + workgroups);
+    hipLaunchKernelGGL(mfma_probe_kernel, dim3(workgroups), dim3(256), 0, st, (const half_t*)data,
+                       (unsigned long long*)out, sink, iters);
+    return hipGetLastError();
+}
+
+static hipError_t launch_clock_probe(void* out, int spins, hipStream_t st) {
+    hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, st, (unsigned long long*)out, spins);
+    return hipGetLastError();
+}
+
+}  // namespace sq
+
+namespace {
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline int launch_code(hipError_t e) { return e == hipSuccess ? SQP_OK : SQP_ERR_LAUNCH; }
+}  // namespace
+
+extern "C" {
+
+int sq_read_probe(const void* w, const void* zs, void* out, int N, int K, int group_size, void* stream) {
+    if (N <= 0 || K <= 0 || N % 8 != 0 || K % 32 != 0) return SQP_ERR_BAD_SHAPE;
+    if ((group_size != 32 && group_size != 64 && group_size != 128) || K % group_size != 0) return SQP_ERR_BAD_SHAPE;
+    if (!w || !zs || !out) return SQP_ERR_NULL_POINTER;
+    if (!aligned16(w) || !aligned16(zs)) return SQP_ERR_MISALIGNED;
+    return launch_code(sq::launch_read_probe(w, zs, out, N, K, group_size, static_cast<hipStream_t>(stream)));
+}
+
+int sq_mfma_probe(const void* data, void* out, int workgroups, int iters, void* stream) {
+    if (!data || !out) return SQP_ERR_NULL_POINTER;
+    if (workgroups <= 0 || workgroups > 65536 || iters <= 0 || iters > (1 << 22)) return SQP_ERR_BAD_SHAPE;
+    if (!aligned16(data)) return SQP_ERR_MISALIGNED;
+    return launch_code(sq::launch_mfma_probe(data, out, workgroups, iters, static_cast<hipStream_t>(stream)));
+}
+
+int sq_clock_probe(void* out, int spins, void* stream) {
+    if (!out) return SQP_ERR_NULL_POINTER;
+    if (spins <= 0 || spins > (1 << 26)) return SQP_ERR_BAD_SHAPE;
+    return launch_code(sq::launch_clock_probe(out, spins, static_cast<hipStream_t>(stream)));
+}
+
+}  // extern "C"

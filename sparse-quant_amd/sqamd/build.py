@@ -1,10 +1,12 @@
-"""Build recipe: libsq_w4a16.so (HIP kernels + C ABI) and the `quant` torch extension.
+"""Build recipe: libsq_w4a16.so (HIP kernels + C ABI), the `quant` torch extension and the
+benchmark's diagnostic library libsq_probes.so.
 
-Both are built in-tree, next to the `sqamd` package (the directory that is put on
+All are built in-tree, next to the `sqamd` package (the directory that is put on
 sys.path so that `import quant` finds the extension):
 
     sparse-quant_amd/libsq_w4a16.so
     sparse-quant_amd/quant.cpython-<abi>.so
+    sparse-quant_amd/libsq_probes.so
 
 hipcc cross-compiles for gfx950 without a GPU.  Run as `python -m sqamd.build`
 from sparse-quant_amd/, or call build_all().
@@ -23,8 +25,11 @@ LIB_PATH = os.path.join(PKG_ROOT, "libsq_w4a16.so")
 EXT_PATH = os.path.join(PKG_ROOT, "quant" + sysconfig.get_config_var("EXT_SUFFIX"))
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-HIP_SOURCES = ["sq_api.hip", "sq_dequant.hip", "sq_repack.hip", "sq_gemv.hip", "sq_gemv2.hip", "sq_skinny.hip", "sq_skinny2.hip", "sq_gemm.hip", "sq_gemm2.hip",
-               "sq_attn.hip", "sq_decode_attn.hip", "sq_layernorm.hip"]
+PROBES_PATH = os.path.join(PKG_ROOT, "libsq_probes.so")
+
+HIP_SOURCES = ["sq_api.hip", "sq_dequant.hip", "sq_repack.hip", "sq_gemv2.hip", "sq_skinny.hip", "sq_skinny2.hip",
+               "sq_gemm.hip", "sq_gemm2.hip", "sq_attn.hip", "sq_decode_attn.hip", "sq_layernorm.hip"]
+PROBE_SOURCES = ["sq_probes.hip"]  # diagnostic kernels, a library of their own (include/sq_probes.h)
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
              # keep the compiler from forming packed-fp32 instructions
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -50,10 +55,10 @@ def _run(cmd):
 
 
 def build_lib(verbose=True):
-    """Compile every HIP source for gfx950 and link libsq_w4a16.so."""
+    """Compile every HIP source for gfx950 and link libsq_w4a16.so and libsq_probes.so."""
     os.makedirs(OBJ_DIR, exist_ok=True)
     hipcc = os.path.join(ROCM, "bin", "hipcc")
-    sources = [s for s in HIP_SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    sources = HIP_SOURCES + PROBE_SOURCES
     objs = [os.path.join(OBJ_DIR, s.replace(".hip", ".o")) for s in sources]
 
     def compile_one(pair):
@@ -63,10 +68,12 @@ def build_lib(verbose=True):
 
     with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
         list(pool.map(compile_one, zip(sources, objs)))
-    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs +
-         ["-Wl,-rpath," + os.path.join(ROCM, "lib")])
-    if verbose:
-        print("built", LIB_PATH)
+    n = len(HIP_SOURCES)
+    for path, part in ((LIB_PATH, objs[:n]), (PROBES_PATH, objs[n:])):
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", path] + part +
+             ["-Wl,-rpath," + os.path.join(ROCM, "lib")])
+        if verbose:
+            print("built", path)
     return LIB_PATH
 
 
@@ -89,6 +96,7 @@ def build_ext(verbose=True):
            os.path.join(CSRC, "quant_ext.cpp"), "-o", EXT_PATH]
     cmd += ["-I" + p for p in inc]
     cmd += ["-L" + p for p in libdirs] + ["-L" + PKG_ROOT]
+    cmd += ["-L" + os.path.join(ROCM, "lib"), "-lamdhip64"]
     cmd += ["-lsq_w4a16", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python"]
     cmd += ["-Wl,-rpath,$ORIGIN"] + ["-Wl,-rpath," + p for p in libdirs]
     _run(cmd)

@@ -35,9 +35,6 @@ SIGNATURES = {
     "sq_convert_awq_to_lmdeploy": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_repack_l2_to_l1": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "sq_convert_2bit_to_4bit": (_i, [_vp, _vp, _i, _i, _vp]),
-    "sq_clock_probe": (_i, [_vp, _i, _vp]),
-    "sq_mfma_probe": (_i, [_vp, _vp, _i, _i, _vp]),
-    "sq_read_probe": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sq_decode_attention": (_i, [_vp] * 7 + [_i] * 4 + [ctypes.c_long] * 7 + [_i, _vp, ctypes.c_float, _vp, ctypes.c_size_t,
                                  _vp]),
     "sq_decode_attention_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
@@ -45,7 +42,16 @@ SIGNATURES = {
     "sq_lut_attention_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, ctypes.c_float, _i, _vp]),
 }
 
+# include/sq_probes.h (libsq_probes.so): diagnostic kernels used by the benchmark only.
+PROBES_PATH = os.path.join(PKG_ROOT, "libsq_probes.so")
+PROBE_SIGNATURES = {
+    "sq_clock_probe": (_i, [_vp, _i, _vp]),
+    "sq_mfma_probe": (_i, [_vp, _vp, _i, _i, _vp]),
+    "sq_read_probe": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+}
+
 _lib = None
+_probes = None
 
 
 class SqError(RuntimeError):
@@ -68,6 +74,21 @@ def lib():
             fn.argtypes = args
         _lib = handle
     return _lib
+
+
+def probes():
+    """The loaded diagnostic library; raises if it has not been built."""
+    global _probes
+    if _probes is None:
+        if not os.path.exists(PROBES_PATH):
+            raise RuntimeError("libsq_probes.so is missing at %s: run `python -m sqamd.build` first" % PROBES_PATH)
+        handle = ctypes.CDLL(PROBES_PATH)
+        for name, (res, args) in PROBE_SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _probes = handle
+    return _probes
 
 
 def strerror(code):
@@ -101,17 +122,24 @@ def gemm(x, w, zs, n, k, group_size, layout=SQ_LAYOUT_L1, algo=SQ_ALGO_AUTO, out
 
 SQ_ALGO_SKINNY_WS = 5
 _workspaces = {}
+_retired = []  # outgrown workspaces: a captured HIP graph may still hold their address
+
+
+def _cached_workspace(key, need, device):
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        if ws is not None:
+            _retired.append(ws)
+        ws = torch.zeros(need, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
 
 
 def workspace(m, n, k, device, stream=None):
     """A zero-initialised workspace tensor, cached per (device, stream) and grown on demand."""
     need = lib().sq_w4a16_workspace_bytes(m, n, k)
     key = (str(device), (stream or torch.cuda.current_stream()).cuda_stream)
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < need:
-        ws = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
+    return _cached_workspace(key, max(need, 1 << 20), device)
 
 
 def gemm_ws(x, w, zs, n, k, group_size, algo=SQ_ALGO_AUTO, out=None, stream=None, ws=None):
@@ -238,10 +266,7 @@ def decode_attention(q, k_cache, v_cache, cache_len, sm_scale, k_new=None, v_new
     if ws is None and use_workspace and b * h < 256:
         need = lib().sq_decode_attention_workspace_bytes(b, h, d)
         key = ("attn", str(q.device), (stream or torch.cuda.current_stream()).cuda_stream)
-        ws = _workspaces.get(key)
-        if ws is None or ws.numel() < need:
-            ws = torch.zeros(need, dtype=torch.uint8, device=q.device)
-            _workspaces[key] = ws
+        ws = _cached_workspace(key, need, q.device)
     _check(lib().sq_decode_attention(_ptr(q3), _ptr(kn) if kn is not None else None,
                                      _ptr(vn) if vn is not None else None, _ptr(k_cache), _ptr(v_cache),
                                      _ptr(mask) if mask is not None else None, _ptr(out), b, h, d, lmax,
@@ -264,7 +289,7 @@ def layernorm(x, gamma, beta, eps=1e-5, out=None, stream=None):
 def mfma_probe(data, workgroups, iters, stream=None):
     """Launch the matrix-instruction loop; returns the int64 tensor of per-workgroup shader ticks."""
     out = torch.zeros(workgroups + 1, dtype=torch.int64, device=data.device)
-    _check(lib().sq_mfma_probe(_ptr(data), _ptr(out), int(workgroups), int(iters), _stream(stream)), "sq_mfma_probe")
+    _check(probes().sq_mfma_probe(_ptr(data), _ptr(out), int(workgroups), int(iters), _stream(stream)), "sq_mfma_probe")
     return out[:workgroups]
 
 
@@ -273,5 +298,5 @@ def clock_probe(spins=400000, stream=None):
     shader ticks, 100 MHz ticks, dummy."""
     dev = torch.device("cuda", torch.cuda.current_device())
     out = torch.zeros(3, dtype=torch.int64, device=dev)
-    _check(lib().sq_clock_probe(_ptr(out), int(spins), _stream(stream)), "sq_clock_probe")
+    _check(probes().sq_clock_probe(_ptr(out), int(spins), _stream(stream)), "sq_clock_probe")
     return out

@@ -78,8 +78,9 @@ class WALinear(nn.Module):
             new.weight, new.zeros_scales = quant_funcs.quant_muxi(module.weight.data, module.in_features,
                                                                   module.out_features, n_bit=n_bit, group_size=g)
         else:
-            new.weight, new.zeros_scales = quant_funcs.quant_lmdeploy(module.weight.data, module.in_features,
-                                                                      module.out_features, group_size=g, n_bit=n_bit)
+            new.weight, new.zeros_scales, _ = quant_funcs.quant_lmdeploy(module.weight.data, module.in_features,
+                                                                         module.out_features, group_size=g,
+                                                                         n_bit=n_bit)
         if module.bias is not None:
             new.bias = module.bias.data.half().unsqueeze(0)
         return new

@@ -10,6 +10,11 @@ weight lives on:
 
 The layout-L2 chain calls the three converter kernels of the `quant` extension,
 exactly like the reference does, so it needs a GPU; the L1 path is pure torch.
+
+Like the reference, the quantiser computes in the dtype of the weight it is given
+(fp16 for the models the reference packs), so scales, zeros and codes of an fp16
+weight are bit-identical to the reference's; pass `compute_dtype=torch.float32` to
+quantise an fp16 weight in fp32 instead.
 """
 import torch
 
@@ -60,14 +65,18 @@ def merge_zeros_scales(zeros, scales):
     return torch.stack([z, s], dim=-1).reshape(z.shape[0], -1).contiguous()
 
 
-def quant_muxi(weight, input_features, output_features, n_bit=4, group_size=64):
+def _as(weight, compute_dtype):
+    return weight if compute_dtype is None else weight.to(compute_dtype)
+
+
+def quant_muxi(weight, input_features, output_features, n_bit=4, group_size=64, compute_dtype=None):
     """fp16 weight [N, K] -> (qweight uint8 [N, K*n_bit/8], zeros_scales fp16 [N, 2K/g]) in layout L1.
 
     The K-interleave permutes within runs of 8, i.e. inside a group, so zeros and
     scales are the same as those of the un-permuted weight.
     """
     assert weight.shape == (output_features, input_features)
-    q, scales, zeros = quantize_tensor(weight.float(), n_bit, group_size)
+    q, scales, zeros = quantize_tensor(_as(weight, compute_dtype), n_bit, group_size)
     q = interleave_k(q)
     if n_bit == 4:
         qweight = write_4bit_tensor(q)
@@ -78,29 +87,37 @@ def quant_muxi(weight, input_features, output_features, n_bit=4, group_size=64):
     return qweight.contiguous(), merge_zeros_scales(zeros, scales)
 
 
-def dequant_to_fp16(weight, n_bit=4, group_size=64):
+def dequant_to_fp16(weight, n_bit=4, group_size=64, compute_dtype=None):
     """The fake-quantised weight: fp16((q - z) * s) with fp16 zeros and scales.
 
     (reference: quantization/muxi/script/quant_dequant_muxi.py:73-85 applied to
     the un-permuted quantisation.)
     """
-    q, scales, zeros = quantize_tensor(weight.float(), n_bit, group_size)
+    q, scales, zeros = quantize_tensor(_as(weight, compute_dtype), n_bit, group_size)
     z = zeros.half().repeat_interleave(group_size, dim=1)
     s = scales.half().repeat_interleave(group_size, dim=1)
     return (q.half() - z) * s
 
 
-def quant_lmdeploy(weight, input_features, output_features, group_size=128, n_bit=4):
-    """fp16 weight [N, K] -> (qweight int32 [K, N/8], zeros_scales fp16 [K/g, 2N]) in layout L2.
+def quant_lmdeploy(weight, input_features, output_features, group_size=128, n_bit=4, compute_dtype=None):
+    """fp16 weight [N, K] -> (qweight int32 [K, N/8], zeros_scales fp16 [K/g, 2N], w_fp16 [N, K]) in
+    layout L2; w_fp16 = (q - z) * s in the compute dtype is the fake-quantised weight the reference
+    returns as its third value (test/nvidia/utils/quant_dequant_nvidia.py:32,70-71).
 
     Same three-step chain as the reference: "ours" bytes (even k in the high
     nibble) -> AWQ order -> tensor-core tile order, plus the transposed merge of
-    zeros and scales; every step is a kernel of the `quant` extension.
+    zeros and scales; every step is a kernel of the `quant` extension.  Only n_bit = 4: the
+    reference's int32 2-bit repacking (convert_4bit_to_2bit, :34-43) keeps, as Python evaluates its
+    shifts and masks, only half of each pair of words, so there is no 2-bit format to be compatible with.
     """
     import quant
 
-    assert n_bit == 4, "the tensor-core layout stores 4-bit weights"
-    q, scales, zeros = quantize_tensor(weight.float(), n_bit, group_size)
+    if n_bit != 4:
+        raise NotImplementedError("the tensor-core layout stores 4-bit weights only")
+    w = _as(weight, compute_dtype)
+    q, scales, zeros = quantize_tensor(w, n_bit, group_size)
+    g = group_size
+    w_fp16 = ((q.reshape(-1, g) - zeros.reshape(-1, 1)) * scales.reshape(-1, 1)).reshape(q.shape)
     q = q.to(torch.uint8)
     ours = ((q[:, 0::2] << 4) | q[:, 1::2]).contiguous()
     dev = weight.device
@@ -111,4 +128,4 @@ def quant_lmdeploy(weight, input_features, output_features, group_size=128, n_bi
     quant.convert_ours_to_awq(ours, awq, input_features, output_features)
     qweight = torch.empty((input_features, output_features // 8), dtype=torch.int32, device=dev)
     quant.convert_awq_to_lmdeploy(awq, qweight, input_features, output_features)
-    return qweight, zeros_scales
+    return qweight, zeros_scales, w_fp16

@@ -156,3 +156,42 @@ def test_package_lut_builder_agrees_with_the_oracle():
             assert not bool(torch.triu(lay, diagonal=1).any())
         lut = layout2lut_single_density(lay[None])[0]
         assert np.array_equal(lut.numpy(), att.layout_to_lut(lay.numpy()))
+
+
+def test_repeated_block_after_a_different_one_counts_twice():
+    """Padding rule: only an entry equal to its predecessor is skipped.  A row [1, 2, 1] therefore
+    attends the keys of block 1 twice; pinned against textbook softmax attention over the explicit
+    concatenation of the visited blocks.  An immediate repeat [1, 1, 2] counts block 1 once."""
+    rng = np.random.default_rng(3)
+    s, d, nb = 192, 16, 3
+    q = rng.normal(size=(1, 1, s, d))
+    k = rng.normal(size=(1, 1, s, d))
+    v = rng.normal(size=(1, 1, s, d))
+    blocks = lambda a, idx: np.concatenate([a[0, 0, 64 * j:64 * j + 64] for j in idx], axis=0)
+
+    def textbook(rows, idx):
+        kk, vv = blocks(k, idx), blocks(v, idx)
+        sc = q[0, 0, rows] @ kk.T * 0.3
+        p = np.exp(sc - sc.max(axis=-1, keepdims=True))
+        return (p / p.sum(axis=-1, keepdims=True)) @ vv
+
+    lut = np.array([[[0, 0, 0], [1, 2, 1], [1, 1, 2]]])
+    counts = att.lut_to_counts(lut, nb)
+    assert counts[0].tolist() == [[1, 0, 0], [0, 2, 1], [0, 1, 1]]
+    out = att.attention_ref(q, k, v, lut, 0.3, False)
+    assert np.allclose(out[0, 0, 64:128], textbook(slice(64, 128), [1, 2, 1]), rtol=1e-12, atol=1e-12)
+    assert np.allclose(out[0, 0, 128:192], textbook(slice(128, 192), [1, 2]), rtol=1e-12, atol=1e-12)
+    assert np.allclose(out[0, 0, :64], textbook(slice(0, 64), [0]), rtol=1e-12, atol=1e-12)
+    # more entries than key blocks: only the first nb are read
+    lut4 = np.array([[[0, 1, 2, 0], [1, 1, 1, 0], [2, 2, 2, 2]]])
+    assert att.lut_to_counts(lut4, nb)[0].tolist() == [[1, 1, 1], [0, 1, 0], [0, 0, 1]]
+
+
+def test_row_without_visible_key_is_nan():
+    # causal, query block 0 pointed at key block 1 only: nothing visible
+    rng = np.random.default_rng(4)
+    q = rng.normal(size=(1, 1, 128, 8))
+    lut = np.array([[[1], [1]]])
+    with np.errstate(invalid="ignore"):
+        out = att.attention_ref(q, q, q, lut, 1.0, True)
+    assert np.all(np.isnan(out[0, 0, :64])) and np.all(np.isfinite(out[0, 0, 64:]))

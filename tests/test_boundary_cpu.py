@@ -14,8 +14,11 @@ REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(REPO, "include", "sq_w4a16.h")
 
 
-def declared_functions():
-    text = open(HEADER).read()
+PROBES_HEADER = os.path.join(REPO, "include", "sq_probes.h")
+
+
+def declared_functions(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(sq_[a-z0-9_]+)\s*\(", text)))
 
@@ -41,6 +44,18 @@ def test_ctypes_binding_covers_header(built_lib):
     for code in range(1, 9):
         assert capi.strerror(code) not in ("ok", "unknown error code")
     assert capi.strerror(999) == "unknown error code"
+
+
+def test_probe_library_exports_its_header(built_lib):
+    from sqamd import capi
+    names = declared_functions(PROBES_HEADER)
+    assert names == sorted(capi.PROBE_SIGNATURES) and len(names) == 3
+    lib = capi.probes()
+    for name in names:
+        assert hasattr(lib, name)
+    assert not set(names) & set(declared_functions()), "diagnostics do not belong to the product header"
+    assert lib.sq_read_probe(None, None, None, 64, 128, 64, None) == 1
+    assert lib.sq_clock_probe(None, 10, None) == 1
 
 
 def test_argument_errors_come_before_any_launch(built_lib):
@@ -126,6 +141,18 @@ def test_host_packers_match_oracle():
         # the fake-quantised weight equals the oracle's dequantisation of the packed tensors
         deq = qf.dequant_to_fp16(torch.from_numpy(w), 4, g).numpy()
         assert np.array_equal(deq.view(np.uint16), orc.dequant_l1(qw.numpy(), zs.numpy(), g).view(np.uint16))
+    # an fp16 weight is quantised in fp16, like the reference does: bit-equal to the oracle's fp16 restatement,
+    # and in fp32 on request
+    wh = w.astype(np.float16)
+    for g in (64, 128):
+        qw, zs = qf.quant_muxi(torch.from_numpy(wh), 256, 32, n_bit=4, group_size=g)
+        q, s, z = orc.rtn_quantize(wh, 4, g, dtype=np.float16)
+        assert np.array_equal(qw.numpy(), orc.pack_l1(q))
+        assert np.array_equal(zs.numpy().view(np.uint16), orc.zeros_scales_l1(z, s).view(np.uint16))
+        qw32, zs32 = qf.quant_muxi(torch.from_numpy(wh), 256, 32, n_bit=4, group_size=g, compute_dtype=torch.float32)
+        q, s, z = orc.rtn_quantize(wh.astype(np.float32), 4, g)
+        assert np.array_equal(qw32.numpy(), orc.pack_l1(q))
+        assert np.array_equal(zs32.numpy().view(np.uint16), orc.zeros_scales_l1(z, s).view(np.uint16))
     # 2-bit packing, then expansion to 4-bit nibbles
     qw2, zs2 = qf.quant_muxi(torch.from_numpy(w), 256, 32, n_bit=2, group_size=64)
     q2, s2, z2 = orc.rtn_quantize(w, 2, 64)

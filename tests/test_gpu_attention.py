@@ -105,3 +105,41 @@ def test_attention_argument_errors(capi):
     assert L.sq_lut_attention_fwd(p, p, p, p, p, 2, 1, 1, 64, 64, 1, 1.0, 0, None) == capi.SQ_ERR_BAD_LAYOUT  # lut width
     assert L.sq_lut_attention_fwd(p, p, None, p, p, 8, 1, 1, 64, 64, 1, 1.0, 0, None) == capi.SQ_ERR_NULL_POINTER
     assert L.sq_lut_attention_fwd(p, p, p, p, p, 8, 1, 1, 0, 64, 1, 1.0, 0, None) == capi.SQ_ERR_BAD_SHAPE
+
+
+@pytest.mark.parametrize("d", [64, 128])
+def test_block_named_again_after_a_different_one_is_attended_twice(capi, d):
+    """Only an entry equal to its predecessor is padding: rows such as [1, 3, 1, 0] visit block 1 twice
+    (its keys carry double weight), [2, 2, 0, 0] visits 2 and 0 once each, entries beyond the sequence
+    select nothing -- the oracle weighs every key block by its number of visits."""
+    rng = np.random.default_rng(31)
+    z, h, s = 2, 2, 250
+    q = rng.normal(size=(z, h, s, d)).astype(np.float16)
+    k = rng.normal(size=(z, h, s, d)).astype(np.float16)
+    v = rng.normal(size=(z, h, s, d)).astype(np.float16)
+    lut = np.array([[[0, 1, 0, 1], [1, 3, 1, 0], [2, 2, 0, 0], [3, 0, 3, 0]],
+                    [[2, 0, 2, 2], [1, 1, 1, 1], [0, 9, 0, 2], [3, 2, 1, 0]]], dtype=np.int64)
+    assert att.lut_to_counts(lut, 4).max() == 2
+    ref = att.attention_ref(q, k, v, lut, 0.11, False)
+    out = capi.lut_attention(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(),
+                             torch.from_numpy(lut).cuda(), 0.11, False)
+    torch.cuda.synchronize()
+    out = out.float().cpu().numpy().astype(np.float64)
+    assert np.max(np.abs(out - ref)) <= TOL * np.max(np.abs(ref))
+
+
+def test_query_rows_without_a_visible_key_are_nan(capi):
+    # causal, query block 0 of head 0 is pointed at key block 1 only: nothing is visible -> NaN, like the
+    # reference's running sums; every other row is unaffected
+    rng = np.random.default_rng(32)
+    z, h, s, d = 1, 2, 128, 64
+    q = rng.normal(size=(z, h, s, d)).astype(np.float16)
+    lut = np.array([[[1], [1]], [[0], [1]]], dtype=np.int64)
+    with np.errstate(invalid="ignore"):
+        ref = att.attention_ref(q, q, q, lut, 0.125, True)
+    qt = torch.from_numpy(q).cuda()
+    out = capi.lut_attention(qt, qt, qt, torch.from_numpy(lut).cuda(), 0.125, True).float().cpu().numpy()
+    assert np.all(np.isnan(out[0, 0, :64])) and np.all(np.isnan(ref[0, 0, :64]))
+    ok = np.isfinite(ref)
+    assert np.array_equal(ok, np.isfinite(out))
+    assert np.max(np.abs(out[ok] - ref[ok])) <= TOL * np.max(np.abs(ref[ok]))

@@ -299,3 +299,23 @@ def test_decode_split_with_mask_and_fully_masked_share(capi):
     out = capi.decode_attention(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(), l, 0.09,
                                 mask=torch.from_numpy(mask).cuda())
     check(out, ref, "masked shares")
+
+
+def test_decode_split_workspace_shared_across_head_counts(capi):
+    """One zeroed workspace used with B*H = 128, then 32, then 128 again: the counters sit in a fixed
+    region in front of the partial states, so a call with fewer heads cannot leave partial states
+    where a later call with more heads reads its counters."""
+    d, l, h = 128, 640, 32
+    need = capi.lib().sq_decode_attention_workspace_bytes(4, h, d)
+    ws = torch.zeros(need, dtype=torch.uint8, device="cuda")
+    scale = 1.0 / np.sqrt(d)
+    for b in (4, 1, 4):
+        q, k, v = make(b, h, l, d, seed=70 + b)
+        qt, kc, vc = torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda()
+        ref = att.decode_attention_ref(q, k, v, scale)
+        out = capi.decode_attention(qt, kc, vc, l, scale, ws=ws)
+        single = capi.decode_attention(qt, kc, vc, l, scale, use_workspace=False)
+        torch.cuda.synchronize()
+        check(out, ref, "shared workspace, b=%d" % b)
+        assert (out.float() - single.float()).abs().max().item() <= 2e-3
+        assert torch.count_nonzero(ws[:1024]).item() == 0

@@ -91,8 +91,9 @@ def test_gemv_parity_small(capi, n, k, g, m, algo_name):
     check_gemm(capi, m, n, k, g, getattr(capi, "SQ_ALGO_" + algo_name))
 
 
-@pytest.mark.parametrize("tune", [1 | (1 << 8), 2 | (4 << 8), 4 | (8 << 8), 1 | (16 << 8), 4 | (3 << 8)])
+@pytest.mark.parametrize("tune", [nr | (ks << 4) for nr in (2, 4, 8) for ks in (1, 2, 4)])
 def test_gemv_every_tuning_is_correct(capi, tune):
+    # tune = row groups per workgroup | k ranges per workgroup << 4
     for m in (1, 4, 7):
         check_gemm(capi, m, 200, 1536, 64, capi.SQ_ALGO_GEMV | (tune << 8))
         check_gemm(capi, m, 200, 1536, 128, capi.SQ_ALGO_GEMV_FIXUP | (tune << 8))
@@ -272,7 +273,8 @@ def test_quant_extension_l2_weights():
     torch.manual_seed(1)
     k, n, g = 1024, 512, 128
     lin = torch.nn.Linear(k, n, bias=False, device=DEV, dtype=torch.float16)
-    qw2, zs2 = qf.quant_lmdeploy(lin.weight.data, k, n, group_size=g, n_bit=4)
+    qw2, zs2, w_fake = qf.quant_lmdeploy(lin.weight.data, k, n, group_size=g, n_bit=4)
+    assert w_fake.dtype == torch.float16 and tuple(w_fake.shape) == (n, k)
     assert qw2.dtype == torch.int32 and tuple(qw2.shape) == (k, n // 8) and tuple(zs2.shape) == (k // g, 2 * n)
     w_fp16 = qf.dequant_to_fp16(lin.weight.data, 4, g)
     assert torch.equal(quant.dequant(qw2, zs2, n, k, g), w_fp16)
@@ -445,7 +447,7 @@ def fused_ref(x, w_hat, bias, residual, act):
 
 FUSED_CASES = [  # (m, n, k, g, algo name, tune) -- one per kernel family and tile variant
     (1, 256, 1024, 128, "GEMV", 0), (3, 136, 640, 32, "GEMV_FIXUP", 0), (8, 200, 1536, 64, "GEMV_FIXUP", 2 | (4 << 4)),
-    (5, 256, 1024, 128, "GEMV", 0x8000 | 1 | (4 << 8)), (17, 136, 640, 32, "SKINNY", 0), (32, 256, 1024, 128, "SKINNY", 0),
+    (5, 256, 1024, 128, "GEMV", 2 | (2 << 4)), (17, 136, 640, 32, "SKINNY", 0), (32, 256, 1024, 128, "SKINNY", 0),
     (9, 520, 1056, 32, "SKINNY_WS", 1), (16, 264, 2048, 128, "SKINNY_WS", 4), (32, 256, 1024, 128, "SKINNY_WS", 2),
     (70, 264, 704, 64, "GEMM", 1), (70, 264, 704, 64, "GEMM", 2), (300, 520, 1056, 32, "GEMM", 4),
     (300, 520, 1056, 32, "GEMM", 8), (300, 520, 1056, 32, "GEMM", 9), (300, 520, 1056, 32, "GEMM", 10),
@@ -559,7 +561,7 @@ def test_reference_grid_int32_layout(k, n):
     torch.manual_seed(k * 3 + n)
     g = 128
     lin = torch.nn.Linear(k, n, bias=False, device=DEV, dtype=torch.float16)
-    qweight, zeros_scales = qf.quant_lmdeploy(lin.weight.data, k, n, group_size=g)
+    qweight, zeros_scales, _ = qf.quant_lmdeploy(lin.weight.data, k, n, group_size=g)
     assert qweight.dtype == torch.int32 and tuple(qweight.shape) == (k, n // 8)
     w_fp16 = qf.dequant_to_fp16(lin.weight.data, 4, g).float()
     for seq in (1, 128):
@@ -629,7 +631,7 @@ def test_read_probe_runs_on_every_reference_shape(capi):
         g = 128 if k % 128 == 0 else 32
         w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=DEV)
         zs = torch.zeros((n, 2 * (k // g)), dtype=torch.float16, device=DEV)
-        rc = capi.lib().sq_read_probe(w.data_ptr(), zs.data_ptr(), out.data_ptr(), n, k, g, None)
+        rc = capi.probes().sq_read_probe(w.data_ptr(), zs.data_ptr(), out.data_ptr(), n, k, g, None)
         assert rc == 0
     torch.cuda.synchronize()
-    assert capi.lib().sq_read_probe(None, None, out.data_ptr(), 4096, 4096, 128, None) == capi.SQ_ERR_NULL_POINTER
+    assert capi.probes().sq_read_probe(None, None, out.data_ptr(), 4096, 4096, 128, None) == capi.SQ_ERR_NULL_POINTER

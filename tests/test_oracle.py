@@ -10,6 +10,8 @@ import ctypes
 import json
 import os
 
+from fractions import Fraction
+
 import numpy as np
 import pytest
 
@@ -233,6 +235,65 @@ def test_rtn_kat():
     q, s, z = orc.rtn_quantize(np.array(k["w"], dtype=np.float32), k["n_bit"], k["group"])
     assert q[0].tolist() == k["q"]
     assert abs(float(s[0, 0]) - k["scale"]) < 1e-6 and float(z[0, 0]) == k["zero"]
+
+
+def _rn16(fr):
+    """Exact rational -> nearest fp16 (ties to even), as a Fraction; written out bit by bit so that it does
+    not lean on numpy's conversions."""
+    from fractions import Fraction
+    if fr == 0:
+        return Fraction(0)
+    sign = -1 if fr < 0 else 1
+    a = abs(fr)
+    e = 0
+    while a >= 2:
+        a /= 2
+        e += 1
+    while a < 1:
+        a *= 2
+        e -= 1
+    e = max(e, -14)                      # subnormals share the exponent of the smallest normal
+    ulp = Fraction(2) ** (e - 10)
+    n = abs(fr) / ulp
+    lo = n.numerator // n.denominator
+    rem = n - lo
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and lo % 2 == 1):
+        lo += 1
+    if lo * ulp >= 65520:
+        return Fraction(sign * 10 ** 9)   # overflow to infinity: any value that every later clamp saturates
+    return sign * lo * ulp
+
+
+def _round_half_even(fr):
+    lo = fr.numerator // fr.denominator
+    rem = fr - lo
+    return lo + 1 if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and lo % 2 == 1) else lo
+
+
+def test_rtn_in_fp16_matches_exact_rational_arithmetic():
+    """The quantiser in fp16 (what the reference computes on the fp16 weights it packs): every operation
+    of the formula done in exact rational arithmetic and rounded to fp16 by hand."""
+    rng = np.random.default_rng(43)
+    w = rng.normal(0, 0.05, size=(6, 64)).astype(np.float16)
+    w[1, :32] = np.float16(0.25)         # a constant group: the 1e-5 clamp
+    differs = False
+    for g in (32, 64):
+        q, s, z = orc.rtn_quantize(w, 4, g, dtype=np.float16)
+        q32, _, _ = orc.rtn_quantize(w.astype(np.float32), 4, g)
+        differs |= not np.array_equal(q, q32)
+        for r in range(w.shape[0]):
+            for gi in range(64 // g):
+                vals = [Fraction(float(v)) for v in w[r, gi * g:(gi + 1) * g]]
+                d = max(_rn16(max(vals) - min(vals)), _rn16(Fraction(1e-5)))
+                sc = _rn16(d / 15)
+                assert Fraction(float(s[r, gi])) == sc
+                zero = min(max(-_round_half_even(_rn16(min(vals) / sc)), 0), 15)
+                assert int(z[r, gi]) == zero
+                for j, v in enumerate(vals):
+                    t = _rn16(v / sc)
+                    want = min(max(_round_half_even(t) + zero, 0), 15)
+                    assert int(q[r, gi * g + j]) == want, (r, gi, j)
+    assert differs, "the fp16 and fp32 quantisers never disagreed: the test does not separate them"
 
 
 def test_rtn_properties():
