@@ -36,6 +36,7 @@ extern "C" {
 #define SQ_ERR_MISALIGNED 6      /* pointer not 16-byte aligned */
 #define SQ_ERR_LAUNCH 7          /* the HIP runtime rejected the launch */
 #define SQ_ERR_WORKSPACE 8       /* workspace missing or too small */
+#define SQ_ERR_STATIC_WS 9       /* sq_w4a16_gemm_static_ws: the shape needs more than SQ_STATIC_WS_BYTES */
 
 #define SQ_LAYOUT_L1 1
 #define SQ_LAYOUT_L2 2
@@ -88,6 +89,25 @@ int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y,
 int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y,
                      int M, int N, int K, int group_size, int layout, int algo,
                      void* workspace, size_t workspace_bytes, void* stream);
+
+/* sq_w4a16_gemm_ws for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
+ * reference.  Same product, same kernels and the same automatic kernel choice, bit-identical
+ * results; the workspace is a buffer of SQ_STATIC_WS_BYTES (16 MiB + 64 KiB) that lives inside
+ * the library's device code, one copy per GPU for the life of the process, so the call
+ * allocates and frees nothing.  The caller still passes inputs and the output.
+ * Limit: shapes with sq_w4a16_workspace_bytes(M, N, K) > SQ_STATIC_WS_BYTES are rejected with
+ * SQ_ERR_STATIC_WS and nothing is launched (every decode batch of up to 32 tokens with
+ * N <= 16384 fits; so do the K splits of the tiled GEMM up to that size).
+ * The first call on a device looks the buffer's address up and enqueues a small kernel on
+ * `stream` that clears its counter region; make that first call outside graph capture.
+ * Every call on a GPU shares that GPU's buffer: calls that overlap in time on one GPU (two
+ * streams, two threads) race; calls on one stream are ordered and safe.  The buffer keeps the
+ * last call's partial sums; the kernels overwrite what they read and leave the counters zero. */
+#define SQ_STATIC_WS_BYTES (16 * 1024 * 1024 + 64 * 1024)
+int sq_w4a16_gemm_static_ws(const void* x, const void* w, const void* zs, void* y,
+                            int M, int N, int K, int group_size, int layout, int algo,
+                            void* stream);
 
 /* Bytes sq_w4a16_gemm_ws / sq_w4a16_gemm_fused can use for this shape (8.06 MiB for
  * every decode batch with N <= 16384; up to tens of MiB for the GEMM split). */

@@ -2,9 +2,52 @@
 // and the contract of every entry point are in include/sq_w4a16.h.
 #include "../../include/sq_w4a16.h"
 
+#include <mutex>
+
 #include "sq_kernels.h"
 
+// Workspace of sq_w4a16_gemm_static_ws: device memory that belongs to the library, so that the
+// call allocates nothing.  Every GPU the library runs on holds its own copy of the array until the
+// process ends; the name below is only the host-side handle of the symbol, the device address is
+// looked up once per device with hipGetSymbolAddress and that pointer is what the kernels get.
+static __device__ __align__(256) unsigned char scratch[SQ_STATIC_WS_BYTES];
+
 namespace {
+
+__global__ void zero_words_kernel(unsigned* p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+constexpr int MAX_DEVICES = 64;
+struct ScratchState {
+    void* ptr = nullptr;
+    bool cleared = false;
+};
+ScratchState g_scratch[MAX_DEVICES];
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device; on the first call per device the counter
+// region (the part every kernel expects to find zero and leaves zero) is cleared by a small fill
+// kernel on `st`, ahead of the first use.  Returns null on failure.
+void* static_workspace(hipStream_t st) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    ScratchState& s = g_scratch[dev];
+    if (!s.ptr) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+        s.ptr = p;
+    }
+    if (!s.cleared) {
+        constexpr int words = 64 * 1024 / 4;
+        hipLaunchKernelGGL(zero_words_kernel, dim3(words / 256), dim3(256), 0, st, static_cast<unsigned*>(s.ptr), words);
+        if (hipGetLastError() != hipSuccess) return nullptr;
+        s.cleared = true;
+    }
+    return s.ptr;
+}
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline int launch_code(hipError_t e) { return e == hipSuccess ? SQ_OK : SQ_ERR_LAUNCH; }
@@ -122,6 +165,7 @@ const char* sq_strerror(int code) {
         case SQ_ERR_MISALIGNED: return "pointer is not 16-byte aligned";
         case SQ_ERR_LAUNCH: return "HIP kernel launch failed";
         case SQ_ERR_WORKSPACE: return "workspace missing or too small";
+        case SQ_ERR_STATIC_WS: return "problem needs a larger workspace than the library's static buffer (SQ_STATIC_WS_BYTES)";
         default: return "unknown error code";
     }
 }
@@ -143,6 +187,24 @@ int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y, int 
                      int layout, int algo, void* workspace, size_t workspace_bytes, void* stream) {
     return gemm_dispatch(x, w, zs, y, M, N, K, group_size, layout, algo, sq::Epilogue{nullptr, nullptr, 0}, workspace,
                          workspace_bytes, stream);
+}
+
+int sq_w4a16_gemm_static_ws(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
+                            int layout, int algo, void* stream) {
+    if (M > 0 && N > 0 && K > 0 && sq_w4a16_workspace_bytes(M, N, K) > (size_t)SQ_STATIC_WS_BYTES) return SQ_ERR_STATIC_WS;
+    // Validate before touching the device, so that argument errors launch nothing (not even the
+    // one-time clearing of the counters).
+    if (M < 0) return SQ_ERR_BAD_SHAPE;
+    const int rc = check_weight(N, K, group_size, layout);
+    if (rc != SQ_OK) return rc;
+    if (layout != SQ_LAYOUT_L1) return SQ_ERR_BAD_LAYOUT;
+    if (M == 0) return SQ_OK;
+    if (!x || !w || !zs || !y) return SQ_ERR_NULL_POINTER;
+    if (!aligned16(x) || !aligned16(w) || !aligned16(zs) || !aligned16(y)) return SQ_ERR_MISALIGNED;
+    void* ws = static_workspace(static_cast<hipStream_t>(stream));
+    if (!ws) return SQ_ERR_LAUNCH;
+    return gemm_dispatch(x, w, zs, y, M, N, K, group_size, layout, algo, sq::Epilogue{nullptr, nullptr, 0}, ws,
+                         (size_t)SQ_STATIC_WS_BYTES, stream);
 }
 
 int sq_w4a16_gemm_fused(const void* x, const void* w, const void* zs, const void* bias, const void* residual, void* y,

@@ -27,6 +27,7 @@ SIGNATURES = {
     "sq_w4a16_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "sq_w4a16_gemm_ex": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "sq_w4a16_gemm_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp]),
+    "sq_w4a16_gemm_static_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "sq_w4a16_gemm_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp]),
     "sq_w4a16_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
     "sq_w4a16_dequant": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
@@ -151,6 +152,20 @@ def gemm_ws(x, w, zs, n, k, group_size, algo=SQ_ALGO_AUTO, out=None, stream=None
         ws = workspace(max(m, 1), n, k, x.device, stream)
     _check(lib().sq_w4a16_gemm_ws(_ptr(x), _ptr(w), _ptr(zs), _ptr(out), m, n, k, group_size, SQ_LAYOUT_L1, algo,
                                   _ptr(ws), ws.numel(), _stream(stream)), "sq_w4a16_gemm_ws")
+    return out
+
+
+SQ_ERR_STATIC_WS = 9
+SQ_STATIC_WS_BYTES = 16 * 1024 * 1024 + 64 * 1024
+
+
+def gemm_static_ws(x, w, zs, n, k, group_size, algo=SQ_ALGO_AUTO, out=None, stream=None):
+    """x fp16 [M,K] -> y fp16 [M,N] through sq_w4a16_gemm_static_ws (workspace inside the library)."""
+    m = x.numel() // k
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
+    _check(lib().sq_w4a16_gemm_static_ws(_ptr(x), _ptr(w), _ptr(zs), _ptr(out), m, n, k, group_size, SQ_LAYOUT_L1, algo,
+                                         _stream(stream)), "sq_w4a16_gemm_static_ws")
     return out
 
 
