@@ -131,6 +131,48 @@ int sq_w4a16_gemm_fused(const void* x, const void* w, const void* zs, const void
                         int layout, int act, int algo, void* workspace, size_t workspace_bytes,
                         void* stream);
 
+/* Up to SQ_SEQUENCE_MAX decode linears (1..4 tokens) with one call:
+ *     for l in 0 .. count-1:  y_l = act_l(x_l * W_hat_l^T + bias_l) + residual_l
+ * executed in order.  No counterpart in the reference, which launches its GEMV once per linear
+ * (quantization/muxi/backend/w4a16_gemm.cuh:14-326 under test/muxi/module/qlinear/qlinear.py:61-70);
+ * at one token every such launch spends about as long getting started as streaming its weights.
+ * Linears that do not depend on each other (q, k and v of a decoder layer) are served by ONE
+ * persistent launch: one workgroup per CU stays resident and the weight stream never stops between
+ * linears.
+ *   depends  set it on linear l when x_l or residual_l (or any buffer it reads) is written by an
+ *            earlier linear of the same call.  Linears without it may run ahead of earlier ones.
+ *            A buffer written by linear i may be read or overwritten by linear j > i only if j, or
+ *            a linear between them, has depends set; y_l must not alias x_l or residual_l.
+ *   mode     SQ_SEQ_AUTO: a linear with depends starts a new launch (the kernel boundary is the
+ *            cheapest dependency on this part); SQ_SEQ_ONE_LAUNCH: everything in one persistent
+ *            launch, dependencies honoured by a grid barrier inside the kernel (slower today; kept
+ *            for measurement).
+ *   workspace  sq_w4a16_gemv_sequence_workspace_bytes() bytes (256), 16-byte aligned, zero before
+ *            the first call (every call leaves it zero); calls that share it must be ordered.
+ *            Word 9 of it is a sticky error flag: it becomes 1 if a grid barrier ever ran out of
+ *            polls (results of that call are then undefined).
+ * Shapes as for sq_w4a16_gemm (all linears share M).  With M > 4, without a workspace, or when the
+ * activations of a linear do not fit the LDS (M * K * 2 bytes beyond about 128 KiB), the linears are
+ * launched one by one on the stream instead: same results.  The persistent kernel needs every
+ * workgroup resident at once (one per CU); other work running on the GPU only delays it. */
+#define SQ_SEQ_AUTO 0
+#define SQ_SEQ_ONE_LAUNCH 1
+#define SQ_SEQUENCE_MAX 8
+typedef struct sq_linear_desc {
+    const void* x;         /* fp16 [M, K] */
+    const void* w;         /* layout L1 */
+    const void* zs;
+    const void* bias;      /* fp16 [N] or NULL */
+    const void* residual;  /* fp16 [M, N] or NULL */
+    void* y;               /* fp16 [M, N] */
+    int N, K, group_size;
+    int act;               /* SQ_ACT_NONE or SQ_ACT_RELU */
+    int depends;           /* see above */
+} sq_linear_desc;
+int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int layout, int mode,
+                           void* workspace, size_t workspace_bytes, void* stream);
+size_t sq_w4a16_gemv_sequence_workspace_bytes(void);
+
 /* out[N,K] (fp16) = W_hat in natural k order, bit-identical to fp16
  * (q_fp16 - z_fp16) * s_fp16.  Replaces dequant
  * (reference: quantization/tianshu/backend/gemm_quant.cu:153-164 and

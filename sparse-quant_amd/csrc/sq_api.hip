@@ -207,6 +207,64 @@ int sq_w4a16_gemm_static_ws(const void* x, const void* w, const void* zs, void* 
                          (size_t)SQ_STATIC_WS_BYTES, stream);
 }
 
+size_t sq_w4a16_gemv_sequence_workspace_bytes(void) { return sq::gemv_seq_workspace_bytes(); }
+
+int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int layout, int mode, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+    if (count < 0 || count > SQ_SEQUENCE_MAX) return SQ_ERR_BAD_SHAPE;
+    if (mode != SQ_SEQ_AUTO && mode != SQ_SEQ_ONE_LAUNCH) return SQ_ERR_BAD_ALGO;
+    if (count == 0) return SQ_OK;
+    if (!linears) return SQ_ERR_NULL_POINTER;
+    if (M < 0) return SQ_ERR_BAD_SHAPE;
+    if (layout != SQ_LAYOUT_L1) return SQ_ERR_BAD_LAYOUT;
+    sq::SeqProblem probs[SQ_SEQUENCE_MAX];
+    for (int l = 0; l < count; l++) {
+        const sq_linear_desc& d = linears[l];
+        const int rc = check_weight(d.N, d.K, d.group_size, layout);
+        if (rc != SQ_OK) return rc;
+        if (d.act != SQ_ACT_NONE && d.act != SQ_ACT_RELU) return SQ_ERR_BAD_ALGO;
+        if (M > 0) {
+            if (!d.x || !d.w || !d.zs || !d.y) return SQ_ERR_NULL_POINTER;
+            if (!aligned16(d.x) || !aligned16(d.w) || !aligned16(d.zs) || !aligned16(d.y)) return SQ_ERR_MISALIGNED;
+            if ((d.bias && (reinterpret_cast<uintptr_t>(d.bias) & 1u)) ||
+                (d.residual && (reinterpret_cast<uintptr_t>(d.residual) & 1u)))
+                return SQ_ERR_MISALIGNED;
+        }
+        probs[l] = sq::SeqProblem{d.x, d.w, d.zs, d.bias, d.residual, d.y, d.N, d.K, d.group_size, d.act, d.depends};
+    }
+    if (M == 0) return SQ_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool ws_ok = workspace && aligned16(workspace) && workspace_bytes >= sq::gemv_seq_workspace_bytes();
+    // Runs of linears without a dependency between them go out as one persistent launch each; a linear that
+    // depends on an earlier one starts a new run, so the dependency is honoured by the kernel boundary
+    // (about 2 us on this part, against 5..9 us for a grid barrier inside the persistent kernel).
+    // SQ_SEQ_ONE_LAUNCH keeps everything in one launch and uses the grid barrier.
+    int l0 = 0;
+    while (l0 < count) {
+        int l1 = l0 + 1;
+        while (l1 < count && (mode == SQ_SEQ_ONE_LAUNCH || !probs[l1].depends)) l1++;
+        bool done = false;
+        if (ws_ok && M <= 4 && (l1 - l0 > 1 || mode == SQ_SEQ_ONE_LAUNCH)) {
+            const int rc = sq::launch_gemv_seq(probs + l0, l1 - l0, M, workspace, 1u << 20, st);
+            if (rc == 2) return SQ_ERR_LAUNCH;
+            done = (rc == 0);
+        }
+        if (!done) {
+            // a single linear, more than 4 tokens, no workspace, or activations beyond the LDS: one launch per linear
+            for (int l = l0; l < l1; l++) {
+                const sq::SeqProblem& q = probs[l];
+                const sq::Epilogue epi{static_cast<const sq::half_t*>(q.bias), static_cast<const sq::half_t*>(q.residual),
+                                       q.act};
+                const int rc = gemm_dispatch(q.x, q.w, q.zs, q.y, M, q.N, q.K, q.group_size, layout, SQ_ALGO_AUTO, epi,
+                                             nullptr, 0, stream);
+                if (rc != SQ_OK) return rc;
+            }
+        }
+        l0 = l1;
+    }
+    return SQ_OK;
+}
+
 int sq_w4a16_gemm_fused(const void* x, const void* w, const void* zs, const void* bias, const void* residual, void* y,
                         int M, int N, int K, int group_size, int layout, int act, int algo, void* workspace,
                         size_t workspace_bytes, void* stream) {

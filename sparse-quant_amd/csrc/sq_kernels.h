@@ -26,6 +26,26 @@ hipError_t launch_2bit_to_4bit(const void* src, void* dst, int N, int K, hipStre
 // sq_gemv2.hip: M <= 8, streaming formulation.  tune = waves per workgroup (1,2,4,8).
 hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
                               bool fixup, int tune, Epilogue epi, hipStream_t st);
+// sq_gemv_seq.hip: up to SEQ_MAX_LINEARS decode linears (M <= 4) in one persistent launch.
+constexpr int SEQ_MAX_LINEARS = 8;
+constexpr size_t SEQ_LDS_LIMIT = 156 * 1024;
+struct SeqProblem {
+    const void* x;
+    const void* w;
+    const void* zs;
+    const void* bias;
+    const void* residual;
+    void* y;
+    int N, K, group_size, act, depends;
+};
+size_t gemv_seq_workspace_bytes();
+// 0: launched; 1: the sequence does not fit this kernel (the caller launches the linears one by
+// one); 2: the HIP runtime rejected the launch.  workspace: gemv_seq_workspace_bytes() bytes, zero
+// between launches.  spin_limit bounds the polls of a grid barrier.
+// trace (diagnostic, normally null): 64 uint64 per workgroup, time stamps of the 100 MHz counter.
+int launch_gemv_seq(const SeqProblem* probs, int count, int M, void* workspace, unsigned spin_limit, hipStream_t st,
+                    unsigned long long* trace = nullptr);
+
 // sq_skinny.hip: M <= 64.  tune = waves | mode << 8 (mode 1 = exact, 2 = fixup).
 hipError_t launch_skinny_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,
                                int tune, Epilogue epi, hipStream_t st);

@@ -27,7 +27,7 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 PROBES_PATH = os.path.join(PKG_ROOT, "libsq_probes.so")
 
-HIP_SOURCES = ["sq_api.hip", "sq_dequant.hip", "sq_repack.hip", "sq_gemv2.hip", "sq_skinny.hip", "sq_skinny2.hip",
+HIP_SOURCES = ["sq_api.hip", "sq_dequant.hip", "sq_repack.hip", "sq_gemv2.hip", "sq_gemv_seq.hip", "sq_skinny.hip", "sq_skinny2.hip",
                "sq_gemm.hip", "sq_gemm2.hip", "sq_attn.hip", "sq_decode_attn.hip", "sq_layernorm.hip"]
 PROBE_SOURCES = ["sq_probes.hip"]  # diagnostic kernels, a library of their own (include/sq_probes.h)
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
@@ -40,6 +40,7 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-W
 # shuttle them through the accumulation registers (hundreds of v_accvgpr moves otherwise).
 PER_FILE_FLAGS = {
     "sq_gemv2.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "sq_gemv_seq.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "sq_skinny2.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "sq_attn.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
 }
@@ -69,7 +70,9 @@ def build_lib(verbose=True):
     with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
         list(pool.map(compile_one, zip(sources, objs)))
     n = len(HIP_SOURCES)
-    for path, part in ((LIB_PATH, objs[:n]), (PROBES_PATH, objs[n:])):
+    # the diagnostic library carries its own copy of the sequence kernel (for its time-stamping instantiation)
+    seq_obj = [o for o in objs[:n] if o.endswith("sq_gemv_seq.o")]
+    for path, part in ((LIB_PATH, objs[:n]), (PROBES_PATH, objs[n:] + seq_obj)):
         _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", path] + part +
              ["-Wl,-rpath," + os.path.join(ROCM, "lib")])
         if verbose:

@@ -49,7 +49,21 @@ PROBE_SIGNATURES = {
     "sq_clock_probe": (_i, [_vp, _i, _vp]),
     "sq_mfma_probe": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_read_probe": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sq_sequence_trace": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
 }
+
+
+
+class LinearDesc(ctypes.Structure):
+    """sq_linear_desc of include/sq_w4a16.h."""
+    _fields_ = [("x", _vp), ("w", _vp), ("zs", _vp), ("bias", _vp), ("residual", _vp), ("y", _vp),
+                ("N", _i), ("K", _i), ("group_size", _i), ("act", _i), ("depends", _i)]
+
+
+SIGNATURES["sq_w4a16_gemv_sequence"] = (_i, [ctypes.POINTER(LinearDesc), _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp])
+SQ_SEQ_AUTO, SQ_SEQ_ONE_LAUNCH = 0, 1
+SIGNATURES["sq_w4a16_gemv_sequence_workspace_bytes"] = (ctypes.c_size_t, [])
+SQ_SEQUENCE_MAX = 8
 
 _lib = None
 _probes = None
@@ -186,6 +200,37 @@ def gemm_fused(x, w, zs, n, k, group_size, bias=None, residual=None, act=SQ_ACT_
     return out
 
 
+class LinearSequence:
+    """Up to SQ_SEQUENCE_MAX decode linears bound once, launched with one call (sq_w4a16_gemv_sequence).
+
+    linears: list of dicts with keys x, w, zs, y (tensors), n, k, group_size and optionally bias,
+    residual, act, depends.  The descriptor array and the workspace are kept; `run()` only launches."""
+
+    def __init__(self, linears, m, device, workspace=True, mode=SQ_SEQ_AUTO):
+        self.count = len(linears)
+        self.m = int(m)
+        self.mode = int(mode)
+        self.descs = (LinearDesc * max(self.count, 1))()
+        self.keep = list(linears)
+        for d, l in zip(self.descs, linears):
+            d.x, d.w, d.zs, d.y = l["x"].data_ptr(), l["w"].data_ptr(), l["zs"].data_ptr(), l["y"].data_ptr()
+            d.bias = l["bias"].data_ptr() if l.get("bias") is not None else None
+            d.residual = l["residual"].data_ptr() if l.get("residual") is not None else None
+            d.N, d.K, d.group_size = int(l["n"]), int(l["k"]), int(l["group_size"])
+            d.act, d.depends = int(l.get("act", SQ_ACT_NONE)), int(bool(l.get("depends", False)))
+        self.ws = torch.zeros(lib().sq_w4a16_gemv_sequence_workspace_bytes(), dtype=torch.uint8,
+                              device=device) if workspace else None
+        self._fn = lib().sq_w4a16_gemv_sequence
+
+    def run(self, stream=None):
+        _check(self._fn(self.descs, self.count, self.m, SQ_LAYOUT_L1, self.mode, _ptr(self.ws),
+                        0 if self.ws is None else self.ws.numel(), _stream(stream)), "sq_w4a16_gemv_sequence")
+
+    def error_flag(self):
+        """The sticky error word of the workspace (synchronises): non-zero if a grid barrier ran out of polls."""
+        return 0 if self.ws is None else int(self.ws.view(torch.int32)[9].item())
+
+
 def dequant(w, zs, n, k, group_size, layout=SQ_LAYOUT_L1, stream=None):
     out = torch.empty((n, k), dtype=torch.float16, device=w.device)
     _check(lib().sq_w4a16_dequant(_ptr(w), _ptr(zs), _ptr(out), n, k, group_size, layout, _stream(stream)),
@@ -299,6 +344,21 @@ def layernorm(x, gamma, beta, eps=1e-5, out=None, stream=None):
     _check(lib().sq_layernorm(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(out), x.numel() // cols, cols, float(eps),
                               _stream(stream)), "sq_layernorm")
     return out
+
+
+def sequence_trace(linears, m, group_size, stream=None):
+    """Run the linears (dicts with x, w, zs, y, n, k, depends) through the time-stamping instantiation of the
+    sequence kernel; returns an int64 tensor [workgroups, 64] of 100 MHz counter readings (see sq_probes.h)."""
+    cnt = len(linears)
+    dev = linears[0]["x"].device
+    arr = lambda key: (ctypes.c_void_p * cnt)(*[l[key].data_ptr() for l in linears])
+    ints = lambda key: (ctypes.c_int * cnt)(*[int(l.get(key, 0)) for l in linears])
+    ws = torch.zeros(256, dtype=torch.uint8, device=dev)
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    trace = torch.zeros((cus, 64), dtype=torch.int64, device=dev)
+    _check(probes().sq_sequence_trace(arr("x"), arr("w"), arr("zs"), arr("y"), ints("n"), ints("k"), ints("depends"), cnt,
+                                      int(m), int(group_size), _ptr(ws), _ptr(trace), _stream(stream)), "sq_sequence_trace")
+    return trace
 
 
 def mfma_probe(data, workgroups, iters, stream=None):
