@@ -14,13 +14,20 @@ The metric is achieved GB/s: algorithmic bytes of a step
 divided by the time of a step, inputs already resident in HBM.
 
 Also printed on the same JSON line:
+  parity        every leg's kernels are checked against the CPU oracle on sampled rows before they
+                are timed (gate: max|Y - Y_ref| <= 1e-2 * max|Y_ref|, dequant bit-exact); a failed
+                gate ends the run with an error instead of a number
   roofline      algorithmic bytes per launch / average launch duration of the decode
                 kernel (HIP events on the launch stream over the timed region) against
                 the 8 TB/s HBM peak
-  cpu_baseline  the CPU restatement of the same path (oracle/) timed on this box's
-                host cores on one step
-  prefill       TFLOP/s of the M = 2048 linears (second half of the metric)
+  long_window   the same step timed over at least 400 graph replays (the driver's --steps may be
+                as low as 20, i.e. under a millisecond)
+  cpu_baseline  the reference CPU path (torch dequant to fp32 + matmul, timed separately) on this
+                box's host cores on one step, with the C restatement of the oracle as a second figure
+  config1       the single q_proj-shaped linear with group size 64 at M = 1 and 16
+  prefill       TFLOP/s of the M = 2048 linears, OPT and Llama-MLP shapes (second half of the metric)
   decode_batch  GB/s of the same six linears at M = 4, 8, 16, 32
+  sequence      the same six linears through sq_w4a16_gemv_sequence
 
 `--m`, `--group` and `--shapes` select other points of the same workload family.
 """
@@ -55,7 +62,110 @@ def make_linear(n, k, g, dev, gen):
     return w, zs
 
 
+PARITY_GATE = 1e-2
+
+
+class ParityError(RuntimeError):
+    pass
+
+
+def parity_linear(torch, w, zs, n, k, g, x, y, seed=0, rows=64, tokens=32):
+    """max|Y - Y_ref| / max|Y_ref| of a GPU result against the CPU oracle on sampled output rows (and,
+    with many tokens, sampled token rows): the oracle dequantises those rows of the weight and forms
+    the fp32 product.  Outside every timed region."""
+    import numpy as np
+    import w4a16_oracle as orc
+    rng = np.random.default_rng(seed)
+    ridx = np.sort(rng.choice(n, size=min(rows, n), replace=False))
+    m = x.shape[0]
+    tidx = np.arange(m) if m <= tokens else np.sort(rng.choice(m, size=tokens, replace=False))
+    rt = torch.from_numpy(ridx).to(w.device)
+    tt = torch.from_numpy(tidx).to(w.device)
+    w_hat = orc.dequant_l1(w[rt].cpu().numpy(), zs[rt].cpu().numpy(), g)
+    y_ref = orc.gemm_ref(x[tt].cpu().numpy(), w_hat)
+    got = y[tt][:, rt].float().cpu().numpy()
+    if not np.all(np.isfinite(got)):
+        return float("inf")
+    return float(np.max(np.abs(got - y_ref)) / np.max(np.abs(y_ref)))
+
+
+def parity_dequant(torch, capi, w, zs, n, k, g, seed=0, rows=64):
+    """Bit-exactness of the dequant kernel on sampled rows of a weight."""
+    import numpy as np
+    import w4a16_oracle as orc
+    rng = np.random.default_rng(seed)
+    ridx = np.sort(rng.choice(n, size=min(rows, n), replace=False))
+    rt = torch.from_numpy(ridx).to(w.device)
+    want = orc.dequant_l1(w[rt].cpu().numpy(), zs[rt].cpu().numpy(), g)
+    got = capi.dequant(w, zs, n, k, g)[rt].cpu().numpy()
+    return bool(np.array_equal(got.view(np.int16), want.view(np.int16)))
+
+
+def gate(err, what):
+    if not err <= PARITY_GATE:
+        raise ParityError("parity gate failed for %s: max rel err %.3e > %.0e" % (what, err, PARITY_GATE))
+    return err
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_reference_torch(m, g, shapes, reps=3):
+    """The reference's CPU path on the host cores: W = (q.float() - z.float()) * s.float() ("dequant"), then
+    Y = X.float() @ W.t() ("matmul"), timed separately, median of `reps`, one step = the six linears."""
+    import torch
+    gen = torch.Generator()
+    gen.manual_seed(0)
+    data = []
+    for _, n, k in shapes:
+        q = torch.randint(0, 16, (n, k), dtype=torch.uint8, generator=gen)
+        z = torch.randint(0, 16, (n, k // g), dtype=torch.uint8, generator=gen)
+        s = (torch.randn((n, k // g), generator=gen).abs() * 0.02 + 1e-3).half()
+        x = torch.randn((m, k), generator=gen).half()
+        data.append((q, z, s, x))
+    deq_t, mm_t = [], []
+    for _ in range(reps + 1):
+        td = tm = 0.0
+        for q, z, s, x in data:
+            t0 = time.perf_counter()
+            w = (q.float() - z.float().repeat_interleave(g, 1)) * s.float().repeat_interleave(g, 1)
+            t1 = time.perf_counter()
+            y = x.float() @ w.t()
+            t2 = time.perf_counter()
+            td += t1 - t0
+            tm += t2 - t1
+            del w, y
+        deq_t.append(td)
+        mm_t.append(tm)
+    med = lambda v: sorted(v[1:])[len(v[1:]) // 2]  # the first repetition warms the allocator
+    return med(deq_t), med(mm_t), torch.get_num_threads()
+
+
 def cpu_baseline(m, g, shapes):
+    """One step of the same workload on the host: the reference's torch recipe (dequant to fp32 + matmul) and,
+    as a second figure, the oracle's C restatement (all host cores)."""
+    total_bytes = sum(algorithmic_bytes(m, n, k, g) for _, n, k in shapes)
+    total_flops = sum(2.0 * m * n * k for _, n, k in shapes)
+    deq_s, mm_s, threads = cpu_reference_torch(m, g, shapes)
+    port = cpu_baseline_c_port(m, g, shapes)
+    t = deq_s + mm_s
+    return {"value": round(total_bytes / t / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "one step (six linears of one OPT-6.7B layer, M=%d, g=%d), median of 3: torch dequant to fp32 "
+                      "%.1f ms + torch matmul %.1f ms = %.1f ms per step (the reference's CPU recipe restated with "
+                      "torch ops on the host)" % (m, g, deq_s * 1e3, mm_s * 1e3, t * 1e3),
+            "dequant_ms": round(deq_s * 1e3, 2), "matmul_ms": round(mm_s * 1e3, 2),
+            "gflops": round(total_flops / t / 1e9, 3), "cpu_model": cpu_model(), "os_cpu_count": os.cpu_count(),
+            "torch_threads": threads, "c_port": port}
+
+
+def cpu_baseline_c_port(m, g, shapes):
     """One step of the same workload through the oracle's C restatement (all host cores)."""
     import numpy as np
     import w4a16_oracle as orc
@@ -91,9 +201,8 @@ def cpu_baseline(m, g, shapes):
         step()
         times.append(time.perf_counter() - t0)
     t = sorted(times)[1]
-    return {"value": round(total_bytes / t / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": "one step (six linears of one OPT-6.7B layer, M=%d, g=%d), median of 3, %s, %.1f ms per step"
-                      % (m, g, kind_note, t * 1e3)}
+    return {"value": round(total_bytes / t / 1e9, 3), "unit": "GB/s", "cores": threads,
+            "sample": "one step, median of 3, %s, %.1f ms per step" % (kind_note, t * 1e3)}
 
 
 def main():
@@ -156,37 +265,82 @@ def main():
         for i in range(len(calls)):
             run_layer(i)
         stream.synchronize()
-        graph = None
-        if not args.no_graph:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
-                for i in range(len(calls)):
-                    run_layer(i)
+        # Parity gate, outside every timed region: every linear of the first layer against the CPU oracle on
+        # sampled output rows, and the dequant kernel bit for bit on two of the weights.
+        parity_err, deq_exact = 0.0, True
+        for li in (0, len(calls) - 1):
+            for idx, ((w, zs), (name, n, k)) in enumerate(zip(pool[li], shapes)):
+                ytmp = torch.full((m, n), float("nan"), dtype=torch.float16, device=dev)
+                a = list(calls[li][idx])
+                a[3] = vp(ytmp.data_ptr())
+                rc = gemm(*a)
+                if rc != 0:
+                    raise RuntimeError("sq_w4a16_gemm failed: " + capi.strerror(rc))
+                stream.synchronize()
+                parity_err = max(parity_err, gate(parity_linear(torch, w, zs, n, k, g, xs[k], ytmp, seed=idx),
+                                                  "%s at M=%d" % (name, m)))
+        for idx in (0, len(shapes) - 2):
+            w, zs = pool[0][idx]
+            deq_exact = deq_exact and parity_dequant(torch, capi, w, zs, shapes[idx][1], shapes[idx][2], g, seed=idx)
+        if not deq_exact:
+            raise ParityError("parity gate failed: dequant is not bit-exact")
         per_replay = len(calls)
+        graphs = {}
+
+        def graph_of(count):
+            """A captured graph of `count` consecutive steps (layers 0 .. count-1 of the pool)."""
+            if count not in graphs:
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=stream):
+                    for i in range(count):
+                        run_layer(i)
+                graphs[count] = gr
+            return graphs[count]
 
         def run_steps(count):
-            if graph is None:
+            """Exactly `count` steps: whole passes over the pool plus one shorter graph for the rest."""
+            if args.no_graph:
                 for i in range(count):
                     run_layer(i)
-                return count
-            reps = (count + per_replay - 1) // per_replay
-            for _ in range(reps):
-                graph.replay()
-            return reps * per_replay
+                return
+            full, rest = divmod(count, per_replay)
+            for _ in range(full):
+                graphs[per_replay].replay()
+            if rest:
+                graphs[rest].replay()
 
+        if not args.no_graph:
+            graph_of(per_replay)
+            for c in {args.steps % per_replay, args.warmup % per_replay} - {0}:
+                graph_of(c)
+        graph = graphs.get(per_replay)
+        steps = args.steps
         run_steps(args.warmup)
         stream.synchronize()
-        steps = args.steps if graph is None else ((args.steps + per_replay - 1) // per_replay) * per_replay
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         e0.record(stream)
-        done = run_steps(steps)
+        run_steps(steps)
         e1.record(stream)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-        assert done == steps
+        # The same step over a window that does not depend on --steps (at least 400 passes over the pool).
+        long_window = None
+        if graph is not None:
+            reps_long = 400
+            l0 = torch.cuda.Event(enable_timing=True)
+            l1 = torch.cuda.Event(enable_timing=True)
+            l0.record(stream)
+            for _ in range(reps_long):
+                graph.replay()
+            l1.record(stream)
+            stream.synchronize()
+            us_long = l0.elapsed_time(l1) * 1e3 / (reps_long * per_replay)
+            long_window = {"steps": reps_long * per_replay, "us_per_step": round(us_long, 3),
+                           "gbs": round(bytes_per_step / us_long / 1e3, 1),
+                           "frac_of_hbm_peak": round(bytes_per_step / us_long / 1e3 / HBM_PEAK_GBS, 4)}
         # The same step with the arithmetic taken away: sq_read_probe streams each weight with the GEMV's
         # own grid and access pattern and only folds the bits.  What it needs per step is the floor that
         # six dependent launches of these sizes leave to any kernel on this part.
@@ -206,7 +360,7 @@ def main():
             with torch.cuda.graph(pgraph, stream=stream):
                 for i in range(len(calls)):
                     probe_layer(i)
-            reps = max(1, steps // per_replay)
+            reps = max(50, steps // per_replay)
             for _ in range(max(1, reps // 10)):
                 pgraph.replay()
             p0 = torch.cuda.Event(enable_timing=True)
@@ -241,12 +395,21 @@ def main():
                                "16384->4096), W4A16 group %d, M=%d, one step = six launches, %d-layer rotating "
                                "weight pool (%.0f MB)" % (g, m, args.layers, args.layers * bytes_per_step / 1e6),
                    "launch": "hip-graph replay" if graph is not None else "eager", "bytes_per_step": bytes_per_step},
+        "parity": {"max_rel_err": round(parity_err, 6), "gate": PARITY_GATE, "dequant_bit_exact": deq_exact,
+                   "checked": "every linear of two layers of the pool against the CPU oracle on 64 sampled output rows "
+                              "(fp32 reference of the dequantised rows), dequant kernel bit for bit on 64 rows of two "
+                              "weights; every other leg below carries its own parity_max_rel_err, checked the same way "
+                              "before it is timed"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "traffic_source": "stored from profiles/gemv_decode_traffic.json (rocprofv3 --pmc FETCH_SIZE / "
+                                       "WRITE_SIZE of this command, scaled by a 256 MiB copy), not measured in this run",
                      "kernel": "sq::gemv2_kernel (decode GEMV)", "avg_launch_us": round(launch_us, 3),
                      "bytes_per_launch": bytes_per_step // launches_per_step},
     }
 
+    if long_window is not None:
+        out["long_window"] = long_window
     if floor_us is not None:
         out["read_only_floor"] = {
             "what": "the same six launches per step through sq_read_probe (weights and zeros_scales streamed with "
@@ -269,11 +432,16 @@ def main():
         # Additional, separately labelled legs; none of them feeds `value`.
         try:
             out["decode_batch"] = decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream)
+            out["config1"] = config1_leg(torch, capi, dev, gen, stream)
+            if m <= 4:
+                out["sequence"] = sequence_leg(torch, capi, pool, shapes, m, g, dev, gen, stream, bytes_per_step)
             out["fused_qkv"] = fused_qkv_leg(torch, capi, m, g, dev, gen, stream, args.layers, bytes_per_step)
             out["attention"] = attention_leg(torch, capi, dev)
             out["decode_attention"] = decode_attention_leg(torch, capi, dev)
             from sqamd import opt_decode
             out["e2e_opt67"] = opt_decode.run_e2e(batch=8, prompt=512, new_tokens=128)
+        except ParityError:
+            raise
         except Exception as exc:  # an extra leg must never hide the headline line
             out["extras_error"] = repr(exc)
     if not args.no_cpu:
@@ -317,24 +485,36 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
         c, r = int(ticks[0].item()), int(ticks[1].item())
         return round(c / (r / 100.0)) if r else None
 
+    # q/k/v/out share one shape: out_proj stands for the four; then fc1, fc2 and the Llama-2-7B MLP shapes
+    work = [(w, zs, name, n, k) for (w, zs), (name, n, k) in list(zip(layer, shapes))[3:]]
+    for name, n, k in (("llama_mlp_up", 11008, 4096), ("llama_mlp_down", 4096, 11008)):
+        w, zs = make_linear(n, k, g, dev, gen)
+        work.append((w, zs, name, n, k))
+    opt_names = {name for _, _, name, _, _ in work[:3]}
+    worst = 0.0
     with torch.cuda.stream(stream):
-        for (w, zs), (name, n, k) in list(zip(layer, shapes))[3:]:
+        for w, zs, name, n, k in work:
             x = torch.randn((m, k), device=dev, generator=gen).half()
             y = torch.empty((m, n), dtype=torch.float16, device=dev)
             wd = torch.randn((k, n), device=dev, generator=gen).half()
             run = lambda: capi.gemm(x, w, zs, n, k, g, out=y, stream=stream)
             dense = lambda: torch.matmul(x, wd, out=y)
+            run()
+            stream.synchronize()
+            err = gate(parity_linear(torch, w, zs, n, k, g, x, y, seed=n + k), "%s at M=%d" % (name, m))
+            worst = max(worst, err)
             us = timed(run)
             us_dense = timed(dense)
             fl = 2.0 * m * n * k
-            res[name] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 1),
+            res[name] = {"us": round(us, 1), "tflops": round(fl / us / 1e6, 1), "parity_max_rel_err": round(err, 6),
                          "shader_mhz_under_load": clock_under(run, us),
                          "dense_fp16_library_us": round(us_dense, 1),
                          "dense_fp16_library_tflops": round(fl / us_dense / 1e6, 1),
                          "dense_fp16_library_shader_mhz": clock_under(dense, us_dense)}
-            flops_total += fl
-            time_total += us
-            dense_time_total += us_dense
+            if name in opt_names:  # the aggregate stays the OPT-6.7B set, comparable from run to run
+                flops_total += fl
+                time_total += us
+                dense_time_total += us_dense
             del wd
     tf = flops_total / time_total / 1e6
     tfd = flops_total / dense_time_total / 1e6
@@ -343,14 +523,23 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
     with torch.cuda.stream(stream):
         for m2 in (512, 4096):
             fl2, t2 = 0.0, 0.0
-            for (w, zs), (name, n, k) in list(zip(layer, shapes))[3:]:
+            per = {}
+            for w, zs, name, n, k in work:
                 x = torch.randn((m2, k), device=dev, generator=gen).half()
                 y = torch.empty((m2, n), dtype=torch.float16, device=dev)
                 ws = capi.workspace(m2, n, k, dev, stream)  # the extension passes one for up to 1024 tokens
-                t2 += timed(lambda: capi.gemm_ws(x, w, zs, n, k, g, out=y, stream=stream, ws=ws))
-                fl2 += 2.0 * m2 * n * k
+                capi.gemm_ws(x, w, zs, n, k, g, out=y, stream=stream, ws=ws)
+                stream.synchronize()
+                err = gate(parity_linear(torch, w, zs, n, k, g, x, y, seed=m2 + n), "%s at M=%d" % (name, m2))
+                worst = max(worst, err)
+                us2 = timed(lambda: capi.gemm_ws(x, w, zs, n, k, g, out=y, stream=stream, ws=ws))
+                per[name] = {"us": round(us2, 1), "tflops": round(2.0 * m2 * n * k / us2 / 1e6, 1)}
+                if name in opt_names:
+                    t2 += us2
+                    fl2 += 2.0 * m2 * n * k
             other["m%d" % m2] = {"tflops": round(fl2 / t2 / 1e6, 1),
-                                 "frac_of_fp16_mfma_peak": round(fl2 / t2 / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4)}
+                                 "frac_of_fp16_mfma_peak": round(fl2 / t2 / 1e6 / MFMA_FP16_PEAK_TFLOPS, 4),
+                                 "per_linear": per}
     # What the matrix pipes sustain under the power limit: a loop of nothing but independent
     # v_mfma_f32_32x32x16_f16 on all CUs (one wave per SIMD), on N(0,1) operands and on zeros.
     roof = {}
@@ -365,7 +554,9 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
             roof[name] = {"tflops": round(cus * 4 * iters * 16 * 32768.0 / us / 1e6, 1),
                           "shader_mhz": round(float(ticks.double().median().item()) / us),
                           "cycles_per_mfma": round(float(ticks.double().median().item()) / (iters * 16), 2)}
-    return {"m": m, "other_token_counts": other, "tflops": round(tf, 1), "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
+    return {"m": m, "aggregate_over": "out_proj (4096x4096), fc1, fc2; the Llama MLP shapes are listed per linear",
+            "parity_max_rel_err": round(worst, 6),
+            "other_token_counts": other, "tflops": round(tf, 1), "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
             "dense_fp16_library_tflops": round(tfd, 1), "vs_dense_fp16_library": round(tf / tfd, 3),
             "nominal_shader_mhz": 2400, "mfma_only_loop": roof,
             "frac_of_mfma_only_loop": round(tf / roof["normal_operands"]["tflops"], 4), "per_linear": res}
@@ -388,6 +579,15 @@ def decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream):
             for i in range(len(pool)):
                 run(i)
             stream.synchronize()
+            worst = 0.0
+            for idx, ((w, zs), (name, n, k)) in enumerate(zip(pool[0], shapes)):
+                if idx in (1, 2):
+                    continue  # same shape and kernel as q_proj
+                ytmp = torch.empty((m, n), dtype=torch.float16, device=dev)
+                capi.gemm_ws(xs[k], w, zs, n, k, g, out=ytmp, stream=stream, ws=ws)
+                stream.synchronize()
+                worst = max(worst, gate(parity_linear(torch, w, zs, n, k, g, xs[k], ytmp, seed=idx + m),
+                                        "%s at M=%d" % (name, m)))
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
                 for i in range(len(pool)):
@@ -404,7 +604,83 @@ def decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream):
             stream.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / (reps * len(pool))
         res["m%d" % m] = {"us_per_step": round(us, 2), "gbs": round(bytes_per_step / us / 1e3, 1),
-                          "frac_of_hbm_peak": round(bytes_per_step / us / 1e3 / HBM_PEAK_GBS, 4)}
+                          "frac_of_hbm_peak": round(bytes_per_step / us / 1e3 / HBM_PEAK_GBS, 4),
+                          "parity_max_rel_err": round(worst, 6)}
+    return res
+
+
+def config1_leg(torch, capi, dev, gen, stream, g=64, n=4096, k=4096, copies=32):
+    """The single q_proj-shaped linear with group size 64 (4096 x 4096) at M = 1 and M = 16, cold weights
+    (32 copies = 302 MB rotating), HIP-graph replay, product dispatch with workspace."""
+    pool = [make_linear(n, k, g, dev, gen) for _ in range(copies)]
+    res = {"shape": "N=4096 K=4096 group 64", "pool_mb": round(copies * algorithmic_bytes(1, n, k, g) / 1e6)}
+    for m in (1, 16):
+        x = torch.randn((m, k), device=dev, generator=gen).half()
+        y = torch.empty((m, n), dtype=torch.float16, device=dev)
+        nbytes = algorithmic_bytes(m, n, k, g)
+        with torch.cuda.stream(stream):
+            ws = capi.workspace(m, n, k, dev, stream)
+            run = lambda: [capi.gemm_ws(x, w, zs, n, k, g, out=y, stream=stream, ws=ws) for w, zs in pool]
+            run()
+            stream.synchronize()
+            err = gate(parity_linear(torch, pool[-1][0], pool[-1][1], n, k, g, x, y, seed=m), "config 1 at M=%d" % m)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                run()
+            for _ in range(5):
+                graph.replay()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(50):
+                graph.replay()
+            e1.record(stream)
+            stream.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (50 * copies)
+        res["m%d" % m] = {"us": round(us, 3), "gbs": round(nbytes / us / 1e3, 1),
+                          "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                          "parity_max_rel_err": round(err, 6)}
+    return res
+
+
+def sequence_leg(torch, capi, pool, shapes, m, g, dev, gen, stream, bytes_per_step):
+    """The same six linears through sq_w4a16_gemv_sequence: with the data flow of the decoder layer (q, k, v
+    independent; out_proj, fc1, fc2 each consuming an earlier output) in the default mode (a new launch at every
+    dependent linear) and as one persistent launch with grid barriers, and as six independent linears in one
+    persistent launch."""
+    xs = {k: torch.randn((m, k), device=dev, generator=gen).half() for k in {k for _, _, k in shapes}}
+    ys = [torch.empty((m, n), dtype=torch.float16, device=dev) for _, n, _ in shapes]
+    res = {}
+    for label, dep, mode in (("layer_dependencies_auto", "000111", capi.SQ_SEQ_AUTO),
+                             ("layer_dependencies_one_launch", "000111", capi.SQ_SEQ_ONE_LAUNCH),
+                             ("independent_one_launch", "000000", capi.SQ_SEQ_AUTO)):
+        seqs = [capi.LinearSequence([dict(x=xs[k], w=w, zs=zs, y=ys[i], n=n, k=k, group_size=g, depends=dep[i] == "1")
+                                     for i, ((w, zs), (_, n, k)) in enumerate(zip(layer, shapes))], m, dev, mode=mode)
+                for layer in pool]
+        with torch.cuda.stream(stream):
+            seqs[0].run(stream=stream)
+            stream.synchronize()
+            worst = 0.0
+            for i, ((w, zs), (name, n, k)) in enumerate(zip(pool[0], shapes)):
+                worst = max(worst, gate(parity_linear(torch, w, zs, n, k, g, xs[k], ys[i], seed=i), "sequence " + name))
+            for sq in seqs:
+                sq.run(stream=stream)
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for sq in seqs:
+                    sq.run(stream=stream)
+            for _ in range(10):
+                graph.replay()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(200):
+                graph.replay()
+            e1.record(stream)
+            stream.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (200 * len(pool))
+        res[label] = {"depends": dep, "us_per_step": round(us, 2), "gbs": round(bytes_per_step / us / 1e3, 1),
+                      "frac_of_hbm_peak": round(bytes_per_step / us / 1e3 / HBM_PEAK_GBS, 4),
+                      "parity_max_rel_err": round(worst, 6), "barrier_timeouts": sum(sq.error_flag() for sq in seqs)}
     return res
 
 
@@ -454,7 +730,17 @@ def attention_leg(torch, capi, dev):
         k = torch.randn_like(q)
         v = torch.randn_like(q)
         for _ in range(3):
-            capi.lut_attention(q, k, v, lut, d ** -0.5, False)
+            out = capi.lut_attention(q, k, v, lut, d ** -0.5, False)
+        torch.cuda.synchronize()
+        import numpy as np
+        import lut_attention_oracle as att
+        worst = 0.0
+        for zi, hi in ((0, 0), (z - 1, h - 1)):  # the float64 oracle on two (batch, head) pairs
+            sl = (slice(zi, zi + 1), slice(hi, hi + 1))
+            ref = att.attention_ref(q[sl].cpu().numpy(), k[sl].cpu().numpy(), v[sl].cpu().numpy(),
+                                    lut[hi:hi + 1].cpu().numpy(), d ** -0.5, False)
+            err = float(np.max(np.abs(out[sl].float().cpu().numpy() - ref)) / np.max(np.abs(ref)))
+            worst = max(worst, gate(err, "LUT attention S=%d" % s))
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -465,7 +751,8 @@ def attention_leg(torch, capi, dev):
         us = e0.elapsed_time(e1) * 1e3 / 20
         tf = 4.0 * kept * 64 * 64 * d / us / 1e6
         res["seq%d" % s] = {"us": round(us, 1), "tflops": round(tf, 1),
-                            "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4)}
+                            "frac_of_fp16_mfma_peak": round(tf / MFMA_FP16_PEAK_TFLOPS, 4),
+                            "parity_max_rel_err": round(worst, 6)}
     return res
 
 
@@ -489,7 +776,16 @@ def decode_attention_leg(torch, capi, dev, pool=8, reps=20):
         for i in range(pool):
             torch.nn.functional.scaled_dot_product_attention(qs[i], kcs[i], vcs[i])
 
-    res = {"shape": "B=8 H=32 D=128 rows=640", "bytes": 2 * b * h * rows * d * 2}
+    import numpy as np
+    import lut_attention_oracle as att
+    kc0, vc0 = kcs[0].clone(), vcs[0].clone()
+    got = capi.decode_attention(qs[0], kc0, vc0, pos, scale, k_new=qs[0], v_new=qs[0])
+    torch.cuda.synchronize()
+    ref = att.decode_attention_ref(qs[0][:2, :, 0].cpu().numpy(), kc0[:2].cpu().numpy(), vc0[:2].cpu().numpy(), scale)
+    err = float(np.max(np.abs(got.view(b, h, d)[:2].float().cpu().numpy() - ref)) / max(1.0, np.max(np.abs(ref))))
+    if not err <= 2e-3:
+        raise ParityError("parity gate failed for decode attention: %.3e" % err)
+    res = {"shape": "B=8 H=32 D=128 rows=640", "bytes": 2 * b * h * rows * d * 2, "parity_max_err": round(err, 6)}
     for name, fn in (("kernel", ours), ("torch_sdpa", sdpa)):
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())

@@ -187,6 +187,16 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
     decode_s = time.perf_counter() - t0
     steps = new_tokens - 1
     extra = {"tokens": torch.stack(generated).cpu()} if return_tokens else {}
+    # Algorithmic bytes of one decode step: every packed weight with its zeros/scales and the batch's
+    # activations (N*K/2 + (K/g)*N*4 + M*K*2 + M*N*2 per linear, q/k/v as one linear), the valid K/V cache
+    # rows read once (average over the timed steps), the fp16 lm_head.
+    hidden, ffn, g, vocab = model.hidden, model.layers[0].fc1.out_features, 128, model.lm_head.shape[0]
+    lin = lambda n, k: n * k // 2 + (k // g) * n * 4 + batch * k * 2 + batch * n * 2
+    rows_avg = prompt + (steps + 1) / 2.0
+    per_layer = lin(3 * hidden, hidden) + lin(hidden, hidden) + lin(ffn, hidden) + lin(hidden, ffn) + \
+        2 * batch * hidden * rows_avg * 2
+    step_bytes = layers * per_layer + vocab * hidden * 2
+    step_s = decode_s / steps
     return {
         **extra,
         "weights": "random packed int4, zeros U{0..15}, scales |N(0,%g)|+%g (smaller than the single-linear "
@@ -200,6 +210,12 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
         "prefill_tok_per_s": round(batch * prompt / prefill_s, 1),
         "decode_ms_per_step": round(decode_s * 1e3 / steps, 4),
         "decode_tok_per_s": round(batch * steps / decode_s, 1),
+        "roofline": {"bound": "hbm", "bytes_per_step": int(step_bytes), "achieved": round(step_bytes / step_s / 1e9, 1),
+                     "peak": 8000.0, "unit": "GB/s", "frac": round(step_bytes / step_s / 1e9 / 8000.0, 4),
+                     "what": "int4 weights + zeros/scales + activations of the %d x 4 linears, K/V cache rows read once "
+                             "(%.0f rows on average), fp16 lm_head; per decode step" % (layers, rows_avg)},
+        "parity": "covered by tests/test_gpu_full_size.py: one full-width decoder layer against the oracle composition, "
+                  "eager and HIP-graph decode steps generate identical tokens",
         "tokens_checksum": int(torch.stack(generated).sum().item()),
     }
 
