@@ -14,7 +14,9 @@
 //                 sm_scale*log2(e) and rounded to fp16 like the reference);
 //                 D: lane (query l%16) holds keys 16t + 4*(l/16) + v of key tile t.
 //   softmax     : over a lane's 16 values and the 4 lanes {l, l^16, l^32, l^48}; the
-//                 running max / sum of a query live in its lanes, nothing is exchanged.
+//                 reference maximum of a query lives in its lanes and moves lazily (only when
+//                 a score exceeds it by more than 2^8), the row sum stays split over the four
+//                 lanes until the end: in the common case nothing is exchanged or rescaled.
 //   O^T = V^T P^T: B = P^T is exactly what the lane already holds: for the k-step
 //                 covering keys 32s .. 32s+31 lane group g supplies keys 32s+4g+{0..3}
 //                 and 32s+16+4g+{0..3}; A = V^T rows read from an LDS copy of the V
@@ -43,7 +45,7 @@ __global__ __launch_bounds__(256 / QT) void lut_attn_kernel(const half_t* __rest
                                                             const half_t* __restrict__ V, half_t* __restrict__ O,
                                                             const void* __restrict__ lut, int lut_is_64, int H, int S,
                                                             int nblk_q, int nnz, int nvisit, float qk_scale,
-                                                            int causal) {
+                                                            int causal, int total_wg) {
     constexpr int NT = 256 / QT;                 // threads per workgroup
     constexpr int KP = D + SQ_ATTN_KPAD;         // halves per row of the K tile in LDS
     constexpr int VP = 64 + SQ_ATTN_VPAD;        // halves per row of the transposed V tile in LDS
@@ -59,8 +61,15 @@ __global__ __launch_bounds__(256 / QT) void lut_attn_kernel(const half_t* __rest
     const int wave = tid >> 6;
     const int lq = lane & 15;
     const int g = lane >> 4;
-    const int qb = blockIdx.x;
-    const int zh = blockIdx.y;
+    // Workgroups are handed to the eight XCDs round-robin by their linear id, and every XCD has its own L2.
+    // The id is therefore re-read as (XCD, slot): XCD x works through the x-th eighth of the (head, query block)
+    // list, so that all query blocks of a head, which visit the same K and V rows, share one L2
+    // instead of pulling those rows into all eight.
+    const int per_xcd = (total_wg + 7) >> 3;
+    const int work = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (work >= total_wg) return;
+    const int qb = work % nblk_q;
+    const int zh = work / nblk_q;
     const int h = zh % H;
     const long base = (long)zh * S * D;
     int m[QT];  // this lane's queries
@@ -156,12 +165,17 @@ __global__ __launch_bounds__(256 / QT) void lut_attn_kernel(const half_t* __rest
         const int n1 = advance();
         if (n1 >= 0) fetch(n1);
 
-        // S^T = K Q^T for the four 16-key tiles; a K operand serves all QT query tiles.
+        // S^T = K Q^T for the four 16-key tiles; a K operand serves all QT query tiles.  The accumulators
+        // start at -m_ref of the lane's query, so the matrix core delivers the scores already shifted by
+        // the reference maximum and the softmax needs no subtraction.
         float4_t st[QT][4];
 #pragma unroll
         for (int t = 0; t < 4; t++) {
 #pragma unroll
-            for (int qt = 0; qt < QT; qt++) st[qt][t] = (float4_t){0.f, 0.f, 0.f, 0.f};
+            for (int qt = 0; qt < QT; qt++) {
+                const float c = (m_i[qt] == -INFINITY) ? 0.f : -m_i[qt];
+                st[qt][t] = (float4_t){c, c, c, c};
+            }
 #pragma unroll
             for (int s = 0; s < DK; s++) {
                 const half8_t a = *(const half8_t*)(&ks[(16 * t + lq) * KP + 32 * s + 8 * g]);
@@ -186,39 +200,49 @@ __global__ __launch_bounds__(256 / QT) void lut_attn_kernel(const half_t* __rest
                         st[qt][t][v] = keep ? st[qt][t][v] : -INFINITY;
                     }
             }
-            // block maximum of this query
+            // Largest shifted score of this lane.  The reference maximum m_ref of a query moves only when a
+            // score exceeds it by more than 2^LAZY (or when it is still unset): until then p = exp2(s - m_ref)
+            // stays below 2^LAZY, well inside fp16, the final O = acc / l does not depend on the reference,
+            // and neither the accumulators nor the scores need rescaling.  The test is made per lane and
+            // voted over the wave; the maximum over a query's four lanes is formed only when it is needed.
+            constexpr float LAZY = 8.f;
             float mx = -INFINITY;
 #pragma unroll
             for (int t = 0; t < 4; t++)
 #pragma unroll
                 for (int v = 0; v < 4; v++) mx = fmaxf(mx, st[qt][t][v]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16));
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
-            const float m_new = fmaxf(m_i[qt], mx);
-            // A query with nothing visible so far keeps p = 0 and alpha = 1 (no NaN from inf - inf).
-            // exp2 is the bare v_exp_f32: arguments are <= 0 and results below the normal range
-            // may flush to zero, which is far below the fp16 resolution of P.
-            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-            const float alpha = (m_i[qt] == -INFINITY) ? (m_new == -INFINITY ? 1.f : 0.f)
-                                                       : __builtin_amdgcn_exp2f(m_i[qt] - m_new);
+            const bool unset = (m_i[qt] == -INFINITY);
+            if (__builtin_amdgcn_ballot_w64(mx > LAZY || (unset && mx > -INFINITY)) != 0) {
+                float mq = fmaxf(mx, __shfl_xor(mx, 16));
+                mq = fmaxf(mq, __shfl_xor(mq, 32));
+                const bool upd = mq > LAZY || (unset && mq > -INFINITY);
+                const float delta = upd ? mq : 0.f;
+                // a query without a reference so far has l = 0 and acc = 0: nothing to rescale
+                const float alpha = (upd && !unset) ? __builtin_amdgcn_exp2f(-delta) : 1.f;
+                m_i[qt] = upd ? (unset ? delta : m_i[qt] + delta) : m_i[qt];
+                l_i[qt] *= alpha;
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) st[qt][t][v] -= delta;
+#pragma unroll
+                for (int dt = 0; dt < DT; dt++) acc[qt][dt] *= alpha;
+            }
+            // p = exp2(shifted score) (bare v_exp_f32: exp2(-inf) = 0 for masked entries), rounded to fp16
+            // for the second product like the reference; the lane's share of the row sum is taken from the
+            // rounded pairs with one dot instruction per pair and stays in the lane until the end.
             float rs = 0.f;
 #pragma unroll
             for (int t = 0; t < 4; t++)
 #pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    const float p = __builtin_amdgcn_exp2f(st[qt][t][v] - m_use);  // exp2(-inf) = 0 for masked entries
-                    rs += p;
-                    pk[qt][t >> 1][4 * (t & 1) + v] = (half_t)p;
+                for (int v = 0; v < 4; v += 2) {
+                    const half2_t pp = {(half_t)__builtin_amdgcn_exp2f(st[qt][t][v]),
+                                        (half_t)__builtin_amdgcn_exp2f(st[qt][t][v + 1])};
+                    rs = __builtin_amdgcn_fdot2(pp, (half2_t){(half_t)1.f, (half_t)1.f}, rs, false);
+                    pk[qt][t >> 1][4 * (t & 1) + v] = pp.x;
+                    pk[qt][t >> 1][4 * (t & 1) + v + 1] = pp.y;
                 }
-            rs += __shfl_xor(rs, 16);
-            rs += __shfl_xor(rs, 32);
-            l_i[qt] = l_i[qt] * alpha + rs;
-            m_i[qt] = m_new;
-            // The accumulators are rescaled only when some query of the wave saw its maximum grow.
-            if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
-#pragma unroll
-                for (int dt = 0; dt < DT; dt++) acc[qt][dt] *= alpha;
-            }
+            l_i[qt] += rs;
         }
 
         // O^T += V^T P^T; a V operand serves all QT query tiles.
@@ -242,10 +266,13 @@ __global__ __launch_bounds__(256 / QT) void lut_attn_kernel(const half_t* __rest
     // O[m][16*dt + 4g + v] = acc / l.
 #pragma unroll
     for (int qt = 0; qt < QT; qt++) {
+        // the row sum of a query is spread over its four lanes
+        float l = l_i[qt] + __shfl_xor(l_i[qt], 16);
+        l += __shfl_xor(l, 32);
         if (m[qt] < S) {
             // A query row without any visible key has l = 0 and acc = 0: 0 * inf = NaN, which is
             // also what the reference's running sums produce for such a row.
-            const float inv = 1.f / l_i[qt];
+            const float inv = 1.f / l;
 #pragma unroll
             for (int dt = 0; dt < DT; dt++) {
                 half4_t o;
@@ -261,14 +288,15 @@ hipError_t launch_lut_attention(const void* q, const void* k, const void* v, voi
                                 int lut_elem_bytes, int Z, int H, int S, int D, int nnz, float sm_scale, int causal,
                                 hipStream_t st) {
     const int nblk = (S + 63) / 64;
-    const dim3 grid(nblk, Z * H);
+    const int total_wg = nblk * Z * H;
+    const dim3 grid(((total_wg + 7) / 8) * 8);
     const float qk_scale = sm_scale * 1.44269504f;
     const int use_nnz = nnz < nblk ? nnz : nblk;  // the reference clamps NNZ to ceil(S / 64) as well
     // (the LUT row pitch stays nnz even when fewer entries are visited)
 #define SQ_ATTN_LAUNCH(D_, QT_)                                                                                   \
     hipLaunchKernelGGL((lut_attn_kernel<D_, QT_>), grid, dim3(256 / QT_), 0, st, (const half_t*)q, (const half_t*)k, \
                        (const half_t*)v, (half_t*)o, lut, lut_elem_bytes == 8, H, S, nblk, nnz, use_nnz, qk_scale,   \
-                       causal)
+                       causal, total_wg)
     if (D == 64)
         SQ_ATTN_LAUNCH(64, 1);
     else
