@@ -109,6 +109,25 @@ int sq_w4a16_gemm_static_ws(const void* x, const void* w, const void* zs, void* 
                             int M, int N, int K, int group_size, int layout, int algo,
                             void* stream);
 
+/* Workspace hygiene (no counterpart in the reference).  Every workspace-taking entry point above
+ * and below relies on one invariant: the counter region at the start of its workspace (64 KiB for
+ * sq_w4a16_gemm_ws / _fused, 1 KiB for sq_decode_attention, all 256 bytes for
+ * sq_w4a16_gemv_sequence) is zero when a call starts, every call leaves it zero, and calls that
+ * share a workspace do not overlap in time.  Inside the kernels, partial results are exchanged
+ * between workgroups with stores and loads at the device-coherent cache level (sc1) followed by a
+ * wait for the stores and a relaxed agent-scope counter; no device-wide release / acquire fence is
+ * used, so correctness rests on that cache-policy behaviour of gfx950.  A launch that dies midway,
+ * or two streams sharing a workspace, can leave counters non-zero; later calls on that workspace
+ * would then never find a last arriver and leave their output unwritten.
+ *   sq_workspace_reset  clears `bytes` (a multiple of 4, workspace 16-byte aligned) with a small
+ *                       fill kernel on `stream` (not a memset node: safe under HIP-graph capture);
+ *                       use it at workspace creation and on error paths.
+ *   sq_workspace_check  debugging aid, the one entry point that SYNCHRONISES: copies the first
+ *                       min(bytes, 64 KiB) back on `stream`, waits, and returns SQ_ERR_WORKSPACE if
+ *                       any word is non-zero (a previous call did not complete, or calls raced). */
+int sq_workspace_reset(void* workspace, size_t bytes, void* stream);
+int sq_workspace_check(const void* workspace, size_t bytes, void* stream);
+
 /* Bytes sq_w4a16_gemm_ws / sq_w4a16_gemm_fused can use for this shape (8.06 MiB for
  * every decode batch with N <= 16384; up to tens of MiB for the GEMM split). */
 size_t sq_w4a16_workspace_bytes(int M, int N, int K);

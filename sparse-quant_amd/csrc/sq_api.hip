@@ -207,6 +207,30 @@ int sq_w4a16_gemm_static_ws(const void* x, const void* w, const void* zs, void* 
                          (size_t)SQ_STATIC_WS_BYTES, stream);
 }
 
+int sq_workspace_reset(void* workspace, size_t bytes, void* stream) {
+    if (!workspace) return SQ_ERR_NULL_POINTER;
+    if (!aligned16(workspace) || bytes % 4 != 0) return SQ_ERR_MISALIGNED;
+    if (bytes == 0) return SQ_OK;
+    if (bytes > ((size_t)1 << 30)) return SQ_ERR_BAD_SHAPE;
+    const int words = (int)(bytes / 4);
+    hipLaunchKernelGGL(zero_words_kernel, dim3((words + 255) / 256), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<unsigned*>(workspace), words);
+    return launch_code(hipGetLastError());
+}
+
+int sq_workspace_check(const void* workspace, size_t bytes, void* stream) {
+    if (!workspace) return SQ_ERR_NULL_POINTER;
+    if (bytes % 4 != 0) return SQ_ERR_MISALIGNED;
+    if (bytes > 65536) bytes = 65536;
+    static thread_local unsigned host[65536 / 4];
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (hipMemcpyAsync(host, workspace, bytes, hipMemcpyDeviceToHost, st) != hipSuccess) return SQ_ERR_LAUNCH;
+    if (hipStreamSynchronize(st) != hipSuccess) return SQ_ERR_LAUNCH;
+    for (size_t i = 0; i < bytes / 4; i++)
+        if (host[i] != 0u) return SQ_ERR_WORKSPACE;
+    return SQ_OK;
+}
+
 size_t sq_w4a16_gemv_sequence_workspace_bytes(void) { return sq::gemv_seq_workspace_bytes(); }
 
 int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int layout, int mode, void* workspace,

@@ -30,6 +30,8 @@ SIGNATURES = {
     "sq_w4a16_gemm_static_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "sq_w4a16_gemm_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp]),
     "sq_w4a16_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
+    "sq_workspace_reset": (_i, [_vp, ctypes.c_size_t, _vp]),
+    "sq_workspace_check": (_i, [_vp, ctypes.c_size_t, _vp]),
     "sq_w4a16_dequant": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "sq_transpose_merge_zeros_scales": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "sq_convert_ours_to_awq": (_i, [_vp, _vp, _i, _i, _vp]),
@@ -155,6 +157,20 @@ def workspace(m, n, k, device, stream=None):
     need = lib().sq_w4a16_workspace_bytes(m, n, k)
     key = (str(device), (stream or torch.cuda.current_stream()).cuda_stream)
     return _cached_workspace(key, max(need, 1 << 20), device)
+
+
+def workspace_reset(ws, nbytes=None, stream=None):
+    """Clear the first nbytes (default: all) of a workspace tensor with the library's fill kernel."""
+    n = ws.numel() if nbytes is None else int(nbytes)
+    _check(lib().sq_workspace_reset(_ptr(ws), n - n % 4, _stream(stream)), "sq_workspace_reset")
+
+
+def workspace_is_clean(ws, nbytes=65536, stream=None):
+    """Debugging aid (synchronises): True if the counter region of a workspace is all zero."""
+    rc = lib().sq_workspace_check(_ptr(ws), min(int(nbytes), ws.numel()) // 4 * 4, _stream(stream))
+    if rc not in (SQ_OK, SQ_ERR_WORKSPACE):
+        raise SqError(rc, "sq_workspace_check")
+    return rc == SQ_OK
 
 
 def gemm_ws(x, w, zs, n, k, group_size, algo=SQ_ALGO_AUTO, out=None, stream=None, ws=None):

@@ -391,6 +391,28 @@ def test_skinny_ws_properties_and_workspace_reuse(capi):
     check_gemm_ws(capi, 100, 256, 1024, 128, capi.SQ_ALGO_AUTO)
 
 
+def test_workspace_check_and_reset(capi):
+    """The debug check reports a workspace whose counters are not zero (what a launch that died midway or two
+    racing streams would leave), the reset kernel repairs it, and a call on the repaired workspace is right."""
+    m, n, k, g = 16, 264, 2048, 128
+    ws = torch.zeros(capi.lib().sq_w4a16_workspace_bytes(m, n, k), dtype=torch.uint8, device=DEV)
+    assert capi.workspace_is_clean(ws)
+    d = linear(n, k, g, 3)
+    x = to_dev(orc.synth_x(m, k, seed=4))
+    good = capi.gemm_ws(x, d["w_dev"], d["zs_dev"], n, k, g, algo=capi.SQ_ALGO_SKINNY_WS | (4 << 8), ws=ws)
+    torch.cuda.synchronize()
+    assert capi.workspace_is_clean(ws)            # every call leaves the counters zero
+    ws[8] = 1                                     # simulate a stale counter
+    assert not capi.workspace_is_clean(ws)
+    capi.workspace_reset(ws, 65536)
+    assert capi.workspace_is_clean(ws)
+    again = capi.gemm_ws(x, d["w_dev"], d["zs_dev"], n, k, g, algo=capi.SQ_ALGO_SKINNY_WS | (4 << 8), ws=ws)
+    assert torch.equal(good, again)
+    L = capi.lib()
+    assert L.sq_workspace_check(None, 64, None) == capi.SQ_ERR_NULL_POINTER
+    assert L.sq_workspace_reset(ws.data_ptr() + 4, 64, None) == capi.SQ_ERR_MISALIGNED
+
+
 def test_skinny_ws_rejects_small_workspace(capi):
     d = linear(256, 1024, 128, seed=0)
     x = to_dev(orc.synth_x(16, 1024))
