@@ -20,8 +20,8 @@ Also printed on the same JSON line:
   roofline      algorithmic bytes per launch / average launch duration of the decode
                 kernel (HIP events on the launch stream over the timed region) against
                 the 8 TB/s HBM peak
-  long_window   the same step timed over at least 400 graph replays (the driver's --steps may be
-                as low as 20, i.e. under a millisecond)
+  long_window   the same step timed over 3200 steps whatever --steps says (the driver's --steps may
+                be as low as 20, i.e. under a millisecond)
   cpu_baseline  the reference CPU path (torch dequant to fp32 + matmul, timed separately) on this
                 box's host cores on one step, with the C restatement of the oracle as a second figure
   config1       the single q_proj-shaped linear with group size 64 at M = 1 and 16
@@ -214,6 +214,9 @@ def main():
     ap.add_argument("--group", type=int, default=128)
     ap.add_argument("--layers", type=int, default=8, help="distinct layers in the rotating weight pool")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--per-linear", action="store_true",
+                    help="headline through one sq_w4a16_gemm call per linear (six launches per step) instead of "
+                         "sq_w4a16_gemv_sequence")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 TFLOP/s leg")
     ap.add_argument("--no-extras", action="store_true",
@@ -239,9 +242,14 @@ def main():
 
     pool = [[make_linear(n, k, g, dev, gen) for _, n, k in shapes] for _ in range(args.layers)]
     xs = {k: torch.randn((m, k), device=dev, generator=gen).half() for k in {k for _, _, k in shapes}}
-    ys = {n: torch.empty((m, n), dtype=torch.float16, device=dev) for n in {n for _, n, _ in shapes}}
+    ys = [torch.empty((m, n), dtype=torch.float16, device=dev) for _, n, _ in shapes]  # one output per linear
     bytes_per_step = sum(algorithmic_bytes(m, n, k, g) for _, n, k in shapes)
-    launches_per_step = len(shapes)
+    # The step goes through sq_w4a16_gemv_sequence with the data flow of the decoder layer: q, k and v do not depend
+    # on each other (one launch for the three), out_proj, fc1 and fc2 each consume an earlier output (a launch
+    # each): four launches per step.  With more than 4 tokens, or --per-linear, one sq_w4a16_gemm per linear.
+    use_sequence = (m <= 4) and not args.per_linear
+    depends = [False, False, False, True, True, True]
+    launches_per_step = 4 if use_sequence else len(shapes)
 
     stream = torch.cuda.Stream(device=dev)
     vp = ctypes.c_void_p
@@ -249,13 +257,21 @@ def main():
     calls = []
     for layer in pool:
         row = []
-        for (w, zs), (_, n, k) in zip(layer, shapes):
-            row.append((vp(xs[k].data_ptr()), vp(w.data_ptr()), vp(zs.data_ptr()), vp(ys[n].data_ptr()), m, n, k, g,
+        for idx, ((w, zs), (_, n, k)) in enumerate(zip(layer, shapes)):
+            row.append((vp(xs[k].data_ptr()), vp(w.data_ptr()), vp(zs.data_ptr()), vp(ys[idx].data_ptr()), m, n, k, g,
                         capi.SQ_LAYOUT_L1, st))
         calls.append(row)
     gemm = lib.sq_w4a16_gemm
+    seqs = None
+    if use_sequence:
+        seqs = [capi.LinearSequence([dict(x=xs[k], w=w, zs=zs, y=ys[idx], n=n, k=k, group_size=g, depends=depends[idx])
+                                     for idx, ((w, zs), (_, n, k)) in enumerate(zip(layer, shapes))], m, dev,
+                                    workspace=False) for layer in pool]
 
     def run_layer(i):
+        if seqs is not None:
+            seqs[i % len(seqs)].run(stream=stream)
+            return
         for a in calls[i % len(calls)]:
             rc = gemm(*a)
             if rc != 0:
@@ -269,15 +285,12 @@ def main():
         # sampled output rows, and the dequant kernel bit for bit on two of the weights.
         parity_err, deq_exact = 0.0, True
         for li in (0, len(calls) - 1):
+            for y in ys:
+                y.fill_(float("nan"))
+            run_layer(li)
+            stream.synchronize()
             for idx, ((w, zs), (name, n, k)) in enumerate(zip(pool[li], shapes)):
-                ytmp = torch.full((m, n), float("nan"), dtype=torch.float16, device=dev)
-                a = list(calls[li][idx])
-                a[3] = vp(ytmp.data_ptr())
-                rc = gemm(*a)
-                if rc != 0:
-                    raise RuntimeError("sq_w4a16_gemm failed: " + capi.strerror(rc))
-                stream.synchronize()
-                parity_err = max(parity_err, gate(parity_linear(torch, w, zs, n, k, g, xs[k], ytmp, seed=idx),
+                parity_err = max(parity_err, gate(parity_linear(torch, w, zs, n, k, g, xs[k], ys[idx], seed=idx),
                                                   "%s at M=%d" % (name, m)))
         for idx in (0, len(shapes) - 2):
             w, zs = pool[0][idx]
@@ -287,8 +300,10 @@ def main():
         per_replay = len(calls)
         graphs = {}
 
+        unit = 64  # steps per replayed graph: eight passes over the pool, so that gaps between graph launches are rare
+
         def graph_of(count):
-            """A captured graph of `count` consecutive steps (layers 0 .. count-1 of the pool)."""
+            """A captured graph of `count` consecutive steps (cycling through the layers of the pool)."""
             if count not in graphs:
                 gr = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(gr, stream=stream):
@@ -303,44 +318,75 @@ def main():
                 for i in range(count):
                     run_layer(i)
                 return
-            full, rest = divmod(count, per_replay)
+            full, rest = divmod(count, unit)
             for _ in range(full):
-                graphs[per_replay].replay()
+                graphs[unit].replay()
             if rest:
                 graphs[rest].replay()
 
         if not args.no_graph:
-            graph_of(per_replay)
-            for c in {args.steps % per_replay, args.warmup % per_replay} - {0}:
+            graph_of(unit)
+            for c in {args.steps % unit, args.warmup % unit} - {0}:
                 graph_of(c)
-        graph = graphs.get(per_replay)
+        graph = graphs.get(unit)
         steps = args.steps
         run_steps(args.warmup)
         stream.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        e0.record(stream)
-        run_steps(steps)
-        e1.record(stream)
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        # The same step over a window that does not depend on --steps (at least 400 passes over the pool).
+        # The timed region is the GPU time of exactly `steps` steps between two events on the launch stream.  It is
+        # queued directly behind a longer untimed-for-the-headline window of the same steps (3200 of them, with
+        # events of its own: `long_window`), without a host synchronisation in between: the host has then
+        # submitted the timed steps before the first event fires and the chip is at its working clocks, which
+        # matters when --steps is small (20 steps are about 0.6 ms, less than the host needs to submit them
+        # after an idle period).
         long_window = None
+        t0 = time.perf_counter()
         if graph is not None:
-            reps_long = 400
+            reps_long = 50
             l0 = torch.cuda.Event(enable_timing=True)
             l1 = torch.cuda.Event(enable_timing=True)
             l0.record(stream)
             for _ in range(reps_long):
                 graph.replay()
             l1.record(stream)
-            stream.synchronize()
-            us_long = l0.elapsed_time(l1) * 1e3 / (reps_long * per_replay)
-            long_window = {"steps": reps_long * per_replay, "us_per_step": round(us_long, 3),
+        e0.record(stream)
+        run_steps(steps)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        if graph is not None:
+            us_long = l0.elapsed_time(l1) * 1e3 / (reps_long * unit)
+            long_window = {"steps": reps_long * unit, "us_per_step": round(us_long, 3),
                            "gbs": round(bytes_per_step / us_long / 1e3, 1),
                            "frac_of_hbm_peak": round(bytes_per_step / us_long / 1e3 / HBM_PEAK_GBS, 4)}
+        # The same step with one sq_w4a16_gemm launch per linear (six launches), for comparison.
+        per_linear = None
+        if seqs is not None and graph is not None:
+            def six(i):
+                for a in calls[i]:
+                    rc = gemm(*a)
+                    if rc != 0:
+                        raise RuntimeError("sq_w4a16_gemm failed: " + capi.strerror(rc))
+            for i in range(len(calls)):
+                six(i)
+            stream.synchronize()
+            g6 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g6, stream=stream):
+                for i in range(len(calls)):
+                    six(i)
+            for _ in range(20):
+                g6.replay()
+            s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s0.record(stream)
+            for _ in range(200):
+                g6.replay()
+            s1.record(stream)
+            stream.synchronize()
+            us6 = s0.elapsed_time(s1) * 1e3 / (200 * per_replay)
+            per_linear = {"launches_per_step": 6, "us_per_step": round(us6, 3), "gbs": round(bytes_per_step / us6 / 1e3, 1),
+                          "frac_of_hbm_peak": round(bytes_per_step / us6 / 1e3 / HBM_PEAK_GBS, 4)}
         # The same step with the arithmetic taken away: sq_read_probe streams each weight with the GEMV's
         # own grid and access pattern and only folds the bits.  What it needs per step is the floor that
         # six dependent launches of these sizes leave to any kernel on this part.
@@ -371,9 +417,9 @@ def main():
             p1.record(stream)
             stream.synchronize()
             floor_us = p0.elapsed_time(p1) * 1e3 / (reps * per_replay)
-    wall_ms = (t1 - t0) * 1e3
+    wall_ms = (t1 - t0) * 1e3  # host wall clock over the long window and the timed steps: reported, not used
     gpu_ms = e0.elapsed_time(e1)
-    ms_per_step = wall_ms / steps
+    ms_per_step = gpu_ms / steps
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
     launch_us = gpu_ms * 1e3 / (steps * launches_per_step)
     achieved = (bytes_per_step / launches_per_step) / (launch_us * 1e-6) / 1e9
@@ -389,11 +435,16 @@ def main():
     out = {
         "metric": "W4A16 linear GB/s at M=1 (OPT-6.7B decoder-layer linears, cold weights)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms_per_step, 6), "timed_region": "HIP events on the launch stream around exactly `steps` "
+        "steps, queued behind the 3200 steps of long_window (host wall clock over both: %.3f ms)" % wall_ms,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int4 weights x fp16 activations, fp32 accumulate", "data": "synthetic",
         "config": {"workload": "OPT-6.7B decoder-layer linears (q,k,v,out 4096x4096; fc1 4096->16384; fc2 "
-                               "16384->4096), W4A16 group %d, M=%d, one step = six launches, %d-layer rotating "
-                               "weight pool (%.0f MB)" % (g, m, args.layers, args.layers * bytes_per_step / 1e6),
+                               "16384->4096), W4A16 group %d, M=%d, one step = the six linears through %s, %d-layer "
+                               "rotating weight pool (%.0f MB)"
+                               % (g, m, "sq_w4a16_gemv_sequence with the layer's data flow (q, k, v in one launch; out_proj, "
+                                        "fc1, fc2 a launch each: four launches)" if use_sequence else
+                                  "one sq_w4a16_gemm each (six launches)", args.layers, args.layers * bytes_per_step / 1e6),
                    "launch": "hip-graph replay" if graph is not None else "eager", "bytes_per_step": bytes_per_step},
         "parity": {"max_rel_err": round(parity_err, 6), "gate": PARITY_GATE, "dequant_bit_exact": deq_exact,
                    "checked": "every linear of two layers of the pool against the CPU oracle on 64 sampled output rows "
@@ -404,16 +455,19 @@ def main():
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "traffic_source": "stored from profiles/gemv_decode_traffic.json (rocprofv3 --pmc FETCH_SIZE / "
                                        "WRITE_SIZE of this command, scaled by a 256 MiB copy), not measured in this run",
-                     "kernel": "sq::gemv2_kernel (decode GEMV)", "avg_launch_us": round(launch_us, 3),
+                     "kernel": "sq::gemv2_kernel / sq::gemv2_group_kernel (decode GEMV)",
+                     "launches_per_step": launches_per_step, "avg_launch_us": round(launch_us, 3),
                      "bytes_per_launch": bytes_per_step // launches_per_step},
     }
 
     if long_window is not None:
         out["long_window"] = long_window
+    if per_linear is not None:
+        out["per_linear_launches"] = per_linear
     if floor_us is not None:
         out["read_only_floor"] = {
-            "what": "the same six launches per step through sq_read_probe (weights and zeros_scales streamed with "
-                    "the GEMV's grid and access pattern, no arithmetic, no activations, no output)",
+            "what": "six launches per step (one per linear) through sq_read_probe (weights and zeros_scales streamed "
+                    "with the single-linear GEMV's grid and access pattern, no arithmetic, no activations, no output)",
             "us_per_step": round(floor_us, 2), "gbs": round(bytes_per_step / floor_us / 1e3, 1),
             "frac_of_hbm_peak": round(bytes_per_step / floor_us / 1e3 / HBM_PEAK_GBS, 4),
             "value_over_floor": round(floor_us / (ms_per_step * 1e3), 4)}
@@ -563,8 +617,10 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
 
 
 def decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream):
-    """GB/s of the same six linears at decode batches M = 4, 8, 16, 32 (the other batch sizes of the decode configuration), through
-    the product dispatch with its workspace (sq_w4a16_gemm_ws), HIP-graph replay over the rotating pool."""
+    """GB/s of the same six linears at decode batches M = 4, 8, 16, 32 (the other batch sizes of the decode configuration):
+    M = 4 through sq_w4a16_gemv_sequence like the headline (q, k, v in one launch), larger batches through the
+    product dispatch with its workspace (sq_w4a16_gemm_ws), one launch per linear; HIP-graph replay over the
+    rotating pool."""
     res = {}
     for m in (4, 8, 16, 32):
         xs = {k: torch.randn((m, k), device=dev, generator=gen).half() for k in {k for _, _, k in shapes}}
@@ -572,20 +628,36 @@ def decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream):
         bytes_per_step = sum(algorithmic_bytes(m, n, k, g) for _, n, k in shapes)
         with torch.cuda.stream(stream):
             ws = capi.workspace(m, 16384, 16384, dev, stream)
+            seqs = None
+            if m <= 4:
+                yl = [torch.empty((m, n), dtype=torch.float16, device=dev) for _, n, _ in shapes]
+                dep = [False, False, False, True, True, True]
+                seqs = [capi.LinearSequence([dict(x=xs[k], w=w, zs=zs, y=yl[i], n=n, k=k, group_size=g, depends=dep[i])
+                                             for i, ((w, zs), (_, n, k)) in enumerate(zip(layer, shapes))], m, dev,
+                                            workspace=False) for layer in pool]
 
             def run(i):
+                if seqs is not None:
+                    seqs[i % len(pool)].run(stream=stream)
+                    return
                 for (w, zs), (_, n, k) in zip(pool[i % len(pool)], shapes):
                     capi.gemm_ws(xs[k], w, zs, n, k, g, out=ys[n], stream=stream, ws=ws)
             for i in range(len(pool)):
                 run(i)
             stream.synchronize()
             worst = 0.0
-            for idx, ((w, zs), (name, n, k)) in enumerate(zip(pool[0], shapes)):
-                if idx in (1, 2):
-                    continue  # same shape and kernel as q_proj
-                ytmp = torch.empty((m, n), dtype=torch.float16, device=dev)
-                capi.gemm_ws(xs[k], w, zs, n, k, g, out=ytmp, stream=stream, ws=ws)
+            if seqs is not None:
+                seqs[0].run(stream=stream)
                 stream.synchronize()
+            for idx, ((w, zs), (name, n, k)) in enumerate(zip(pool[0], shapes)):
+                if seqs is not None:
+                    ytmp = yl[idx]
+                else:
+                    if idx in (1, 2):
+                        continue  # same shape and kernel as q_proj
+                    ytmp = torch.empty((m, n), dtype=torch.float16, device=dev)
+                    capi.gemm_ws(xs[k], w, zs, n, k, g, out=ytmp, stream=stream, ws=ws)
+                    stream.synchronize()
                 worst = max(worst, gate(parity_linear(torch, w, zs, n, k, g, xs[k], ytmp, seed=idx + m),
                                         "%s at M=%d" % (name, m)))
             graph = torch.cuda.CUDAGraph()
@@ -605,7 +677,7 @@ def decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream):
         us = e0.elapsed_time(e1) * 1e3 / (reps * len(pool))
         res["m%d" % m] = {"us_per_step": round(us, 2), "gbs": round(bytes_per_step / us / 1e3, 1),
                           "frac_of_hbm_peak": round(bytes_per_step / us / 1e3 / HBM_PEAK_GBS, 4),
-                          "parity_max_rel_err": round(worst, 6)}
+                          "launches_per_step": 4 if seqs is not None else 6, "parity_max_rel_err": round(worst, 6)}
     return res
 
 

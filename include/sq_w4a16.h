@@ -155,25 +155,29 @@ int sq_w4a16_gemm_fused(const void* x, const void* w, const void* zs, const void
  * executed in order.  No counterpart in the reference, which launches its GEMV once per linear
  * (quantization/muxi/backend/w4a16_gemm.cuh:14-326 under test/muxi/module/qlinear/qlinear.py:61-70);
  * at one token every such launch spends about as long getting started as streaming its weights.
- * Linears that do not depend on each other (q, k and v of a decoder layer) are served by ONE
- * persistent launch: one workgroup per CU stays resident and the weight stream never stops between
- * linears.
+ * Consecutive linears that do not depend on each other and share K and the group size (q, k and v
+ * of a decoder layer, kept as three weights) are served by ONE launch of the decode GEMV whose grid
+ * is the concatenation of their row blocks; a linear that depends on an earlier one starts a new
+ * launch.
  *   depends  set it on linear l when x_l or residual_l (or any buffer it reads) is written by an
  *            earlier linear of the same call.  Linears without it may run ahead of earlier ones.
  *            A buffer written by linear i may be read or overwritten by linear j > i only if j, or
  *            a linear between them, has depends set; y_l must not alias x_l or residual_l.
- *   mode     SQ_SEQ_AUTO: a linear with depends starts a new launch (the kernel boundary is the
- *            cheapest dependency on this part); SQ_SEQ_ONE_LAUNCH: everything in one persistent
- *            launch, dependencies honoured by a grid barrier inside the kernel (slower today; kept
- *            for measurement).
- *   workspace  sq_w4a16_gemv_sequence_workspace_bytes() bytes (256), 16-byte aligned, zero before
+ *   mode     SQ_SEQ_AUTO: as above (the kernel boundary is the cheapest dependency on this part);
+ *            SQ_SEQ_ONE_LAUNCH: everything in one persistent launch (one workgroup per CU stays
+ *            resident, the weight stream never stops between linears, dependencies are honoured by a
+ *            grid barrier inside the kernel); faster than one launch per linear only when nothing
+ *            depends on anything, kept for that case and for measurement.
+ *   workspace  used by SQ_SEQ_ONE_LAUNCH only (may be NULL otherwise):
+ *            sq_w4a16_gemv_sequence_workspace_bytes() bytes (256), 16-byte aligned, zero before
  *            the first call (every call leaves it zero); calls that share it must be ordered.
  *            Word 9 of it is a sticky error flag: it becomes 1 if a grid barrier ever ran out of
  *            polls (results of that call are then undefined).
- * Shapes as for sq_w4a16_gemm (all linears share M).  With M > 4, without a workspace, or when the
- * activations of a linear do not fit the LDS (M * K * 2 bytes beyond about 128 KiB), the linears are
- * launched one by one on the stream instead: same results.  The persistent kernel needs every
- * workgroup resident at once (one per CU); other work running on the GPU only delays it. */
+ * Shapes as for sq_w4a16_gemm (all linears share M).  With M > 4, K > 8192 or a lone linear the
+ * linears are launched one by one on the stream (the automatic dispatch of sq_w4a16_gemm): same
+ * results.  SQ_SEQ_ONE_LAUNCH falls back to the same when there is no workspace, M > 4, or the
+ * activations of a linear do not fit the LDS (M * K * 2 bytes beyond about 128 KiB); its persistent
+ * kernel needs every workgroup resident at once (one per CU); other work on the GPU only delays it. */
 #define SQ_SEQ_AUTO 0
 #define SQ_SEQ_ONE_LAUNCH 1
 #define SQ_SEQUENCE_MAX 8

@@ -259,22 +259,33 @@ int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int 
     if (M == 0) return SQ_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool ws_ok = workspace && aligned16(workspace) && workspace_bytes >= sq::gemv_seq_workspace_bytes();
-    // Runs of linears without a dependency between them go out as one persistent launch each; a linear that
-    // depends on an earlier one starts a new run, so the dependency is honoured by the kernel boundary
-    // (about 2 us on this part, against 5..9 us for a grid barrier inside the persistent kernel).
-    // SQ_SEQ_ONE_LAUNCH keeps everything in one launch and uses the grid barrier.
+    if (mode == SQ_SEQ_ONE_LAUNCH && ws_ok && M <= 4) {
+        // everything in one persistent launch, dependencies honoured by a grid barrier inside the kernel
+        const int rc = sq::launch_gemv_seq(probs, count, M, workspace, 1u << 20, st);
+        if (rc == 0) return SQ_OK;
+        if (rc == 2) return SQ_ERR_LAUNCH;
+    }
+    // A linear that depends on an earlier one starts a new launch: the kernel boundary is the cheapest way to
+    // honour a dependency on this part (about 2 us, against 5..9 us for a grid barrier inside a persistent
+    // kernel).  Consecutive linears that do not depend on each other and share K and the group size (q, k and
+    // v of a decoder layer) go out as ONE launch of the single-linear GEMV whose grid is the concatenation of
+    // their row blocks.  Everything else (more than 4 tokens, K beyond 8192, a lone linear) is one launch per
+    // linear through the automatic dispatch.
     int l0 = 0;
     while (l0 < count) {
         int l1 = l0 + 1;
-        while (l1 < count && (mode == SQ_SEQ_ONE_LAUNCH || !probs[l1].depends)) l1++;
+        while (l1 < count && l1 - l0 < sq::GEMV_GROUP_MAX && !probs[l1].depends && probs[l1].K == probs[l0].K &&
+               probs[l1].group_size == probs[l0].group_size)
+            l1++;
         bool done = false;
-        if (ws_ok && M <= 4 && (l1 - l0 > 1 || mode == SQ_SEQ_ONE_LAUNCH)) {
-            const int rc = sq::launch_gemv_seq(probs + l0, l1 - l0, M, workspace, 1u << 20, st);
-            if (rc == 2) return SQ_ERR_LAUNCH;
-            done = (rc == 0);
+        if (l1 - l0 > 1 && M <= 4 && probs[l0].K <= 8192) {
+            const hipError_t e = sq::launch_gemv2_group(probs + l0, l1 - l0, M, st);
+            if (e == hipSuccess)
+                done = true;
+            else if (e != hipErrorInvalidValue)
+                return SQ_ERR_LAUNCH;
         }
         if (!done) {
-            // a single linear, more than 4 tokens, no workspace, or activations beyond the LDS: one launch per linear
             for (int l = l0; l < l1; l++) {
                 const sq::SeqProblem& q = probs[l];
                 const sq::Epilogue epi{static_cast<const sq::half_t*>(q.bias), static_cast<const sq::half_t*>(q.residual),

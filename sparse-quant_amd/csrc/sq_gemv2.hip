@@ -35,11 +35,9 @@
 namespace sq {
 
 template <int MROWS, int NR, int KS, int S, bool FIXUP>
-__global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __restrict__ W,
-                                                             const half2_t* __restrict__ ZS,
-                                                             const half_t* __restrict__ X,
-                                                             half_t* __restrict__ Y, int M, int N, int K,
-                                                             int gshift, Epilogue epi) {
+__device__ __forceinline__ void gemv2_body(const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS,
+                                           const half_t* __restrict__ X, half_t* __restrict__ Y, int M, int N, int K,
+                                           int gshift, const Epilogue& epi, int blk) {
     constexpr int MT = (MROWS + 3) / 4;
     // Fixup mode, where the zero point is applied: with up to 4 tokens through per-run activation
     // sums staged beside the activations; with more, where that vector arithmetic starts to
@@ -63,7 +61,7 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
     const int wq_ = wave / NR;  // k range of this wave
     const int i = lane & 3;
     const int b = lane >> 2;
-    const int out_row = blockIdx.x * (4 * NR) + 4 * wr + i;
+    const int out_row = blk * (4 * NR) + 4 * wr + i;
     const int row = imin(out_row, N - 1);
     const int groups = K >> gshift;
     const int nsteps = (K + 511) >> 9;
@@ -208,10 +206,69 @@ __global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __re
             float sum = 0.f;
 #pragma unroll
             for (int q = 0; q < KS; q++) sum += red[q][r][m][ri];
-            const int orow = blockIdx.x * (4 * NR) + 4 * r + ri;
+            const int orow = blk * (4 * NR) + 4 * r + ri;
             if (orow < N && m < M) Y[(long)m * N + orow] = epilogue(sum, m, orow, N, epi);
         }
     }
+}
+
+template <int MROWS, int NR, int KS, int S, bool FIXUP>
+__global__ __launch_bounds__(64 * NR * KS) void gemv2_kernel(const uint8_t* __restrict__ W,
+                                                             const half2_t* __restrict__ ZS,
+                                                             const half_t* __restrict__ X,
+                                                             half_t* __restrict__ Y, int M, int N, int K,
+                                                             int gshift, Epilogue epi) {
+    gemv2_body<MROWS, NR, KS, S, FIXUP>(W, ZS, X, Y, M, N, K, gshift, epi, blockIdx.x);
+}
+
+// Up to four linears that do not depend on each other and share M, K and the group size (q, k and v of a
+// decoder layer) in one launch: the grid is the concatenation of their row blocks, a workgroup looks its
+// linear up by its block index and then runs the single-linear body unchanged.
+struct Gemv2Group {
+    const uint8_t* W[GEMV_GROUP_MAX];
+    const half2_t* ZS[GEMV_GROUP_MAX];
+    const half_t* X[GEMV_GROUP_MAX];
+    half_t* Y[GEMV_GROUP_MAX];
+    const half_t* bias[GEMV_GROUP_MAX];
+    const half_t* residual[GEMV_GROUP_MAX];
+    int N[GEMV_GROUP_MAX];
+    int act[GEMV_GROUP_MAX];
+    int blk_end[GEMV_GROUP_MAX];  // first block index behind linear p
+    int count;
+};
+
+template <int MROWS, int NR, int KS, int S, bool FIXUP>
+__global__ __launch_bounds__(64 * NR * KS) void gemv2_group_kernel(const Gemv2Group grp, int M, int K, int gshift) {
+    int p = 0;
+#pragma unroll
+    for (int q = 0; q < GEMV_GROUP_MAX - 1; q++)
+        if (q + 1 < grp.count && (int)blockIdx.x >= grp.blk_end[q]) p = q + 1;
+    const int blk = blockIdx.x - (p > 0 ? grp.blk_end[p - 1] : 0);
+    const Epilogue epi{grp.bias[p], grp.residual[p], grp.act[p]};
+    gemv2_body<MROWS, NR, KS, S, FIXUP>(grp.W[p], grp.ZS[p], grp.X[p], grp.Y[p], M, grp.N[p], K, gshift, epi, blk);
+}
+
+template <int MROWS, int NR, int KS, int S>
+static hipError_t launch_group_cfg(const SeqProblem* probs, int count, int M, int K, int gshift, hipStream_t st) {
+    Gemv2Group g;
+    int blocks = 0;
+    for (int p = 0; p < GEMV_GROUP_MAX; p++) {
+        const SeqProblem& q = probs[p < count ? p : 0];
+        g.W[p] = (const uint8_t*)q.w;
+        g.ZS[p] = (const half2_t*)q.zs;
+        g.X[p] = (const half_t*)q.x;
+        g.Y[p] = (half_t*)q.y;
+        g.bias[p] = (const half_t*)q.bias;
+        g.residual[p] = (const half_t*)q.residual;
+        g.N[p] = q.N;
+        g.act[p] = q.act;
+        if (p < count) blocks += (q.N + 4 * NR - 1) / (4 * NR);
+        g.blk_end[p] = blocks;
+    }
+    g.count = count;
+    hipLaunchKernelGGL((gemv2_group_kernel<MROWS, NR, KS, S, true>), dim3(blocks), dim3(64 * NR * KS), 0, st, g, M, K,
+                       gshift);
+    return hipGetLastError();
 }
 
 template <int MROWS, int NR, int KS, int S>
@@ -276,6 +333,41 @@ hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void
     if (M <= 2) return launch_rows<2>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
     if (M <= 4) return launch_rows<4>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
     return launch_rows<8>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
+}
+
+// Grouped launch (fixup arithmetic, as the automatic dispatch uses): count in 2..GEMV_GROUP_MAX linears with
+// the same K <= 8192 and group size, M <= 4.  Returns hipErrorInvalidValue when the group does not qualify.
+hipError_t launch_gemv2_group(const SeqProblem* probs, int count, int M, hipStream_t st) {
+    if (count < 2 || count > GEMV_GROUP_MAX || M < 1 || M > 4) return hipErrorInvalidValue;
+    const int K = probs[0].K, g = probs[0].group_size;
+    for (int p = 1; p < count; p++)
+        if (probs[p].K != K || probs[p].group_size != g) return hipErrorInvalidValue;
+    const int nsteps = (K + 511) / 512;
+    if (nsteps > 16) return hipErrorInvalidValue;
+    int gshift = 0;
+    while ((1 << gshift) < g) gshift++;
+    // the single-linear choices for a weight of this K: one k range, four row groups (two k ranges for 3..4
+    // tokens on K >= 4096), all k-steps of a wave in one round
+    const int ks = (M >= 3 && nsteps >= 8) ? 2 : 1;
+    const int spw = (nsteps + ks - 1) / ks;
+#define SQ_GROUP(MR_, KS_, S_) return launch_group_cfg<MR_, 4, KS_, S_>(probs, count, M, K, gshift, st)
+    if (M <= 1) {
+        if (spw >= 8) SQ_GROUP(1, 1, 8);
+        if (spw >= 4) SQ_GROUP(1, 1, 4);
+        SQ_GROUP(1, 1, 2);
+    }
+    if (M <= 2) {
+        if (spw >= 8) SQ_GROUP(2, 1, 8);
+        if (spw >= 4) SQ_GROUP(2, 1, 4);
+        SQ_GROUP(2, 1, 2);
+    }
+    if (ks == 2) {
+        if (spw >= 4) SQ_GROUP(4, 2, 4);
+        SQ_GROUP(4, 2, 2);
+    }
+    if (spw >= 4) SQ_GROUP(4, 1, 4);
+    SQ_GROUP(4, 1, 2);
+#undef SQ_GROUP
 }
 
 }  // namespace sq

@@ -38,6 +38,11 @@ struct SeqProblem {
     void* y;
     int N, K, group_size, act, depends;
 };
+// sq_gemv2.hip: 2..GEMV_GROUP_MAX independent decode linears with equal K (<= 8192) and group size, M <= 4, as one
+// launch of the single-linear GEMV (the grid is the concatenation of their row blocks).  hipErrorInvalidValue
+// when the group does not qualify.
+constexpr int GEMV_GROUP_MAX = 4;
+hipError_t launch_gemv2_group(const SeqProblem* probs, int count, int M, hipStream_t st);
 size_t gemv_seq_workspace_bytes();
 // 0: launched; 1: the sequence does not fit this kernel (the caller launches the linears one by
 // one); 2: the HIP runtime rejected the launch.  workspace: gemv_seq_workspace_bytes() bytes, zero
