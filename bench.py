@@ -617,10 +617,9 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
 
 
 def decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream):
-    """GB/s of the same six linears at decode batches M = 4, 8, 16, 32 (the other batch sizes of the decode configuration):
-    M = 4 through sq_w4a16_gemv_sequence like the headline (q, k, v in one launch), larger batches through the
-    product dispatch with its workspace (sq_w4a16_gemm_ws), one launch per linear; HIP-graph replay over the
-    rotating pool."""
+    """GB/s of the same six linears at decode batches M = 4, 8, 16, 32 (the other batch sizes of the decode configuration),
+    through sq_w4a16_gemv_sequence like the headline (q, k, v in one launch, the others a launch each, split-K
+    workspace for 5..32 tokens); HIP-graph replay over the rotating pool."""
     res = {}
     for m in (4, 8, 16, 32):
         xs = {k: torch.randn((m, k), device=dev, generator=gen).half() for k in {k for _, _, k in shapes}}
@@ -629,12 +628,14 @@ def decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream):
         with torch.cuda.stream(stream):
             ws = capi.workspace(m, 16384, 16384, dev, stream)
             seqs = None
-            if m <= 4:
+            if m <= 32:
                 yl = [torch.empty((m, n), dtype=torch.float16, device=dev) for _, n, _ in shapes]
                 dep = [False, False, False, True, True, True]
                 seqs = [capi.LinearSequence([dict(x=xs[k], w=w, zs=zs, y=yl[i], n=n, k=k, group_size=g, depends=dep[i])
                                              for i, ((w, zs), (_, n, k)) in enumerate(zip(layer, shapes))], m, dev,
                                             workspace=False) for layer in pool]
+                for sq in seqs:  # one shared split-K workspace (the calls are ordered on one stream)
+                    sq.ws = ws
 
             def run(i):
                 if seqs is not None:

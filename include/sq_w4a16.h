@@ -156,8 +156,9 @@ int sq_w4a16_gemm_fused(const void* x, const void* w, const void* zs, const void
  * (quantization/muxi/backend/w4a16_gemm.cuh:14-326 under test/muxi/module/qlinear/qlinear.py:61-70);
  * at one token every such launch spends about as long getting started as streaming its weights.
  * Consecutive linears that do not depend on each other and share K and the group size (q, k and v
- * of a decoder layer, kept as three weights) are served by ONE launch of the decode GEMV whose grid
- * is the concatenation of their row blocks; a linear that depends on an earlier one starts a new
+ * of a decoder layer, kept as three weights) are served by ONE launch whose grid is the
+ * concatenation of their row blocks (the decode GEMV up to 4 tokens; the split-K decode kernel for
+ * 5..32 tokens when a workspace is given); a linear that depends on an earlier one starts a new
  * launch.
  *   depends  set it on linear l when x_l or residual_l (or any buffer it reads) is written by an
  *            earlier linear of the same call.  Linears without it may run ahead of earlier ones.
@@ -168,14 +169,16 @@ int sq_w4a16_gemm_fused(const void* x, const void* w, const void* zs, const void
  *            resident, the weight stream never stops between linears, dependencies are honoured by a
  *            grid barrier inside the kernel); faster than one launch per linear only when nothing
  *            depends on anything, kept for that case and for measurement.
- *   workspace  used by SQ_SEQ_ONE_LAUNCH only (may be NULL otherwise):
- *            sq_w4a16_gemv_sequence_workspace_bytes() bytes (256), 16-byte aligned, zero before
- *            the first call (every call leaves it zero); calls that share it must be ordered.
+ *   workspace  NULL, or sq_w4a16_gemv_sequence_workspace_bytes(linears, count, M) bytes, 16-byte
+ *            aligned, its first 64 KiB zero before the first call (every call leaves them zero);
+ *            calls that share it must be ordered.  Up to 4 tokens it is used by
+ *            SQ_SEQ_ONE_LAUNCH only (256 bytes); with 5..32 tokens it is the split-K workspace of
+ *            sq_w4a16_gemm_ws, sized for the linears that may share a launch.
  *            Word 9 of it is a sticky error flag: it becomes 1 if a grid barrier ever ran out of
  *            polls (results of that call are then undefined).
- * Shapes as for sq_w4a16_gemm (all linears share M).  With M > 4, K > 8192 or a lone linear the
- * linears are launched one by one on the stream (the automatic dispatch of sq_w4a16_gemm): same
- * results.  SQ_SEQ_ONE_LAUNCH falls back to the same when there is no workspace, M > 4, or the
+ * Shapes as for sq_w4a16_gemm (all linears share M).  A lone linear, M > 32, and whatever does not
+ * fit the rules above is launched linear by linear on the stream (the automatic dispatch of
+ * sq_w4a16_gemm_ws): same results.  SQ_SEQ_ONE_LAUNCH falls back to the same when there is no workspace, M > 4, or the
  * activations of a linear do not fit the LDS (M * K * 2 bytes beyond about 128 KiB); its persistent
  * kernel needs every workgroup resident at once (one per CU); other work on the GPU only delays it. */
 #define SQ_SEQ_AUTO 0
@@ -194,7 +197,7 @@ typedef struct sq_linear_desc {
 } sq_linear_desc;
 int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int layout, int mode,
                            void* workspace, size_t workspace_bytes, void* stream);
-size_t sq_w4a16_gemv_sequence_workspace_bytes(void);
+size_t sq_w4a16_gemv_sequence_workspace_bytes(const sq_linear_desc* linears, int count, int M);
 
 /* out[N,K] (fp16) = W_hat in natural k order, bit-identical to fp16
  * (q_fp16 - z_fp16) * s_fp16.  Replaces dequant

@@ -231,7 +231,22 @@ int sq_workspace_check(const void* workspace, size_t bytes, void* stream) {
     return SQ_OK;
 }
 
-size_t sq_w4a16_gemv_sequence_workspace_bytes(void) { return sq::gemv_seq_workspace_bytes(); }
+size_t sq_w4a16_gemv_sequence_workspace_bytes(const sq_linear_desc* linears, int count, int M) {
+    size_t need = sq::gemv_seq_workspace_bytes();
+    if (!linears || count <= 0 || count > SQ_SEQUENCE_MAX || M <= 4) return need;
+    // more than 4 tokens: what sq_w4a16_gemm_ws wants for the largest run of linears that may share a launch
+    // (their rows concatenated, each rounded up to a 64-row block) and for every single linear
+    long rows = 0;
+    int kmax = 0;
+    for (int l = 0; l < count; l++) {
+        if (linears[l].N <= 0 || linears[l].K <= 0) return need;
+        rows += ((long)linears[l].N + 63) / 64 * 64;
+        if (linears[l].K > kmax) kmax = linears[l].K;
+    }
+    if (rows > (1L << 30)) return need;
+    const size_t a = sq_w4a16_workspace_bytes(M, (int)rows, kmax);
+    return a > need ? a : need;
+}
 
 int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int layout, int mode, void* workspace,
                            size_t workspace_bytes, void* stream) {
@@ -259,6 +274,7 @@ int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int 
     if (M == 0) return SQ_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool ws_ok = workspace && aligned16(workspace) && workspace_bytes >= sq::gemv_seq_workspace_bytes();
+    if (workspace && !aligned16(workspace)) workspace = nullptr;
     if (mode == SQ_SEQ_ONE_LAUNCH && ws_ok && M <= 4) {
         // everything in one persistent launch, dependencies honoured by a grid barrier inside the kernel
         const int rc = sq::launch_gemv_seq(probs, count, M, workspace, 1u << 20, st);
@@ -284,6 +300,18 @@ int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int 
                 done = true;
             else if (e != hipErrorInvalidValue)
                 return SQ_ERR_LAUNCH;
+        } else if (l1 - l0 > 1 && M > 4 && M <= 32 && workspace && aligned16(workspace)) {
+            // the split-K decode kernel on the concatenated row blocks, where it is what one linear of the
+            // group's total size would get (large weight, more than 16 tokens, or long K)
+            long elems = 0;
+            for (int l = l0; l < l1; l++) elems += (long)probs[l].N * probs[l].K;
+            if (elems >= (1L << 25) || M > 16 || probs[l0].K > 8192) {
+                const hipError_t e = sq::launch_skinny2_group(probs + l0, l1 - l0, M, workspace, workspace_bytes, st);
+                if (e == hipSuccess)
+                    done = true;
+                else if (e != hipErrorInvalidValue)
+                    return SQ_ERR_LAUNCH;
+            }
         }
         if (!done) {
             for (int l = l0; l < l1; l++) {
@@ -291,7 +319,7 @@ int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int 
                 const sq::Epilogue epi{static_cast<const sq::half_t*>(q.bias), static_cast<const sq::half_t*>(q.residual),
                                        q.act};
                 const int rc = gemm_dispatch(q.x, q.w, q.zs, q.y, M, q.N, q.K, q.group_size, layout, SQ_ALGO_AUTO, epi,
-                                             nullptr, 0, stream);
+                                             M > 4 ? workspace : nullptr, M > 4 ? workspace_bytes : 0, stream);
                 if (rc != SQ_OK) return rc;
             }
         }

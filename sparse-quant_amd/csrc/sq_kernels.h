@@ -43,6 +43,10 @@ struct SeqProblem {
 // when the group does not qualify.
 constexpr int GEMV_GROUP_MAX = 4;
 hipError_t launch_gemv2_group(const SeqProblem* probs, int count, int M, hipStream_t st);
+// sq_skinny2.hip: the same for 5 <= M <= 32 (group size 128) with the split-K decode kernel; ws as for
+// sq_w4a16_gemm_ws, at least skinny2_group_workspace_bytes().
+size_t skinny2_group_workspace_bytes(const SeqProblem* probs, int count, int M);
+hipError_t launch_skinny2_group(const SeqProblem* probs, int count, int M, void* ws, size_t ws_bytes, hipStream_t st);
 size_t gemv_seq_workspace_bytes();
 // 0: launched; 1: the sequence does not fit this kernel (the caller launches the linears one by
 // one); 2: the HIP runtime rejected the launch.  workspace: gemv_seq_workspace_bytes() bytes, zero

@@ -42,12 +42,13 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// rb = row block inside this linear; slot = index of the row block in the workspace (counter and partial
+// tiles), which differs from rb when several linears share a launch.
 template <int MT, int NWV, int S, int RT, bool FIXUP>
-__global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __restrict__ W,
-                                                           const half2_t* __restrict__ ZS,
-                                                           const half_t* __restrict__ X, half_t* __restrict__ Y,
-                                                           float* part, unsigned* counters, int M, int N, int K,
-                                                           int gshift, int ksplit, Epilogue epi) {
+__device__ __forceinline__ void skinny2_body(const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS,
+                                             const half_t* __restrict__ X, half_t* __restrict__ Y, float* part,
+                                             unsigned* counters, int M, int N, int K, int gshift, int ksplit,
+                                             const Epilogue& epi, int rb, int slot, int nslots) {
     constexpr int TILE = RT * MT * 4 * 64;  // floats a wave contributes: [rt][mt][v][lane]
     constexpr int ROWS = 16 * RT;           // weight rows per workgroup
     constexpr int XBUF = MT * 16 * SK2_XPITCH;
@@ -63,7 +64,6 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
     const int wave = tid >> 6;
     const int li = lane & 15;
     const int lj = lane >> 4;
-    const int rb = blockIdx.x;
     const int ks = blockIdx.y;
     const int groups = K >> gshift;
     const int nchunks = (K + 127) >> 7;
@@ -264,7 +264,7 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
     // the counter increment, and the last arriver reads the partials past its own caches.
     // (128-bit accesses with the same cache policy bit the compiler gives those atomics: the
     // exchange is bound by the number of requests, not by bytes.)
-    float* mine = part + ((long)ks * gridDim.x + rb) * TILE;
+    float* mine = part + ((long)ks * nslots + slot) * TILE;
     for (int t4 = tid * 4; t4 < TILE; t4 += 4 * 64 * NWV) {
         float4_t sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
-        const unsigned old = __hip_atomic_fetch_add(&counters[rb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned old = __hip_atomic_fetch_add(&counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         last_flag = (old == (unsigned)(ksplit - 1)) ? 1u : 0u;
     }
     __syncthreads();
@@ -283,7 +283,7 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
         // eight loads regardless of ksplit (absent partials re-read partial 0 and are dropped)
         const float* src[8];
 #pragma unroll
-        for (int q = 0; q < 8; q++) src[q] = part + ((long)(q < ksplit ? q : 0) * gridDim.x + rb) * TILE + t4;
+        for (int q = 0; q < 8; q++) src[q] = part + ((long)(q < ksplit ? q : 0) * nslots + slot) * TILE + t4;
         float4_t pv[8];
         load8_coherent_x4(src, pv);
         float4_t sum = pv[0];
@@ -300,7 +300,45 @@ __global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __rest
         }
     }
     // leave the workspace ready for the next call
-    if (tid == 0) __hip_atomic_store(&counters[rb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0) __hip_atomic_store(&counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int MT, int NWV, int S, int RT, bool FIXUP>
+__global__ __launch_bounds__(64 * NWV) void skinny2_kernel(const uint8_t* __restrict__ W,
+                                                           const half2_t* __restrict__ ZS,
+                                                           const half_t* __restrict__ X, half_t* __restrict__ Y,
+                                                           float* part, unsigned* counters, int M, int N, int K,
+                                                           int gshift, int ksplit, Epilogue epi) {
+    skinny2_body<MT, NWV, S, RT, FIXUP>(W, ZS, X, Y, part, counters, M, N, K, gshift, ksplit, epi, blockIdx.x, blockIdx.x,
+                                        gridDim.x);
+}
+
+// Up to four linears that do not depend on each other and share M, K and the group size in one launch: the
+// grid's x dimension is the concatenation of their 64-row blocks.
+struct Skinny2Group {
+    const uint8_t* W[GEMV_GROUP_MAX];
+    const half2_t* ZS[GEMV_GROUP_MAX];
+    const half_t* X[GEMV_GROUP_MAX];
+    half_t* Y[GEMV_GROUP_MAX];
+    const half_t* bias[GEMV_GROUP_MAX];
+    const half_t* residual[GEMV_GROUP_MAX];
+    int N[GEMV_GROUP_MAX];
+    int act[GEMV_GROUP_MAX];
+    int blk_end[GEMV_GROUP_MAX];  // first row block behind linear p
+    int count;
+};
+
+template <int MT, int NWV, int S, int RT, bool FIXUP>
+__global__ __launch_bounds__(64 * NWV) void skinny2_group_kernel(const Skinny2Group grp, float* part, unsigned* counters,
+                                                                 int M, int K, int gshift, int ksplit) {
+    int p = 0;
+#pragma unroll
+    for (int q = 0; q < GEMV_GROUP_MAX - 1; q++)
+        if (q + 1 < grp.count && (int)blockIdx.x >= grp.blk_end[q]) p = q + 1;
+    const int rb = blockIdx.x - (p > 0 ? grp.blk_end[p - 1] : 0);
+    const Epilogue epi{grp.bias[p], grp.residual[p], grp.act[p]};
+    skinny2_body<MT, NWV, S, RT, FIXUP>(grp.W[p], grp.ZS[p], grp.X[p], grp.Y[p], part, counters, M, grp.N[p], K, gshift,
+                                        ksplit, epi, rb, blockIdx.x, gridDim.x);
 }
 
 size_t skinny2_workspace_bytes(int M, int N, int K) {
@@ -358,6 +396,62 @@ hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, vo
     if (mt == 2) return launch_cfg<2, 4, 2, 4>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
     if (nwv == 8) return launch_cfg<1, 8, 2, 4>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
     return launch_cfg<1, 4, 2, 4>(x, w, zs, y, ws, M, N, K, gshift, fixup, ksplit, epi, st);
+}
+
+template <int MT, int NWV>
+static hipError_t launch_group_cfg(const SeqProblem* probs, int count, void* ws, int M, int K, int gshift, int ksplit,
+                                   hipStream_t st) {
+    Skinny2Group g;
+    int blocks = 0;
+    for (int p = 0; p < GEMV_GROUP_MAX; p++) {
+        const SeqProblem& q = probs[p < count ? p : 0];
+        g.W[p] = (const uint8_t*)q.w;
+        g.ZS[p] = (const half2_t*)q.zs;
+        g.X[p] = (const half_t*)q.x;
+        g.Y[p] = (half_t*)q.y;
+        g.bias[p] = (const half_t*)q.bias;
+        g.residual[p] = (const half_t*)q.residual;
+        g.N[p] = q.N;
+        g.act[p] = q.act;
+        if (p < count) blocks += (q.N + 63) / 64;
+        g.blk_end[p] = blocks;
+    }
+    g.count = count;
+    unsigned* counters = (unsigned*)ws;
+    float* part = (float*)((char*)ws + SK2_COUNTER_BYTES);
+    hipLaunchKernelGGL((skinny2_group_kernel<MT, NWV, 2, 4, true>), dim3(blocks, ksplit), dim3(64 * NWV), 0, st, g, part,
+                       counters, M, K, gshift, ksplit);
+    return hipGetLastError();
+}
+
+// Workspace for a grouped launch: as for one linear whose N is the sum of the group's (rounded up to 64 each).
+size_t skinny2_group_workspace_bytes(const SeqProblem* probs, int count, int M) {
+    int rows = 0;
+    for (int p = 0; p < count; p++) rows += ((probs[p].N + 63) / 64) * 64;
+    return skinny2_workspace_bytes(M, rows, probs[0].K);
+}
+
+// Grouped launch (fixup arithmetic, group size 128): count in 2..GEMV_GROUP_MAX linears with the same K and
+// group size, 5 <= M <= 32.  hipErrorInvalidValue when the group does not qualify.
+hipError_t launch_skinny2_group(const SeqProblem* probs, int count, int M, void* ws, size_t ws_bytes, hipStream_t st) {
+    if (count < 2 || count > GEMV_GROUP_MAX || M < 5 || M > 32 || !ws) return hipErrorInvalidValue;
+    const int K = probs[0].K;
+    if (probs[0].group_size != 128) return hipErrorInvalidValue;
+    for (int p = 1; p < count; p++)
+        if (probs[p].K != K || probs[p].group_size != 128) return hipErrorInvalidValue;
+    int row_blocks = 0;
+    for (int p = 0; p < count; p++) row_blocks += (probs[p].N + 63) / 64;
+    if (row_blocks > 16384 || ws_bytes < skinny2_group_workspace_bytes(probs, count, M)) return hipErrorInvalidValue;
+    const int mt = (M + 15) / 16;
+    const int nchunks = (K + 127) / 128;
+    int ksplit = 1;  // same rule as for one linear with all the rows
+    while (ksplit < 8 && row_blocks * ksplit * 2 <= 256 && nchunks / (ksplit * 2) >= 8) ksplit *= 2;
+    const int cps = (nchunks + ksplit - 1) / ksplit;
+    const int nwv = (mt == 2 || cps >= 16) ? 8 : 4;
+    if (mt == 2 && nwv == 8) return launch_group_cfg<2, 8>(probs, count, ws, M, K, 7, ksplit, st);
+    if (mt == 2) return launch_group_cfg<2, 4>(probs, count, ws, M, K, 7, ksplit, st);
+    if (nwv == 8) return launch_group_cfg<1, 8>(probs, count, ws, M, K, 7, ksplit, st);
+    return launch_group_cfg<1, 4>(probs, count, ws, M, K, 7, ksplit, st);
 }
 
 }  // namespace sq

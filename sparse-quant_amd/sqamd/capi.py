@@ -64,7 +64,7 @@ class LinearDesc(ctypes.Structure):
 
 SIGNATURES["sq_w4a16_gemv_sequence"] = (_i, [ctypes.POINTER(LinearDesc), _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp])
 SQ_SEQ_AUTO, SQ_SEQ_ONE_LAUNCH = 0, 1
-SIGNATURES["sq_w4a16_gemv_sequence_workspace_bytes"] = (ctypes.c_size_t, [])
+SIGNATURES["sq_w4a16_gemv_sequence_workspace_bytes"] = (ctypes.c_size_t, [ctypes.POINTER(LinearDesc), _i, _i])
 SQ_SEQUENCE_MAX = 8
 
 _lib = None
@@ -234,8 +234,8 @@ class LinearSequence:
             d.residual = l["residual"].data_ptr() if l.get("residual") is not None else None
             d.N, d.K, d.group_size = int(l["n"]), int(l["k"]), int(l["group_size"])
             d.act, d.depends = int(l.get("act", SQ_ACT_NONE)), int(bool(l.get("depends", False)))
-        self.ws = torch.zeros(lib().sq_w4a16_gemv_sequence_workspace_bytes(), dtype=torch.uint8,
-                              device=device) if workspace else None
+        self.ws = torch.zeros(lib().sq_w4a16_gemv_sequence_workspace_bytes(self.descs, self.count, self.m),
+                              dtype=torch.uint8, device=device) if workspace else None
         self._fn = lib().sq_w4a16_gemv_sequence
 
     def run(self, stream=None):

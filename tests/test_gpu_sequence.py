@@ -184,6 +184,54 @@ def test_opt67_layer_linears_in_one_launch(capi, m, mode):
     assert seq.error_flag() == 0 and torch.count_nonzero(seq.ws).item() == 0
 
 
+@pytest.mark.parametrize("m", [5, 8, 16, 32])
+def test_grouped_launch_for_decode_batches(capi, m):
+    """5..32 tokens: q, k and v (three weights, one input) share one launch of the split-K decode kernel, a
+    dependent linear follows in a launch of its own; against the oracle on sampled rows and against one
+    sq_w4a16_gemm_ws launch per linear (same kernel, same arithmetic: bit-identical)."""
+    g, h = 128, 4096
+    rng = np.random.default_rng(m)
+    x = orc.synth_x(m, h, seed=60 + m)
+    xd = to_dev(x)
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(m)
+    lin, ys, checks = [], [], []
+    for idx, n in enumerate((4096, 4096, 4096, 2112)):
+        w = torch.randint(0, 256, (n, h // 2), dtype=torch.uint8, device=DEV, generator=gen)
+        z = torch.randint(0, 16, (n, h // g), device=DEV, generator=gen).half() + 64
+        s = (torch.randn((n, h // g), device=DEV, generator=gen).abs() * 0.02 + 1e-3).half()
+        zs = torch.stack([z, s], dim=-1).reshape(n, 2 * (h // g)).contiguous()
+        y = torch.full((m, n), float("nan"), dtype=torch.float16, device=DEV)
+        bias = (torch.randn(n, device=DEV, generator=gen) * 0.5).half() if idx == 1 else None
+        ys.append(y)
+        lin.append(dict(x=xd, w=w, zs=zs, y=y, n=n, k=h, group_size=g, bias=bias, depends=(idx == 3)))
+        rows = np.sort(rng.choice(n, size=64, replace=False))
+        ridx = torch.from_numpy(rows).to(DEV)
+        ref = orc.gemm_ref(x, orc.dequant_l1(w[ridx].cpu().numpy(), zs[ridx].cpu().numpy(), g)).astype(np.float64)
+        if bias is not None:
+            ref = ref + bias[ridx].float().cpu().numpy()[None, :]
+        checks.append((ridx, ref))
+    seq = capi.LinearSequence(lin, m, DEV)
+    assert seq.ws.numel() >= capi.lib().sq_w4a16_workspace_bytes(m, 3 * 4096, h)
+    for rep in range(2):
+        seq.run()
+        torch.cuda.synchronize()
+        for y, (ridx, ref) in zip(ys, checks):
+            assert torch.isfinite(y).all()
+            assert rel_err(y[:, ridx].float().cpu().numpy(), ref) <= 5e-3
+        assert capi.workspace_is_clean(seq.ws)
+    for l, y in zip(lin, ys):
+        single = capi.gemm_fused(l["x"], l["w"], l["zs"], l["n"], l["k"], g, bias=l["bias"])
+        assert (single.float() - y.float()).abs().max().item() <= 5e-3 * y.float().abs().max().item()
+    # without a workspace the same call launches linear by linear
+    ys2 = [torch.empty_like(y) for y in ys]
+    lin2 = [dict(l, y=y2) for l, y2 in zip(lin, ys2)]
+    capi.LinearSequence(lin2, m, DEV, workspace=False).run()
+    torch.cuda.synchronize()
+    for a, b in zip(ys, ys2):
+        assert (a.float() - b.float()).abs().max().item() <= 5e-3 * b.float().abs().max().item()
+
+
 def test_llama_mlp_shapes_and_more_than_four_tokens(capi):
     g = 128
     d1, d2 = make_linear(11008, 4096, g, 21), make_linear(4096, 11008, g, 22, 0.05)
@@ -214,6 +262,7 @@ def test_sequence_rejections(capi):
         d.N, d.K, d.group_size = 64, 128, 64
     ws = ctypes.c_void_p(p)
     call = lambda count, m, layout=1, mode=0: L.sq_w4a16_gemv_sequence(descs, count, m, layout, mode, ws, 256, None)
+    assert L.sq_w4a16_gemv_sequence_workspace_bytes(descs, 2, 1) == 256
     assert call(2, 1, mode=5) == capi.SQ_ERR_BAD_ALGO
     assert call(9, 1) == capi.SQ_ERR_BAD_SHAPE
     assert call(0, 1) == capi.SQ_OK
