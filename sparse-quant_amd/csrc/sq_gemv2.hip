@@ -35,6 +35,29 @@
 namespace sq {
 
 template <int MROWS, int NR, int KS, int S, bool FIXUP>
+struct Gemv2Lds {
+    static constexpr int PITCH = 1024 * S + 16;
+    static constexpr bool SUMS = FIXUP && MROWS <= 4;
+    static constexpr int XSUM_OFF = KS * MROWS * PITCH;
+    static constexpr int RED_OFF = XSUM_OFF + (SUMS ? KS * S * 16 * MROWS * 2 * 4 : 0);
+    static constexpr int BYTES = RED_OFF + KS * NR * MROWS * 4 * 4;
+};
+
+// Launch with Gemv2Lds::BYTES of dynamic LDS; instantiations beyond 64 KiB need the attribute first.
+template <typename Kern>
+static hipError_t gemv2_allow_lds(Kern kern, int bytes, bool* done) {
+    if (bytes <= 64 * 1024) return hipSuccess;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    if (!done[dev]) {
+        const hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e != hipSuccess) return e;
+        done[dev] = true;
+    }
+    return hipSuccess;
+}
+
+template <int MROWS, int NR, int KS, int S, bool FIXUP>
 __device__ __forceinline__ void gemv2_body(const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS,
                                            const half_t* __restrict__ X, half_t* __restrict__ Y, int M, int N, int K,
                                            int gshift, const Epilogue& epi, int blk) {
@@ -48,10 +71,14 @@ __device__ __forceinline__ void gemv2_body(const uint8_t* __restrict__ W, const 
     constexpr int STAGE_TOTAL = KS * MROWS * S * 64;     // 128-bit words staged per round
     constexpr int STAGE_PER_THREAD = (STAGE_TOTAL + NT - 1) / NT;
 
-    __shared__ __attribute__((aligned(16))) uint8_t xbuf[KS][MROWS * PITCH];
-    // per run of 32 k and token: {sum of x, 960 * sum of x over the positions unpacked with bias 1024}
-    __shared__ __attribute__((aligned(16))) float xsum[KS][S * 16][MROWS][2];
-    __shared__ float red[KS][NR][MROWS][4];
+    // Dynamic LDS (Gemv2Lds gives the layout to the launcher): staged activations; per run of 32 k and token
+    // {sum of x, 960 * sum of x over the positions unpacked with bias 1024} (only where the zero point is
+    // applied through them); the partial sums of the k ranges.
+    using Lds = Gemv2Lds<MROWS, NR, KS, S, FIXUP>;
+    extern __shared__ __attribute__((aligned(16))) uint8_t gemv2_lds[];
+    uint8_t(*xbuf)[MROWS * PITCH] = reinterpret_cast<uint8_t(*)[MROWS * PITCH]>(gemv2_lds);
+    float(*xsum)[S * 16][MROWS][2] = reinterpret_cast<float(*)[S * 16][MROWS][2]>(gemv2_lds + Lds::XSUM_OFF);
+    float(*red)[NR][MROWS][4] = reinterpret_cast<float(*)[NR][MROWS][4]>(gemv2_lds + Lds::RED_OFF);
 
     const NibbleMasks nm = nibble_masks();
     const int tid = threadIdx.x;
@@ -266,7 +293,11 @@ static hipError_t launch_group_cfg(const SeqProblem* probs, int count, int M, in
         g.blk_end[p] = blocks;
     }
     g.count = count;
-    hipLaunchKernelGGL((gemv2_group_kernel<MROWS, NR, KS, S, true>), dim3(blocks), dim3(64 * NR * KS), 0, st, g, M, K,
+    constexpr int lds = Gemv2Lds<MROWS, NR, KS, S, true>::BYTES;
+    static bool allowed[64] = {};
+    const hipError_t e = gemv2_allow_lds(gemv2_group_kernel<MROWS, NR, KS, S, true>, lds, allowed);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((gemv2_group_kernel<MROWS, NR, KS, S, true>), dim3(blocks), dim3(64 * NR * KS), lds, st, g, M, K,
                        gshift);
     return hipGetLastError();
 }
@@ -275,16 +306,25 @@ template <int MROWS, int NR, int KS, int S>
 static hipError_t launch_cfg(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int gshift,
                              bool fixup, Epilogue epi, hipStream_t st) {
     const dim3 grid((N + 4 * NR - 1) / (4 * NR));
-    if (fixup)
-        hipLaunchKernelGGL((gemv2_kernel<MROWS, NR, KS, S, true>), grid, dim3(64 * NR * KS), 0, st, (const uint8_t*)w,
+    static bool allowed[2][64] = {};
+    if (fixup) {
+        constexpr int lds = Gemv2Lds<MROWS, NR, KS, S, true>::BYTES;
+        const hipError_t e = gemv2_allow_lds(gemv2_kernel<MROWS, NR, KS, S, true>, lds, allowed[1]);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL((gemv2_kernel<MROWS, NR, KS, S, true>), grid, dim3(64 * NR * KS), lds, st, (const uint8_t*)w,
                            (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift, epi);
-    else
-        hipLaunchKernelGGL((gemv2_kernel<MROWS, NR, KS, S, false>), grid, dim3(64 * NR * KS), 0, st,
+    } else {
+        constexpr int lds = Gemv2Lds<MROWS, NR, KS, S, false>::BYTES;
+        const hipError_t e = gemv2_allow_lds(gemv2_kernel<MROWS, NR, KS, S, false>, lds, allowed[0]);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL((gemv2_kernel<MROWS, NR, KS, S, false>), grid, dim3(64 * NR * KS), lds, st,
                            (const uint8_t*)w, (const half2_t*)zs, (const half_t*)x, (half_t*)y, M, N, K, gshift, epi);
+    }
     return hipGetLastError();
 }
 
-// Staged activations are kept under 48 KiB of LDS: KS * MROWS * S KiB.
+// Staged activations: KS * MROWS * S KiB of LDS; several k ranges per workgroup only while that stays under
+// 48 KiB (a single range may take up to 64 KiB: eight tokens with all eight k-steps of K = 4096 in one round).
 template <int MROWS, int S>
 static hipError_t launch_steps(int nr, int ks, const void* x, const void* w, const void* zs, void* y, int M, int N,
                                int K, int gshift, bool fixup, Epilogue epi, hipStream_t st) {
@@ -306,7 +346,7 @@ static hipError_t launch_steps(int nr, int ks, const void* x, const void* w, con
 template <int MROWS>
 static hipError_t launch_rows(int nr, int ks, int steps, const void* x, const void* w, const void* zs, void* y,
                               int M, int N, int K, int gshift, bool fixup, Epilogue epi, hipStream_t st) {
-    constexpr int S_MAX = (MROWS >= 4) ? 4 : 8;
+    constexpr int S_MAX = (MROWS == 4) ? 4 : 8;
     if (steps >= 8 && S_MAX >= 8) return launch_steps<MROWS, S_MAX>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
     if (steps >= 4) return launch_steps<MROWS, 4>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
     return launch_steps<MROWS, 2>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
