@@ -176,9 +176,11 @@ __device__ __forceinline__ void gemv2_body(const uint8_t* __restrict__ W, const 
                     }
                 }
             } else {
-                float4_t tmp[MT];
+                // Two accumulators per token tile (words 0, 1 and words 2, 3): with one wave per SIMD a single
+                // chain of dependent matrix instructions would leave their latency exposed.
+                float4_t tmp[MT], tmp2[MT];
 #pragma unroll
-                for (int mt = 0; mt < MT; mt++) tmp[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                for (int mt = 0; mt < MT; mt++) tmp[mt] = tmp2[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
                 // zero-point operand for the mixed-bias unpack: -(1024 + z) where the weight carries
                 // bias 1024 (positions 0, 1 of each four), -(64 + z) elsewhere; both exact in fp16
                 const half_t nz = -p.x;
@@ -189,14 +191,17 @@ __device__ __forceinline__ void gemv2_body(const uint8_t* __restrict__ W, const 
                     const half8_t wv = unpack8_mixed(wq[s][t], nm);
 #pragma unroll
                     for (int mt = 0; mt < MT; mt++) {
-                        tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, wv.lo, tmp[mt], 0, 0, 0);
-                        tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].hi, wv.hi, tmp[mt], 0, 0, 0);
+                        float4_t& tq = (t < 2) ? tmp[mt] : tmp2[mt];
+                        tq = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, wv.lo, tq, 0, 0, 0);
+                        tq = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].hi, wv.hi, tq, 0, 0, 0);
                         if (ZMFMA) {
-                            tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, nzb, tmp[mt], 0, 0, 0);
-                            tmp[mt] = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].hi, nzb, tmp[mt], 0, 0, 0);
+                            tq = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].lo, nzb, tq, 0, 0, 0);
+                            tq = __builtin_amdgcn_mfma_f32_4x4x4f16(xa[mt][t].hi, nzb, tq, 0, 0, 0);
                         }
                     }
                 }
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) tmp[mt] += tmp2[mt];
                 const float zf = (float)p.x;
                 const float sf = (float)p.y;
                 const float* xs = &xsum[wq_][16 * s + b][0][0];
