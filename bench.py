@@ -79,13 +79,16 @@ def parity_linear(torch, w, zs, n, k, g, x, y, seed=0, rows=64, tokens=32):
     ridx = np.sort(rng.choice(n, size=min(rows, n), replace=False))
     m = x.shape[0]
     tidx = np.arange(m) if m <= tokens else np.sort(rng.choice(m, size=tokens, replace=False))
-    rt = torch.from_numpy(ridx).to(w.device)
-    tt = torch.from_numpy(tidx).to(w.device)
-    w_hat = orc.dequant_l1(w[rt].cpu().numpy(), zs[rt].cpu().numpy(), g)
-    y_ref = orc.gemm_ref(x[tt].cpu().numpy(), w_hat)
-    got = y[tt][:, rt].float().cpu().numpy()
-    if not np.all(np.isfinite(got)):
-        return float("inf")
+    # Whole tensors come to the host and are sampled there, so that the check does not depend on the ordering
+    # of index uploads and device-side gathers (a run under rocprofv3 --pmc once sampled non-finite data that way).
+    torch.cuda.synchronize()
+    w_hat = orc.dequant_l1(w.cpu().numpy()[ridx], zs.cpu().numpy()[ridx], g)
+    y_ref = orc.gemm_ref(x.cpu().numpy()[tidx], w_hat)
+    got = y.float().cpu().numpy()[tidx][:, ridx]
+    if not np.all(np.isfinite(got)) or not np.all(np.isfinite(y_ref)):
+        raise ParityError("parity gate: non-finite data (sampled result %d, activations %d, dequantised weight rows %d "
+                          "of %d x %d non-finite)" % (np.sum(~np.isfinite(got)), np.sum(~np.isfinite(x.cpu().numpy())),
+                                                      np.sum(~np.isfinite(w_hat)), n, k))
     return float(np.max(np.abs(got - y_ref)) / np.max(np.abs(y_ref)))
 
 
@@ -95,9 +98,9 @@ def parity_dequant(torch, capi, w, zs, n, k, g, seed=0, rows=64):
     import w4a16_oracle as orc
     rng = np.random.default_rng(seed)
     ridx = np.sort(rng.choice(n, size=min(rows, n), replace=False))
-    rt = torch.from_numpy(ridx).to(w.device)
-    want = orc.dequant_l1(w[rt].cpu().numpy(), zs[rt].cpu().numpy(), g)
-    got = capi.dequant(w, zs, n, k, g)[rt].cpu().numpy()
+    torch.cuda.synchronize()
+    want = orc.dequant_l1(w.cpu().numpy()[ridx], zs.cpu().numpy()[ridx], g)
+    got = capi.dequant(w, zs, n, k, g).cpu().numpy()[ridx]
     return bool(np.array_equal(got.view(np.int16), want.view(np.int16)))
 
 
@@ -277,6 +280,7 @@ def main():
             if rc != 0:
                 raise RuntimeError("sq_w4a16_gemm failed: " + capi.strerror(rc))
 
+    torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
     with torch.cuda.stream(stream):
         for i in range(len(calls)):
             run_layer(i)
@@ -531,6 +535,7 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
         n = max(8, int(3000.0 / us))           # about 3 ms of load on either side of the probe
         for _ in range(n):
             fn()
+        torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
         with torch.cuda.stream(side):
             ticks = capi.clock_probe(spins=200000, stream=side)
         for _ in range(2 * n):
@@ -546,6 +551,7 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
         work.append((w, zs, name, n, k))
     opt_names = {name for _, _, name, _, _ in work[:3]}
     worst = 0.0
+    torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
     with torch.cuda.stream(stream):
         for w, zs, name, n, k in work:
             x = torch.randn((m, k), device=dev, generator=gen).half()
@@ -574,6 +580,7 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
     tfd = flops_total / dense_time_total / 1e6
     # the other two token counts of the same configuration, aggregate only
     other = {}
+    torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
     with torch.cuda.stream(stream):
         for m2 in (512, 4096):
             fl2, t2 = 0.0, 0.0
@@ -597,6 +604,7 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
     # What the matrix pipes sustain under the power limit: a loop of nothing but independent
     # v_mfma_f32_32x32x16_f16 on all CUs (one wave per SIMD), on N(0,1) operands and on zeros.
     roof = {}
+    torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
     with torch.cuda.stream(stream):
         cus = torch.cuda.get_device_properties(dev).multi_processor_count
         iters = 20000
@@ -625,6 +633,7 @@ def decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream):
         xs = {k: torch.randn((m, k), device=dev, generator=gen).half() for k in {k for _, _, k in shapes}}
         ys = {n: torch.empty((m, n), dtype=torch.float16, device=dev) for n in {n for _, n, _ in shapes}}
         bytes_per_step = sum(algorithmic_bytes(m, n, k, g) for _, n, k in shapes)
+        torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
         with torch.cuda.stream(stream):
             ws = capi.workspace(m, 16384, 16384, dev, stream)
             seqs = None
@@ -691,6 +700,7 @@ def config1_leg(torch, capi, dev, gen, stream, g=64, n=4096, k=4096, copies=32):
         x = torch.randn((m, k), device=dev, generator=gen).half()
         y = torch.empty((m, n), dtype=torch.float16, device=dev)
         nbytes = algorithmic_bytes(m, n, k, g)
+        torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
         with torch.cuda.stream(stream):
             ws = capi.workspace(m, n, k, dev, stream)
             run = lambda: [capi.gemm_ws(x, w, zs, n, k, g, out=y, stream=stream, ws=ws) for w, zs in pool]
@@ -729,6 +739,7 @@ def sequence_leg(torch, capi, pool, shapes, m, g, dev, gen, stream, bytes_per_st
         seqs = [capi.LinearSequence([dict(x=xs[k], w=w, zs=zs, y=ys[i], n=n, k=k, group_size=g, depends=dep[i] == "1")
                                      for i, ((w, zs), (_, n, k)) in enumerate(zip(layer, shapes))], m, dev, mode=mode)
                 for layer in pool]
+        torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
         with torch.cuda.stream(stream):
             seqs[0].run(stream=stream)
             stream.synchronize()
@@ -765,6 +776,7 @@ def fused_qkv_leg(torch, capi, m, g, dev, gen, stream, layers, bytes_per_step):
     xs = {k: torch.randn((m, k), device=dev, generator=gen).half() for k in (4096, 16384)}
     ys = {n: torch.empty((m, n), dtype=torch.float16, device=dev) for n in (12288, 4096, 16384)}
     steps = 2000
+    torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
     with torch.cuda.stream(stream):
         def run(i):
             for (w, zs), (_, n, k) in zip(pool[i % layers], shapes):

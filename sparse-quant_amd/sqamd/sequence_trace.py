@@ -70,6 +70,7 @@ def main(m=1, dep="000111", g=128, layers=8):
     stream = torch.cuda.Stream()
 
     def timed(fn, reps=200):
+        torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
         with torch.cuda.stream(stream):
             fn()
             stream.synchronize()
