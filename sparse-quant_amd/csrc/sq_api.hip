@@ -98,7 +98,13 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
                            (N + 63) / 64 <= 16384;
         const bool gemm_ws = workspace && aligned16(workspace) && M > 32 &&
                              workspace_bytes >= sq::gemm_workspace_bytes(M, N, K);
-        if (ws_ok && M > 4 && M <= 32 && (large || M > 16 || K > 8192)) {
+        // 5..16 tokens at group size 128: the streaming kernel wherever its K range fits (a K beyond 4096
+        // needs the workspace).  Against the split-K kernel at 8 tokens: fc1 10.0 against 13.3 us, q/k/v in
+        // one launch 8.6 against 12.1, fc2 12.7 against 14.6; against the GEMV on 4096 x 4096: 4.9 against 6.5.
+        const bool stream_ok = M > 4 && M <= 16 && group_size == 128 && K % 128 == 0 && (K <= 4096 || (ws_ok && K <= 32768));
+        if (stream_ok) {
+            kernel = SQ_ALGO_STREAM;
+        } else if (ws_ok && M > 4 && M <= 32 && (large || M > 16 || K > 8192)) {
             kernel = SQ_ALGO_SKINNY_WS;
         } else if (ws_ok && M > 32 && M <= 48 && (large || K > 8192)) {
             // 33..48 tokens on a large weight: two blocks through the split-K decode kernel are
@@ -140,6 +146,13 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
                 (N + 63) / 64 > 16384)
                 return SQ_ERR_WORKSPACE;
             return launch_code(sq::launch_skinny2_tuned(x, w, zs, y, workspace, M, N, K, group_size, tune, epi, st));
+        case SQ_ALGO_STREAM: {
+            if (M > 16 || group_size != 128) return SQ_ERR_BAD_ALGO;
+            const bool ws_fits = workspace && aligned16(workspace) &&
+                                 workspace_bytes >= sq::skinny2_workspace_bytes(M, N, K);
+            const hipError_t e = sq::launch_skinny3_tuned(x, w, zs, y, ws_fits ? workspace : nullptr, M, N, K, tune, epi, st);
+            return e == hipErrorInvalidValue ? SQ_ERR_WORKSPACE : launch_code(e);
+        }
         case SQ_ALGO_GEMM:
             return launch_code(sq::launch_gemm_tuned(x, w, zs, y, aligned16(workspace) ? workspace : nullptr,
                                                      workspace_bytes, M, N, K, group_size, tune, epi, st));
@@ -300,7 +313,16 @@ int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int 
                 done = true;
             else if (e != hipErrorInvalidValue)
                 return SQ_ERR_LAUNCH;
-        } else if (l1 - l0 > 1 && M > 4 && M <= 32 && workspace && aligned16(workspace)) {
+        } else if (l1 - l0 > 1 && M > 4 && M <= 16 && probs[l0].group_size == 128 && probs[l0].K % 128 == 0 &&
+                   (probs[l0].K <= 4096 || workspace)) {
+            // the streaming decode kernel on the concatenated row blocks (a K beyond 4096 needs the workspace)
+            const hipError_t e = sq::launch_skinny3_group(probs + l0, l1 - l0, M, workspace, workspace_bytes, st);
+            if (e == hipSuccess)
+                done = true;
+            else if (e != hipErrorInvalidValue)
+                return SQ_ERR_LAUNCH;
+        }
+        if (!done && l1 - l0 > 1 && M > 4 && M <= 32 && workspace && aligned16(workspace)) {
             // the split-K decode kernel on the concatenated row blocks, where it is what one linear of the
             // group's total size would get (large weight, more than 16 tokens, or long K)
             long elems = 0;

@@ -1,0 +1,450 @@
+// Streaming skinny GEMM for up to 16 tokens, group size 128, layout L1: the decode kernel for small batches.
+//
+// The matrix instruction, the operand mapping and the per-chunk arithmetic are those of the split-K
+// decode kernel in sq_skinny2.hip (v_mfma_f32_16x16x32_f16, weights as the B operand straight from
+// registers, per 128-wide chunk s * (acc - (64 + z) * sum_x) in fp32), with the shift-free unpack of the
+// GEMV (1024 + q on four of every eight positions; the chunk's accumulator starts at -960 * the sum of x
+// over those positions, itself one more matrix instruction, so the extra bias costs no vector arithmetic).
+// What differs is the order of memory operations, which is what bounds this regime.  Measured with time
+// stamps inside the kernel (fc1 of OPT-6.7B, 8 tokens), the split-K kernel spends its time in two serial
+// trips of "request, wait for everything, compute"; here:
+//
+//   * A workgroup (eight waves) owns 16 * RT weight rows and one K range of at most 8 * CH chunks.  Its
+//     zeros/scales and ALL activations of that range are requested first; a bare s_barrier makes sure every
+//     wave has done so before any wave requests weights (a CU serves its vector memory requests in order).
+//   * The weights go out in units of four loads (two row tiles x the two 64-byte halves of a 128-byte line),
+//     one unit ahead of the one being consumed.  A CU accepts only a few dozen such requests; a wave that
+//     issues into a full queue stalls at that instruction, and a wave that has requested all its weights up
+//     front reaches the parking of the activations only when most of the stream has arrived (first
+//     arithmetic 5.3 us after launch instead of 1.9 us).
+//   * The activations are parked in LDS (row-major per token, pitch = 16 mod 256 bytes: the operand-order
+//     reads of 16 lanes fall into 16 different 16-byte slots).  The vector memory counter retires in order,
+//     so waiting for them leaves the first weight unit in flight.
+//   * Barriers are s_waitcnt lgkmcnt(0) + s_barrier, not __syncthreads(): the latter also waits for every
+//     outstanding vector memory load.
+//   * The main part is straight-line code (no loop, no branch), each request pinned in place by a
+//     scheduling barrier; a chunk slot beyond the K range reads a valid address and meets zero activations.
+//
+// Partial tiles of the eight waves meet in LDS; with ksplit > 1 the workgroups of a row block exchange
+// fp32 partial tiles through the workspace exactly as the split-K decode kernel does (same layout, same
+// counters: a workspace sized for that kernel serves this one).
+// (replaces w4a16_gemm_wmma_kernel for small batches, reference:
+// quantization/muxi/backend/w4a16_gemm.cuh:466-600)
+#include "sq_common.h"
+#include "sq_kernels.h"
+
+namespace sq {
+
+namespace {
+
+constexpr int SK3_COUNTER_BYTES = 65536;  // start of the workspace: one uint32 per row block
+constexpr int SK3_NWV = 8;
+constexpr int SK3_NT = 64 * SK3_NWV;
+constexpr int SK3_ZPITCH = 33;
+#ifndef SQ_SK3_DEPTH
+#define SQ_SK3_DEPTH 1
+#endif
+#ifndef SQ_SK3_DEPTH_PRE
+#define SQ_SK3_DEPTH_PRE 1
+#endif
+constexpr int SK3_DEPTH_PRE = SQ_SK3_DEPTH_PRE;  // units requested before the activations are parked
+constexpr int SK3_DEPTH = SQ_SK3_DEPTH;  // units of four weight loads requested ahead of the one being consumed
+
+template <int MROWS, int RT, int CH>
+struct Sk3Lds {
+    static constexpr int CHUNKS = SK3_NWV * CH;          // chunk slots of a workgroup
+    static constexpr int XPITCH = CHUNKS * 256 + 16;     // bytes per staged token row
+    static constexpr int X_BYTES = MROWS * XPITCH;
+    static constexpr int TILE = RT * 4 * 64;             // floats a wave contributes: [rt][v][lane]
+    static constexpr int RED_BYTES = SK3_NWV * TILE * 4;
+    static constexpr int Z_OFF = X_BYTES > RED_BYTES ? X_BYTES : RED_BYTES;  // the partials reuse the activations' space
+    static constexpr int FLAG_OFF = Z_OFF + 16 * RT * SK3_ZPITCH * 4;
+    static constexpr int BYTES = FLAG_OFF + 16;
+};
+
+__device__ __forceinline__ void sk3_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// rb = row block inside this linear; slot = index of the row block in the workspace, which differs from
+// rb when several linears share a launch.
+template <int MROWS, int RT, int CH, int DEPTH>
+__device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ZS,
+                                             const half_t* __restrict__ X, half_t* __restrict__ Y, float* part,
+                                             unsigned* counters, int M, int N, int K, int ksplit, const Epilogue& epi,
+                                             int rb, int slot, int nslots) {
+    using L = Sk3Lds<MROWS, RT, CH>;
+    constexpr int ROWS = 16 * RT;
+    constexpr int TILE = L::TILE;
+    constexpr int WPR = L::CHUNKS * 16;  // 128-bit words per staged token row
+    constexpr int XPT = MROWS * WPR / SK3_NT;
+    constexpr int ZPT = (ROWS * 32 + SK3_NT - 1) / SK3_NT;
+    static_assert(CH == 1 || CH == 2 || CH == 4, "chunk slots per wave");
+    static_assert(MROWS * WPR % SK3_NT == 0, "activation words divide over the threads");
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t sk3_lds[];
+    uint8_t* xl = sk3_lds;
+    uint32_t* zsl = (uint32_t*)(sk3_lds + L::Z_OFF);
+    unsigned* last_flag = (unsigned*)(sk3_lds + L::FLAG_OFF);
+    float* red = (float*)sk3_lds;
+
+    const NibbleMasks nm = nibble_masks();
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int li = lane & 15;
+    const int lj = lane >> 4;
+    const int ks = blockIdx.y;
+    const int groups = K >> 7;  // group size 128: one (z, s) pair per chunk
+    const int cps = (groups + ksplit - 1) / ksplit;
+    int c_begin = ks * cps;
+    int nc = imin(c_begin + cps, groups) - c_begin;
+    if (nc <= 0) {  // an empty K range (the host does not create one) streams chunk 0 against zeros
+        nc = 0;
+        c_begin = 0;
+    }
+
+    // 1. zeros/scales of the row block and K range (row-contiguous)
+    uint32_t zreg[ZPT];
+#pragma unroll
+    for (int p = 0; p < ZPT; p++) {
+        const int idx = tid + p * SK3_NT;
+        const int r = (idx >> 5) % ROWS, col = idx & 31;
+        const int row = imin(rb * ROWS + r, N - 1);
+        zreg[p] = ZS[(long)row * groups + c_begin + (col < nc ? col : 0)];
+    }
+    // 2. every activation of the K range (tokens beyond M and chunk slots beyond the range: zeros)
+    u32x4_t xr[XPT];
+#pragma unroll
+    for (int p = 0; p < XPT; p++) {
+        const int idx = tid + p * SK3_NT;
+        const int m = idx / WPR, col = idx % WPR;
+        const bool ok = (m < M) && (col < nc * 16);
+        const u32x4_t v = *(const u32x4_t*)(X + (ok ? (long)m * K + c_begin * 128 + col * 8 : 0));
+        xr[p] = ok ? v : (u32x4_t){0u, 0u, 0u, 0u};
+    }
+    // Every wave has issued its activation loads before any wave issues a weight load: a CU serves its
+    // vector memory requests in order, and activations queued behind another wave's sixteen weight loads
+    // would reach the barrier below only when most of the stream has already arrived.
+    asm volatile("s_barrier" ::: "memory");
+    // 3. the wave's weight loads, in units of four (two row tiles x the two 64-byte halves of a 128-byte
+    //    line back to back, so that the line is requested from L2 once), DEPTH units ahead of the arithmetic
+    constexpr int RTU = RT >= 2 ? 2 : 1;        // row tiles per unit
+    constexpr int RG = RT / RTU;                // units per chunk pair
+    constexpr int HN = CH == 1 ? 1 : 2;         // chunk slots per unit
+    constexpr int NU = (CH == 1 ? 1 : CH / 2) * RG;
+    u32x4_t wq[CH][RT];
+    int slot_of[CH];
+#pragma unroll
+    for (int u = 0; u < CH; u++) slot_of[u] = (CH == 1) ? wave : 2 * (wave + SK3_NWV * (u >> 1)) + (u & 1);
+    const uint8_t* wrow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) wrow[rt] = W + (long)imin(rb * ROWS + 16 * rt + li, N - 1) * (K >> 1) + lj * 16;
+    auto issue_unit = [&](int un) {
+        const int pr = un / RG, rg = un % RG;
+#pragma unroll
+        for (int r = 0; r < RTU; r++)
+#pragma unroll
+            for (int h = 0; h < HN; h++) {
+                const int cl = slot_of[2 * pr + h];
+                wq[2 * pr + h][RTU * rg + r] =
+                    *(const u32x4_t*)(wrow[RTU * rg + r] + (long)(c_begin + (cl < nc ? cl : 0)) * 64);
+            }
+    };
+#pragma unroll
+    for (int un = 0; un < NU; un++)
+        if (un < SK3_DEPTH_PRE) issue_unit(un);
+    // 4. park zeros/scales and activations (waits for 1 and 2 only: the weight loads stay in flight)
+#pragma unroll
+    for (int p = 0; p < ZPT; p++) {
+        const int idx = tid + p * SK3_NT;
+        if (idx < ROWS * 32) zsl[(idx >> 5) * SK3_ZPITCH + (idx & 31)] = zreg[p];
+    }
+#pragma unroll
+    for (int p = 0; p < XPT; p++) {
+        const int idx = tid + p * SK3_NT;
+        *(u32x4_t*)(xl + (idx / WPR) * L::XPITCH + (idx % WPR) * 16) = xr[p];
+    }
+    sk3_barrier();
+
+    // 5. the wave's units in issue order, the next request going out before each unit's arithmetic
+    float4_t acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) acc[rt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    const half8_t ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f,
+                          (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
+    const uint8_t* xrd = xl + (li & (MROWS - 1)) * L::XPITCH + lj * 64;  // token li (a token >= MROWS repeats one: ignored)
+    float4_t xsum[CH], x960[CH];
+    const half8_t m960 = {(half_t)-960.f, (half_t)-960.f, (half_t)0.f, (half_t)0.f,
+                          (half_t)-960.f, (half_t)-960.f, (half_t)0.f, (half_t)0.f};
+#pragma unroll
+    for (int un = SK3_DEPTH_PRE; un < NU; un++)
+        if (un < DEPTH) issue_unit(un);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int un = 0; un < NU; un++) {
+        if (un + DEPTH < NU) {
+            issue_unit(un + DEPTH);
+            __builtin_amdgcn_sched_barrier(0);  // the request goes out here, not wherever the scheduler finds room
+        }
+        const int pr = un / RG, rg = un % RG;
+#pragma unroll
+        for (int h = 0; h < HN; h++) {
+            const int u = 2 * pr + h;
+            const int cl = slot_of[u];
+            const int zcol = cl < nc ? cl : 0;
+            half8_t xa[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) xa[t] = *(const half8_t*)(xrd + cl * 256 + 16 * t);
+            if (rg == 0) {
+                xsum[u] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                x960[u] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    xsum[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t], ones, xsum[u], 0, 0, 0);
+                    x960[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t], m960, x960[u], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < RTU; r++) {
+                const int rt = RTU * rg + r;
+                const half2_t zsv = bit_cast<half2_t>(zsl[(16 * rt + li) * SK3_ZPITCH + zcol]);
+                // shift-free unpack (1024 + q on four of every eight positions); the accumulator starts at
+                // -960 * (sum of x over those positions), which takes the extra bias out again
+                float4_t tmp = x960[u];
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+                    tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t], unpack8_mixed(wq[u][rt][t], nm), tmp, 0, 0, 0);
+                const float zf = (float)zsv.x;
+                const float sf = (float)zsv.y;
+#pragma unroll
+                for (int v = 0; v < 4; v++) acc[rt][v] += sf * (tmp[v] - zf * xsum[u][v]);
+            }
+        }
+    }
+    sk3_barrier();  // every wave is done with the activations, which the partials now overwrite
+
+    // Sum the waves' partial tiles: red[wave][rt][v][lane].
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int v = 0; v < 4; v++) red[wave * TILE + (rt * 4 + v) * 64 + lane] = acc[rt][v];
+    sk3_barrier();
+
+    // Element t of the tile: lane l = t % 64, v, rt -> token m = 4 (l / 16) + v, row n = ROWS rb + 16 rt + l % 16.
+    if (ksplit == 1) {
+        for (int t = tid; t < TILE; t += SK3_NT) {
+            float sum = 0.f;
+#pragma unroll
+            for (int p = 0; p < SK3_NWV; p++) sum += red[p * TILE + t];
+            const int l = t & 63, v = (t >> 6) & 3, rt = t >> 8;
+            const int m = 4 * (l >> 4) + v;
+            const int n = rb * ROWS + 16 * rt + (l & 15);
+            if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum, m, n, N, epi);
+        }
+        return;
+    }
+    // Cross-workgroup exchange as in the split-K decode kernel: partial tiles as stores at the
+    // agent-coherent level, a wait for them, one relaxed counter per row block; the last arriver adds
+    // the partials in a fixed order, writes Y and resets the counter.
+    float* mine = part + ((long)ks * nslots + slot) * TILE;
+    for (int t4 = tid * 4; t4 < TILE; t4 += 4 * SK3_NT) {
+        float4_t sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int p = 0; p < SK3_NWV; p++) sum += *(const float4_t*)(&red[p * TILE + t4]);
+        store_coherent_x4(mine + t4, sum);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    sk3_barrier();
+    if (tid == 0) {
+        const unsigned old = __hip_atomic_fetch_add(&counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *last_flag = (old == (unsigned)(ksplit - 1)) ? 1u : 0u;
+    }
+    sk3_barrier();
+    if (!*last_flag) return;
+    for (int t4 = tid * 4; t4 < TILE; t4 += 4 * SK3_NT) {
+        const float* src[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) src[q] = part + ((long)(q < ksplit ? q : 0) * nslots + slot) * TILE + t4;
+        float4_t pv[8];
+        load8_coherent_x4(src, pv);
+        float4_t sum = pv[0];
+#pragma unroll
+        for (int q = 1; q < 8; q++)
+            if (q < ksplit) sum += pv[q];  // fixed order
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int t = t4 + e;
+            const int l = t & 63, v = (t >> 6) & 3, rt = t >> 8;
+            const int m = 4 * (l >> 4) + v;
+            const int n = rb * ROWS + 16 * rt + (l & 15);
+            if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum[e], m, n, N, epi);
+        }
+    }
+    if (tid == 0) __hip_atomic_store(&counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int MROWS, int RT, int CH>
+__global__ __launch_bounds__(SK3_NT) void skinny3_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ZS,
+                                                         const half_t* __restrict__ X, half_t* __restrict__ Y,
+                                                         float* part, unsigned* counters, int M, int N, int K,
+                                                         int ksplit, Epilogue epi) {
+    skinny3_body<MROWS, RT, CH, SK3_DEPTH>(W, ZS, X, Y, part, counters, M, N, K, ksplit, epi, blockIdx.x, blockIdx.x, gridDim.x);
+}
+
+struct Skinny3Group {
+    const uint8_t* W[GEMV_GROUP_MAX];
+    const uint32_t* ZS[GEMV_GROUP_MAX];
+    const half_t* X[GEMV_GROUP_MAX];
+    half_t* Y[GEMV_GROUP_MAX];
+    const half_t* bias[GEMV_GROUP_MAX];
+    const half_t* residual[GEMV_GROUP_MAX];
+    int N[GEMV_GROUP_MAX];
+    int act[GEMV_GROUP_MAX];
+    int blk_end[GEMV_GROUP_MAX];  // first row block behind linear p
+    int count;
+};
+
+template <int MROWS, int RT, int CH>
+__global__ __launch_bounds__(SK3_NT) void skinny3_group_kernel(const Skinny3Group grp, float* part, unsigned* counters,
+                                                               int M, int K, int ksplit) {
+    int p = 0;
+#pragma unroll
+    for (int q = 0; q < GEMV_GROUP_MAX - 1; q++)
+        if (q + 1 < grp.count && (int)blockIdx.x >= grp.blk_end[q]) p = q + 1;
+    const int rb = blockIdx.x - (p > 0 ? grp.blk_end[p - 1] : 0);
+    const Epilogue epi{grp.bias[p], grp.residual[p], grp.act[p]};
+    skinny3_body<MROWS, RT, CH, SK3_DEPTH>(grp.W[p], grp.ZS[p], grp.X[p], grp.Y[p], part, counters, M, grp.N[p], K, ksplit, epi, rb,
+                                blockIdx.x, gridDim.x);
+}
+
+template <typename Kern>
+hipError_t allow_lds(Kern kern, int bytes, bool* done) {
+    if (bytes <= 64 * 1024) return hipSuccess;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+    if (!done[dev]) {
+        const hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e != hipSuccess) return e;
+        done[dev] = true;
+    }
+    return hipSuccess;
+}
+
+template <int MROWS, int RT, int CH>
+hipError_t launch_cfg(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K, int ksplit,
+                      Epilogue epi, hipStream_t st) {
+    static bool allowed[64];
+    constexpr int lds = Sk3Lds<MROWS, RT, CH>::BYTES;
+    const hipError_t e = allow_lds(skinny3_kernel<MROWS, RT, CH>, lds, allowed);
+    if (e != hipSuccess) return e;
+    const dim3 grid((N + 16 * RT - 1) / (16 * RT), ksplit);
+    hipLaunchKernelGGL((skinny3_kernel<MROWS, RT, CH>), grid, dim3(SK3_NT), lds, st, (const uint8_t*)w, (const uint32_t*)zs,
+                       (const half_t*)x, (half_t*)y, ws ? (float*)((char*)ws + SK3_COUNTER_BYTES) : nullptr, (unsigned*)ws,
+                       M, N, K, ksplit, epi);
+    return hipGetLastError();
+}
+
+template <int MROWS, int RT, int CH>
+hipError_t launch_group_cfg(const SeqProblem* probs, int count, void* ws, int M, int K, int ksplit, hipStream_t st) {
+    static bool allowed[64];
+    constexpr int lds = Sk3Lds<MROWS, RT, CH>::BYTES;
+    const hipError_t e = allow_lds(skinny3_group_kernel<MROWS, RT, CH>, lds, allowed);
+    if (e != hipSuccess) return e;
+    Skinny3Group g;
+    int blocks = 0;
+    for (int p = 0; p < GEMV_GROUP_MAX; p++) {
+        const SeqProblem& q = probs[p < count ? p : 0];
+        g.W[p] = (const uint8_t*)q.w;
+        g.ZS[p] = (const uint32_t*)q.zs;
+        g.X[p] = (const half_t*)q.x;
+        g.Y[p] = (half_t*)q.y;
+        g.bias[p] = (const half_t*)q.bias;
+        g.residual[p] = (const half_t*)q.residual;
+        g.N[p] = q.N;
+        g.act[p] = q.act;
+        if (p < count) blocks += (q.N + 16 * RT - 1) / (16 * RT);
+        g.blk_end[p] = blocks;
+    }
+    g.count = count;
+    hipLaunchKernelGGL((skinny3_group_kernel<MROWS, RT, CH>), dim3(blocks, ksplit), dim3(SK3_NT), lds, st, g,
+                       ws ? (float*)((char*)ws + SK3_COUNTER_BYTES) : nullptr, (unsigned*)ws, M, K, ksplit);
+    return hipGetLastError();
+}
+
+// Shape of a launch: rows per workgroup (16 RT), chunk slots per wave (CH) and the K split.  `blocks64` = 64-row
+// blocks of all linears of the launch together.
+struct Sk3Plan {
+    int rt, ch, ksplit;
+};
+
+Sk3Plan plan(int blocks64, int K, bool have_ws, int tune) {
+    const int groups = K / 128;
+    Sk3Plan p{4, 4, (groups + 31) / 32};
+    // Few rows: 16-row workgroups (four times as many) when 64-row ones would leave most CUs idle.
+    if (blocks64 * p.ksplit < 128) p.rt = 1;
+    if (tune & 0xF) p.rt = (tune & 0xF) == 1 ? 1 : 4;
+    if ((tune >> 4) & 0xF) p.ksplit = (tune >> 4) & 0xF;
+    const int cps = (groups + p.ksplit - 1) / p.ksplit;
+    p.ch = cps <= 8 ? 1 : cps <= 16 ? 2 : 4;
+    if (cps > 32 || (p.ksplit > 1 && !have_ws) || p.ksplit > 8 || (p.ksplit - 1) * cps >= groups) p.ksplit = 0;  // does not fit
+    return p;
+}
+
+}  // namespace
+
+// 5 <= M <= 16, group size 128, K % 128 == 0.  tune = rows per workgroup (1: 16, 4: 64) | ksplit << 4, 0 = heuristic.
+// hipErrorInvalidValue when the shape does not fit (K range per workgroup beyond 4096, or a K split without a workspace).
+hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
+                                int tune, Epilogue epi, hipStream_t st) {
+    if (M < 1 || M > 16 || K % 128 != 0) return hipErrorInvalidValue;
+    const Sk3Plan p = plan((N + 63) / 64, K, ws != nullptr, tune);
+    if (p.ksplit == 0) return hipErrorInvalidValue;
+    if (p.ksplit > 1 && (N + 16 * p.rt - 1) / (16 * p.rt) > 16384) return hipErrorInvalidValue;
+#define SQ_SK3(MR, RT, CH) return launch_cfg<MR, RT, CH>(x, w, zs, y, ws, M, N, K, p.ksplit, epi, st)
+#define SQ_SK3_CH(MR, RT)            \
+    do {                             \
+        if (p.ch == 1) SQ_SK3(MR, RT, 1); \
+        if (p.ch == 2) SQ_SK3(MR, RT, 2); \
+        SQ_SK3(MR, RT, 4);           \
+    } while (0)
+    if (M <= 8) {
+        if (p.rt == 1) SQ_SK3_CH(8, 1);
+        SQ_SK3_CH(8, 4);
+    }
+    if (p.rt == 1) SQ_SK3_CH(16, 1);
+    SQ_SK3_CH(16, 4);
+#undef SQ_SK3_CH
+#undef SQ_SK3
+}
+
+// Grouped launch: count in 2..GEMV_GROUP_MAX linears with the same K, group size 128, 5 <= M <= 16.
+hipError_t launch_skinny3_group(const SeqProblem* probs, int count, int M, void* ws, size_t ws_bytes, hipStream_t st) {
+    if (count < 2 || count > GEMV_GROUP_MAX || M < 1 || M > 16) return hipErrorInvalidValue;
+    const int K = probs[0].K;
+    if (K % 128 != 0) return hipErrorInvalidValue;
+    int blocks64 = 0;
+    for (int p = 0; p < count; p++) {
+        if (probs[p].K != K || probs[p].group_size != 128) return hipErrorInvalidValue;
+        blocks64 += (probs[p].N + 63) / 64;
+    }
+    const Sk3Plan pl = plan(blocks64, K, ws != nullptr, 0);
+    if (pl.ksplit == 0) return hipErrorInvalidValue;
+    if (pl.ksplit > 1 && (blocks64 * (4 / pl.rt) > 16384 || ws_bytes < skinny2_group_workspace_bytes(probs, count, M)))
+        return hipErrorInvalidValue;
+#define SQ_SK3(MR, RT, CH) return launch_group_cfg<MR, RT, CH>(probs, count, ws, M, K, pl.ksplit, st)
+#define SQ_SK3_CH(MR, RT)             \
+    do {                              \
+        if (pl.ch == 1) SQ_SK3(MR, RT, 1); \
+        if (pl.ch == 2) SQ_SK3(MR, RT, 2); \
+        SQ_SK3(MR, RT, 4);            \
+    } while (0)
+    if (M <= 8) {
+        if (pl.rt == 1) SQ_SK3_CH(8, 1);
+        SQ_SK3_CH(8, 4);
+    }
+    if (pl.rt == 1) SQ_SK3_CH(16, 1);
+    SQ_SK3_CH(16, 4);
+#undef SQ_SK3_CH
+#undef SQ_SK3
+}
+
+}  // namespace sq

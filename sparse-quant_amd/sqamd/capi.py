@@ -138,6 +138,7 @@ def gemm(x, w, zs, n, k, group_size, layout=SQ_LAYOUT_L1, algo=SQ_ALGO_AUTO, out
 
 
 SQ_ALGO_SKINNY_WS = 5
+SQ_ALGO_STREAM = 6
 _workspaces = {}
 _retired = []  # outgrown workspaces: a captured HIP graph may still hold their address
 
