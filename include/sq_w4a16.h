@@ -298,6 +298,24 @@ size_t sq_decode_attention_workspace_bytes(int B, int H, int D);
 int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, int rows, int cols, float eps,
                  void* stream);
 
+/* LayerNorm followed by the fused linear, y = act(LN(x) W_hat^T + bias) + residual, as ONE entry point: what a
+ * pre-LN decoder layer does in front of q/k/v and fc1 (reference: test/nvidia/module/opt/modeling_opt_ours.py:
+ * 561-562 with 505-506, and 603-604 with 608; nn.LayerNorm and the linear are separate modules there).
+ * Where sq_w4a16_ln_fusable() says 1 (layout L1, group size 128, up to 8 tokens, 2048 < K <= 4096) the
+ * normalisation happens inside the linear's kernel: every workgroup of the streaming decode kernel stages the
+ * whole activation rows in LDS anyway, computes mean and variance there while its first weights are in flight,
+ * and no LayerNorm launch, no normalised copy in memory and no second read of it exist; x_norm is then not
+ * touched and may be NULL.  Otherwise sq_layernorm writes x_norm [M, K] (fp16, caller-allocated, must not be NULL)
+ * and the linear runs on it through the automatic dispatch (workspace as for sq_w4a16_gemm_fused, may be NULL).
+ * Same arithmetic as sq_layernorm (fp32 statistics, mean first, then the variance around it, one rounding to
+ * fp16); the summation order of the statistics differs, so the normalised row can differ from sq_layernorm's by
+ * one fp16 ulp in rare elements.  ln_gamma / ln_beta fp16 [K] or NULL. */
+int sq_w4a16_ln_fusable(int M, int N, int K, int group_size, int layout);
+int sq_w4a16_gemm_ln_fused(const void* x, const void* ln_gamma, const void* ln_beta, float ln_eps, void* x_norm,
+                           const void* w, const void* zs, const void* bias, const void* residual, void* y, int M, int N,
+                           int K, int group_size, int layout, int act, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
 #ifdef __cplusplus
 }
 #endif

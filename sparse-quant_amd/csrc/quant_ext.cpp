@@ -141,9 +141,16 @@ at::Tensor workspace_for(const at::Tensor& like, void* stream, size_t bytes) {
     return ws;
 }
 
+// LayerNorm in front of the linear (weight / bias fp16 [K] or absent).
+struct LnArgs {
+    c10::optional<at::Tensor> weight, bias;
+    double eps;
+};
+
 at::Tensor gemm_impl(const at::Tensor& I, const at::Tensor& W, const at::Tensor& ZS, int N, int group_size, int algo,
                      const c10::optional<at::Tensor>& bias = c10::nullopt,
-                     const c10::optional<at::Tensor>& residual = c10::nullopt, int act = SQ_ACT_NONE) {
+                     const c10::optional<at::Tensor>& residual = c10::nullopt, int act = SQ_ACT_NONE,
+                     const LnArgs* ln = nullptr) {
     SQ_CHECK_DEVICE(I);
     SQ_CHECK_DEVICE(W);
     SQ_CHECK_DEVICE(ZS);
@@ -203,10 +210,31 @@ at::Tensor gemm_impl(const at::Tensor& I, const at::Tensor& W, const at::Tensor&
     void* ws_ptr = nullptr;
     size_t ws_bytes = 0;
     at::Tensor ws;
-    if (M > 4 && M <= 1024 && ((algo & 0xFF) == SQ_ALGO_AUTO || (algo & 0xFF) == SQ_ALGO_SKINNY_WS)) {
+    if (M > 2 && M <= 1024 && ((algo & 0xFF) == SQ_ALGO_AUTO || (algo & 0xFF) == SQ_ALGO_SKINNY_WS || (algo & 0xFF) == SQ_ALGO_STREAM)) {
         ws = workspace_for(I, stream, sq_w4a16_workspace_bytes((int)M, N, (int)K));
         ws_ptr = ws.data_ptr();
         ws_bytes = (size_t)ws.numel();
+    }
+    if (ln) {
+        const void* g_ptr = nullptr;
+        const void* b_ptr = nullptr;
+        for (int which = 0; which < 2; which++) {
+            const c10::optional<at::Tensor>& t = which ? ln->bias : ln->weight;
+            if (!t.has_value() || !t->defined()) continue;
+            SQ_CHECK_DEVICE((*t));
+            SQ_CHECK_CONTIGUOUS((*t));
+            SQ_CHECK_DTYPE((*t), at::kHalf);
+            if (t->numel() != K) throw std::invalid_argument("LayerNorm parameters must have K elements!");
+            (which ? b_ptr : g_ptr) = t->data_ptr();
+        }
+        at::Tensor scratch;  // normalised rows, only where the kernel cannot normalise in place
+        if (!sq_w4a16_ln_fusable((int)M, N, (int)K, group_size, SQ_LAYOUT_L1)) scratch = torch::empty_like(I);
+        raise_if_error(sq_w4a16_gemm_ln_fused(I.data_ptr(), g_ptr, b_ptr, (float)ln->eps,
+                                              scratch.defined() ? scratch.data_ptr() : nullptr, w_ptr, zs_ptr, bias_ptr,
+                                              res_ptr, O.data_ptr(), (int)M, N, (int)K, group_size, SQ_LAYOUT_L1, act,
+                                              ws_ptr, ws_bytes, stream),
+                       "gemm_awq_ln_fused_ut");
+        return O;
     }
     raise_if_error(sq_w4a16_gemm_fused(I.data_ptr(), w_ptr, zs_ptr, bias_ptr, res_ptr, O.data_ptr(), (int)M, N, (int)K,
                                        group_size, SQ_LAYOUT_L1, act, algo, ws_ptr, ws_bytes, stream),
@@ -244,6 +272,22 @@ at::Tensor gemm_awq_fused_ut(at::Tensor I, at::Tensor W, at::Tensor W_zeros_scal
     else if (act != "none" && !act.empty())
         throw std::invalid_argument("unknown activation: " + act);
     return gemm_impl(I, W, W_zeros_scales, N, group_size, SQ_ALGO_AUTO, bias, residual, a);
+}
+
+// act(LayerNorm(I) W_hat^T + bias) + residual: the pre-LN pattern of a decoder layer (nn.LayerNorm followed by
+// the linear).  With up to 8 tokens, group size 128 and 2048 < K <= 4096 the normalisation happens inside the
+// linear's kernel; otherwise a LayerNorm launch into a temporary comes first.
+at::Tensor gemm_awq_ln_fused_ut(at::Tensor I, c10::optional<at::Tensor> ln_weight, c10::optional<at::Tensor> ln_bias,
+                                double ln_eps, at::Tensor W, at::Tensor W_zeros_scales, c10::optional<at::Tensor> bias,
+                                c10::optional<at::Tensor> residual, const std::string& act, const int N,
+                                const int group_size) {
+    int a = SQ_ACT_NONE;
+    if (act == "relu")
+        a = SQ_ACT_RELU;
+    else if (act != "none" && !act.empty())
+        throw std::invalid_argument("unknown activation: " + act);
+    const LnArgs ln{ln_weight, ln_bias, ln_eps};
+    return gemm_impl(I, W, W_zeros_scales, N, group_size, SQ_ALGO_AUTO, bias, residual, a, &ln);
 }
 
 // Same with an explicit kernel id (SQ_ALGO_* | tuning word << 8); for tests and benchmarks.
@@ -366,6 +410,10 @@ PYBIND11_MODULE(quant, m) {
     m.def("gemm_awq_algo", &gemm_awq_algo);
     m.def("gemm_awq_residual_ut", &gemm_awq_residual_ut);
     m.def("gemm_awq_fused_ut", &gemm_awq_fused_ut, py::arg("I"), py::arg("W"), py::arg("W_zeros_scales"),
+          py::arg("bias") = py::none(), py::arg("residual") = py::none(), py::arg("act") = "none", py::arg("N"),
+          py::arg("group_size"));
+    m.def("gemm_awq_ln_fused_ut", &gemm_awq_ln_fused_ut, py::arg("I"), py::arg("ln_weight") = py::none(),
+          py::arg("ln_bias") = py::none(), py::arg("ln_eps") = 1e-5, py::arg("W"), py::arg("W_zeros_scales"),
           py::arg("bias") = py::none(), py::arg("residual") = py::none(), py::arg("act") = "none", py::arg("N"),
           py::arg("group_size"));
     m.def("convert_2bit_to_4bit", &convert_2bit_to_4bit);

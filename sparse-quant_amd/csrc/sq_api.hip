@@ -101,7 +101,10 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
         // 5..16 tokens at group size 128: the streaming kernel wherever its K range fits (a K beyond 4096
         // needs the workspace).  Against the split-K kernel at 8 tokens: fc1 10.0 against 13.3 us, q/k/v in
         // one launch 8.6 against 12.1, fc2 12.7 against 14.6; against the GEMV on 4096 x 4096: 4.9 against 6.5.
-        const bool stream_ok = M > 4 && M <= 16 && group_size == 128 && K % 128 == 0 && (K <= 4096 || (ws_ok && K <= 32768));
+        // With 3 or 4 tokens it also beats the GEMV on fc1 / fc2-class weights (9.7 against 10.7 us, 11.9 against
+        // 13.6 us at 4 tokens); on 4096 x 4096 and with 1 or 2 tokens the GEMV stays ahead.
+        const bool stream_ok = (M > 4 || (M >= 3 && large)) && M <= 16 && group_size == 128 && K % 128 == 0 &&
+                               (K <= 4096 || (ws_ok && K <= 32768));
         if (stream_ok) {
             kernel = SQ_ALGO_STREAM;
         } else if (ws_ok && M > 4 && M <= 32 && (large || M > 16 || K > 8192)) {
@@ -150,7 +153,7 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
             if (M > 16 || group_size != 128) return SQ_ERR_BAD_ALGO;
             const bool ws_fits = workspace && aligned16(workspace) &&
                                  workspace_bytes >= sq::skinny2_workspace_bytes(M, N, K);
-            const hipError_t e = sq::launch_skinny3_tuned(x, w, zs, y, ws_fits ? workspace : nullptr, M, N, K, tune, epi, st);
+            const hipError_t e = sq::launch_skinny3_tuned(x, w, zs, y, ws_fits ? workspace : nullptr, M, N, K, tune, epi, nullptr, st);
             return e == hipErrorInvalidValue ? SQ_ERR_WORKSPACE : launch_code(e);
         }
         case SQ_ALGO_GEMM:
@@ -246,8 +249,8 @@ int sq_workspace_check(const void* workspace, size_t bytes, void* stream) {
 
 size_t sq_w4a16_gemv_sequence_workspace_bytes(const sq_linear_desc* linears, int count, int M) {
     size_t need = sq::gemv_seq_workspace_bytes();
-    if (!linears || count <= 0 || count > SQ_SEQUENCE_MAX || M <= 4) return need;
-    // more than 4 tokens: what sq_w4a16_gemm_ws wants for the largest run of linears that may share a launch
+    if (!linears || count <= 0 || count > SQ_SEQUENCE_MAX || M <= 2) return need;
+    // more than 2 tokens: what sq_w4a16_gemm_ws wants for the largest run of linears that may share a launch
     // (their rows concatenated, each rounded up to a 64-row block) and for every single linear
     long rows = 0;
     int kmax = 0;
@@ -341,7 +344,7 @@ int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int 
                 const sq::Epilogue epi{static_cast<const sq::half_t*>(q.bias), static_cast<const sq::half_t*>(q.residual),
                                        q.act};
                 const int rc = gemm_dispatch(q.x, q.w, q.zs, q.y, M, q.N, q.K, q.group_size, layout, SQ_ALGO_AUTO, epi,
-                                             M > 4 ? workspace : nullptr, M > 4 ? workspace_bytes : 0, stream);
+                                             M > 2 ? workspace : nullptr, M > 2 ? workspace_bytes : 0, stream);
                 if (rc != SQ_OK) return rc;
             }
         }
@@ -469,6 +472,44 @@ int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, in
     if (!aligned16(x) || !aligned16(y) || (gamma && !aligned16(gamma)) || (beta && !aligned16(beta)))
         return SQ_ERR_MISALIGNED;
     return launch_code(sq::launch_layernorm(x, gamma, beta, y, rows, cols, eps, static_cast<hipStream_t>(stream)));
+}
+
+int sq_w4a16_ln_fusable(int M, int N, int K, int group_size, int layout) {
+    return layout == SQ_LAYOUT_L1 && M >= 1 && M <= 8 && N > 0 && group_size == 128 && K % 128 == 0 && K > 2048 &&
+                   K <= 4096
+               ? 1
+               : 0;
+}
+
+int sq_w4a16_gemm_ln_fused(const void* x, const void* ln_gamma, const void* ln_beta, float ln_eps, void* x_norm,
+                           const void* w, const void* zs, const void* bias, const void* residual, void* y, int M, int N,
+                           int K, int group_size, int layout, int act, void* workspace, size_t workspace_bytes,
+                           void* stream) {
+    if (act != SQ_ACT_NONE && act != SQ_ACT_RELU) return SQ_ERR_BAD_ALGO;
+    if (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)) return SQ_ERR_MISALIGNED;
+    if (residual && (reinterpret_cast<uintptr_t>(residual) & 1u)) return SQ_ERR_MISALIGNED;
+    if ((ln_gamma && !aligned16(ln_gamma)) || (ln_beta && !aligned16(ln_beta))) return SQ_ERR_MISALIGNED;
+    if (M < 0) return SQ_ERR_BAD_SHAPE;
+    const int rc = check_weight(N, K, group_size, layout);
+    if (rc != SQ_OK) return rc;
+    if (layout != SQ_LAYOUT_L1) return SQ_ERR_BAD_LAYOUT;
+    if (M == 0) return SQ_OK;
+    const sq::Epilogue epi{static_cast<const sq::half_t*>(bias), static_cast<const sq::half_t*>(residual), act};
+    if (sq_w4a16_ln_fusable(M, N, K, group_size, layout)) {
+        if (!x || !w || !zs || !y) return SQ_ERR_NULL_POINTER;
+        if (!aligned16(x) || !aligned16(w) || !aligned16(zs) || !aligned16(y)) return SQ_ERR_MISALIGNED;
+        const sq::LnPre ln{static_cast<const sq::half_t*>(ln_gamma), static_cast<const sq::half_t*>(ln_beta), ln_eps};
+        const hipError_t e = sq::launch_skinny3_tuned(x, w, zs, y, nullptr, M, N, K, 0, epi, &ln,
+                                                      static_cast<hipStream_t>(stream));
+        if (e != hipErrorInvalidValue) return launch_code(e);
+    }
+    // Not fusable: the LayerNorm kernel into the caller's scratch rows, then the linear on those.
+    if (!x_norm) return SQ_ERR_NULL_POINTER;
+    if (K > 16384) return SQ_ERR_BAD_SHAPE;
+    const int rl = sq_layernorm(x, ln_gamma, ln_beta, x_norm, M, K, ln_eps, stream);
+    if (rl != SQ_OK) return rl;
+    return gemm_dispatch(x_norm, w, zs, y, M, N, K, group_size, layout, SQ_ALGO_AUTO, epi, workspace, workspace_bytes,
+                         stream);
 }
 
 }  // extern "C"

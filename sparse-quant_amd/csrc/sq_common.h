@@ -121,6 +121,14 @@ __device__ __forceinline__ half8_t unpack8_mixed(uint32_t w, const NibbleMasks& 
 
 __device__ __forceinline__ int imin(int a, int b) { return a < b ? a : b; }
 
+// LayerNorm applied to the activations on their way into a linear (fp32 statistics over the K columns of a
+// token, biased variance, one rounding to fp16): x_hat = (x - mean) * rsqrt(var + eps) * gamma + beta.
+struct LnPre {
+    const half_t* gamma;  // [K] or null (1)
+    const half_t* beta;   // [K] or null (0)
+    float eps;
+};
+
 // What happens to an fp32 accumulator on its way to Y[m, n]: + bias[n], activation,
 // + residual[m, n] (each optional), one rounding to fp16 at the end.
 struct Epilogue {

@@ -59,18 +59,19 @@ struct Sk3Lds {
     static constexpr int RED_BYTES = SK3_NWV * TILE * 4;
     static constexpr int Z_OFF = X_BYTES > RED_BYTES ? X_BYTES : RED_BYTES;  // the partials reuse the activations' space
     static constexpr int FLAG_OFF = Z_OFF + 16 * RT * SK3_ZPITCH * 4;
-    static constexpr int BYTES = FLAG_OFF + 16;
+    static constexpr int LN_OFF = FLAG_OFF + 16;         // fused LayerNorm: mean and reciprocal deviation per token
+    static constexpr int BYTES = LN_OFF + 2 * MROWS * 4;
 };
 
 __device__ __forceinline__ void sk3_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // rb = row block inside this linear; slot = index of the row block in the workspace, which differs from
 // rb when several linears share a launch.
-template <int MROWS, int RT, int CH, int DEPTH>
+template <int MROWS, int RT, int CH, int DEPTH, bool LN>
 __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ZS,
                                              const half_t* __restrict__ X, half_t* __restrict__ Y, float* part,
                                              unsigned* counters, int M, int N, int K, int ksplit, const Epilogue& epi,
-                                             int rb, int slot, int nslots) {
+                                             const LnPre& ln, int rb, int slot, int nslots) {
     using L = Sk3Lds<MROWS, RT, CH>;
     constexpr int ROWS = 16 * RT;
     constexpr int TILE = L::TILE;
@@ -79,6 +80,7 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     constexpr int ZPT = (ROWS * 32 + SK3_NT - 1) / SK3_NT;
     static_assert(CH == 1 || CH == 2 || CH == 4, "chunk slots per wave");
     static_assert(MROWS * WPR % SK3_NT == 0, "activation words divide over the threads");
+    static_assert(!LN || WPR == SK3_NT, "fused LayerNorm: thread t holds columns 8t .. 8t+7 of every token");
 
     extern __shared__ __attribute__((aligned(16))) uint8_t sk3_lds[];
     uint8_t* xl = sk3_lds;
@@ -118,13 +120,31 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
         const int idx = tid + p * SK3_NT;
         const int m = idx / WPR, col = idx % WPR;
         const bool ok = (m < M) && (col < nc * 16);
+        // (masked with an AND, not selected: a select lets the compiler move the load under a branch, and its
+        // wait counts around loads under branches are conservative)
+        const uint32_t keep = ok ? 0xffffffffu : 0u;
         const u32x4_t v = *(const u32x4_t*)(X + (ok ? (long)m * K + c_begin * 128 + col * 8 : 0));
-        xr[p] = ok ? v : (u32x4_t){0u, 0u, 0u, 0u};
+        xr[p] = (u32x4_t){v.x & keep, v.y & keep, v.z & keep, v.w & keep};
+    }
+    // (fused LayerNorm: its scale and shift for this thread's eight columns)
+    u32x4_t lg = {0x3c003c00u, 0x3c003c00u, 0x3c003c00u, 0x3c003c00u}, lb = {0u, 0u, 0u, 0u};
+    if (LN) {
+        // unconditional loads (a missing scale or shift reads the activations' first bytes and is masked out)
+        const bool ok = tid < nc * 16;
+        const long off = ok ? c_begin * 128 + tid * 8 : 0;
+        const uint32_t kg = ln.gamma ? 0xffffffffu : 0u, kb = ln.beta ? 0xffffffffu : 0u;
+        const u32x4_t gv = *(const u32x4_t*)((ln.gamma ? ln.gamma : X) + off);
+        const u32x4_t bv = *(const u32x4_t*)((ln.beta ? ln.beta : X) + off);
+        lg = (u32x4_t){(gv.x & kg) | (lg.x & ~kg), (gv.y & kg) | (lg.y & ~kg), (gv.z & kg) | (lg.z & ~kg),
+                       (gv.w & kg) | (lg.w & ~kg)};
+        lb = (u32x4_t){bv.x & kb, bv.y & kb, bv.z & kb, bv.w & kb};
     }
     // Every wave has issued its activation loads before any wave issues a weight load: a CU serves its
     // vector memory requests in order, and activations queued behind another wave's sixteen weight loads
     // would reach the barrier below only when most of the stream has already arrived.
+    __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);  // nothing that waits for a load moves above the weight requests
     // 3. the wave's weight loads, in units of four (two row tiles x the two 64-byte halves of a 128-byte
     //    line back to back, so that the line is requested from L2 once), DEPTH units ahead of the arithmetic
     constexpr int RTU = RT >= 2 ? 2 : 1;        // row tiles per unit
@@ -149,9 +169,74 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
                     *(const u32x4_t*)(wrow[RTU * rg + r] + (long)(c_begin + (cl < nc ? cl : 0)) * 64);
             }
     };
+    // (in front of a fused LayerNorm a 16-row workgroup, whose units are two loads, sends two of them: measured)
+    constexpr int PRE = (LN && RT == 1) ? 2 : SK3_DEPTH_PRE;
+    constexpr int STEADY = LN ? (DEPTH > PRE ? DEPTH : PRE) : DEPTH;
 #pragma unroll
     for (int un = 0; un < NU; un++)
-        if (un < SK3_DEPTH_PRE) issue_unit(un);
+        if (un < PRE) issue_unit(un);
+    __builtin_amdgcn_sched_barrier(0);
+    // (fused LayerNorm, while the first weights are on their way: thread t holds columns 8t .. 8t+7 of every
+    // token.  Per-thread partial sums go to LDS (the activations' space, not yet in use), wave w adds up the 512
+    // partials of token w and leaves the statistic where every thread reads it; mean first, then the squared
+    // deviations around it.  The normalised row replaces the raw one before it is parked.)
+    if (LN) {
+        float* scr = (float*)sk3_lds;                    // [MROWS][512] partials
+        float* stat = (float*)(sk3_lds + L::LN_OFF);     // [2][MROWS]: mean, 1 / sqrt(var + eps)
+        const bool cok = tid < nc * 16;
+        const float inv_k = 1.f / (float)(nc * 128);
+        auto token_sums = [&](const float (&part)[XPT], int which, bool finish_var) {
+#pragma unroll
+            for (int p = 0; p < XPT; p++) scr[p * SK3_NT + tid] = part[p];
+            sk3_barrier();
+            if (wave < MROWS) {
+                float a = 0.f;
+#pragma unroll
+                for (int j = 0; j < SK3_NT / 64; j++) a += scr[wave * SK3_NT + lane + 64 * j];
+                a = row_sum_stride4(quad_sum(a));  // every lane: the sum of its 16-lane row
+                const float tot = (bit_cast<float>(__builtin_amdgcn_readlane(bit_cast<int>(a), 0)) +
+                                   bit_cast<float>(__builtin_amdgcn_readlane(bit_cast<int>(a), 16))) +
+                                  (bit_cast<float>(__builtin_amdgcn_readlane(bit_cast<int>(a), 32)) +
+                                   bit_cast<float>(__builtin_amdgcn_readlane(bit_cast<int>(a), 48)));
+                if (lane == 0) stat[which * MROWS + wave] = finish_var ? rsqrtf(tot * inv_k + ln.eps) : tot * inv_k;
+            }
+            sk3_barrier();
+        };
+        float part[XPT], mean[XPT];
+#pragma unroll
+        for (int p = 0; p < XPT; p++) {
+            const half8_t h = bit_cast<half8_t>(xr[p]);
+            float a = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) a += (float)h[e];
+            part[p] = a;  // zero where the token or the column does not exist
+        }
+        token_sums(part, 0, false);
+#pragma unroll
+        for (int p = 0; p < XPT; p++) {
+            mean[p] = stat[p];
+            const half8_t h = bit_cast<half8_t>(xr[p]);
+            float q = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float dlt = (float)h[e] - mean[p];
+                q += dlt * dlt;
+            }
+            part[p] = cok ? q : 0.f;
+        }
+        token_sums(part, 1, true);
+        const half8_t g8 = bit_cast<half8_t>(lg), b8 = bit_cast<half8_t>(lb);
+#pragma unroll
+        for (int p = 0; p < XPT; p++) {
+            const float rstd = stat[MROWS + p];
+            const half8_t h = bit_cast<half8_t>(xr[p]);
+            half8_t o;
+#pragma unroll
+            for (int e = 0; e < 8; e++) o[e] = (half_t)(((float)h[e] - mean[p]) * rstd * (float)g8[e] + (float)b8[e]);
+            xr[p] = (cok && p < M) ? bit_cast<u32x4_t>(o) : (u32x4_t){0u, 0u, 0u, 0u};
+        }
+        sk3_barrier();  // the partials' space becomes the activations' space
+    }
     // 4. park zeros/scales and activations (waits for 1 and 2 only: the weight loads stay in flight)
 #pragma unroll
     for (int p = 0; p < ZPT; p++) {
@@ -176,13 +261,13 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     const half8_t m960 = {(half_t)-960.f, (half_t)-960.f, (half_t)0.f, (half_t)0.f,
                           (half_t)-960.f, (half_t)-960.f, (half_t)0.f, (half_t)0.f};
 #pragma unroll
-    for (int un = SK3_DEPTH_PRE; un < NU; un++)
-        if (un < DEPTH) issue_unit(un);
+    for (int un = PRE; un < NU; un++)
+        if (un < STEADY) issue_unit(un);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int un = 0; un < NU; un++) {
-        if (un + DEPTH < NU) {
-            issue_unit(un + DEPTH);
+        if (un + STEADY < NU) {
+            issue_unit(un + STEADY);
             __builtin_amdgcn_sched_barrier(0);  // the request goes out here, not wherever the scheduler finds room
         }
         const int pr = un / RG, rg = un % RG;
@@ -282,12 +367,13 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     if (tid == 0) __hip_atomic_store(&counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int MROWS, int RT, int CH>
+template <int MROWS, int RT, int CH, bool LN>
 __global__ __launch_bounds__(SK3_NT) void skinny3_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ZS,
                                                          const half_t* __restrict__ X, half_t* __restrict__ Y,
                                                          float* part, unsigned* counters, int M, int N, int K,
-                                                         int ksplit, Epilogue epi) {
-    skinny3_body<MROWS, RT, CH, SK3_DEPTH>(W, ZS, X, Y, part, counters, M, N, K, ksplit, epi, blockIdx.x, blockIdx.x, gridDim.x);
+                                                         int ksplit, Epilogue epi, LnPre ln) {
+    skinny3_body<MROWS, RT, CH, SK3_DEPTH, LN>(W, ZS, X, Y, part, counters, M, N, K, ksplit, epi, ln, blockIdx.x, blockIdx.x,
+                                               gridDim.x);
 }
 
 struct Skinny3Group {
@@ -312,8 +398,8 @@ __global__ __launch_bounds__(SK3_NT) void skinny3_group_kernel(const Skinny3Grou
         if (q + 1 < grp.count && (int)blockIdx.x >= grp.blk_end[q]) p = q + 1;
     const int rb = blockIdx.x - (p > 0 ? grp.blk_end[p - 1] : 0);
     const Epilogue epi{grp.bias[p], grp.residual[p], grp.act[p]};
-    skinny3_body<MROWS, RT, CH, SK3_DEPTH>(grp.W[p], grp.ZS[p], grp.X[p], grp.Y[p], part, counters, M, grp.N[p], K, ksplit, epi, rb,
-                                blockIdx.x, gridDim.x);
+    skinny3_body<MROWS, RT, CH, SK3_DEPTH, false>(grp.W[p], grp.ZS[p], grp.X[p], grp.Y[p], part, counters, M, grp.N[p], K,
+                                                  ksplit, epi, LnPre{nullptr, nullptr, 0.f}, rb, blockIdx.x, gridDim.x);
 }
 
 template <typename Kern>
@@ -329,17 +415,17 @@ hipError_t allow_lds(Kern kern, int bytes, bool* done) {
     return hipSuccess;
 }
 
-template <int MROWS, int RT, int CH>
+template <int MROWS, int RT, int CH, bool LN>
 hipError_t launch_cfg(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K, int ksplit,
-                      Epilogue epi, hipStream_t st) {
+                      Epilogue epi, LnPre ln, hipStream_t st) {
     static bool allowed[64];
     constexpr int lds = Sk3Lds<MROWS, RT, CH>::BYTES;
-    const hipError_t e = allow_lds(skinny3_kernel<MROWS, RT, CH>, lds, allowed);
+    const hipError_t e = allow_lds(skinny3_kernel<MROWS, RT, CH, LN>, lds, allowed);
     if (e != hipSuccess) return e;
     const dim3 grid((N + 16 * RT - 1) / (16 * RT), ksplit);
-    hipLaunchKernelGGL((skinny3_kernel<MROWS, RT, CH>), grid, dim3(SK3_NT), lds, st, (const uint8_t*)w, (const uint32_t*)zs,
-                       (const half_t*)x, (half_t*)y, ws ? (float*)((char*)ws + SK3_COUNTER_BYTES) : nullptr, (unsigned*)ws,
-                       M, N, K, ksplit, epi);
+    hipLaunchKernelGGL((skinny3_kernel<MROWS, RT, CH, LN>), grid, dim3(SK3_NT), lds, st, (const uint8_t*)w,
+                       (const uint32_t*)zs, (const half_t*)x, (half_t*)y,
+                       ws ? (float*)((char*)ws + SK3_COUNTER_BYTES) : nullptr, (unsigned*)ws, M, N, K, ksplit, epi, ln);
     return hipGetLastError();
 }
 
@@ -391,21 +477,40 @@ Sk3Plan plan(int blocks64, int K, bool have_ws, int tune) {
 
 }  // namespace
 
-// 5 <= M <= 16, group size 128, K % 128 == 0.  tune = rows per workgroup (1: 16, 4: 64) | ksplit << 4, 0 = heuristic.
-// hipErrorInvalidValue when the shape does not fit (K range per workgroup beyond 4096, or a K split without a workspace).
+// M <= 16, group size 128, K % 128 == 0.  tune = rows per workgroup (1: 16, 4: 64) | ksplit << 4, 0 = heuristic.
+// ln (may be null): LayerNorm of the activations inside the kernel; possible when a workgroup holds whole rows
+// (2048 < K <= 4096, no K split) of at most 8 tokens.  hipErrorInvalidValue when the shape does not fit (K range per workgroup beyond
+// 4096, a K split without a workspace, or a LayerNorm over rows the workgroup does not hold whole).
 hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
-                                int tune, Epilogue epi, hipStream_t st) {
+                                int tune, Epilogue epi, const LnPre* ln, hipStream_t st) {
     if (M < 1 || M > 16 || K % 128 != 0) return hipErrorInvalidValue;
     const Sk3Plan p = plan((N + 63) / 64, K, ws != nullptr, tune);
     if (p.ksplit == 0) return hipErrorInvalidValue;
     if (p.ksplit > 1 && (N + 16 * p.rt - 1) / (16 * p.rt) > 16384) return hipErrorInvalidValue;
-#define SQ_SK3(MR, RT, CH) return launch_cfg<MR, RT, CH>(x, w, zs, y, ws, M, N, K, p.ksplit, epi, st)
+    if (ln) {
+        if (p.ksplit != 1 || p.ch != 4) return hipErrorInvalidValue;
+#define SQ_SK3_LN(MR, RT) return launch_cfg<MR, RT, 4, true>(x, w, zs, y, ws, M, N, K, 1, epi, *ln, st)
+        if (M <= 4) {
+            if (p.rt == 1) SQ_SK3_LN(4, 1);
+            SQ_SK3_LN(4, 4);
+        }
+        if (M > 8) return hipErrorInvalidValue;  // sixteen rows of statistics per thread do not fit the registers
+        if (p.rt == 1) SQ_SK3_LN(8, 1);
+        SQ_SK3_LN(8, 4);
+#undef SQ_SK3_LN
+    }
+    const LnPre none{nullptr, nullptr, 0.f};
+#define SQ_SK3(MR, RT, CH) return launch_cfg<MR, RT, CH, false>(x, w, zs, y, ws, M, N, K, p.ksplit, epi, none, st)
 #define SQ_SK3_CH(MR, RT)            \
     do {                             \
         if (p.ch == 1) SQ_SK3(MR, RT, 1); \
         if (p.ch == 2) SQ_SK3(MR, RT, 2); \
         SQ_SK3(MR, RT, 4);           \
     } while (0)
+    if (M <= 4) {
+        if (p.rt == 1) SQ_SK3_CH(4, 1);
+        SQ_SK3_CH(4, 4);
+    }
     if (M <= 8) {
         if (p.rt == 1) SQ_SK3_CH(8, 1);
         SQ_SK3_CH(8, 4);
@@ -437,6 +542,10 @@ hipError_t launch_skinny3_group(const SeqProblem* probs, int count, int M, void*
         if (pl.ch == 2) SQ_SK3(MR, RT, 2); \
         SQ_SK3(MR, RT, 4);            \
     } while (0)
+    if (M <= 4) {
+        if (pl.rt == 1) SQ_SK3_CH(4, 1);
+        SQ_SK3_CH(4, 4);
+    }
     if (M <= 8) {
         if (pl.rt == 1) SQ_SK3_CH(8, 1);
         SQ_SK3_CH(8, 4);

@@ -42,6 +42,9 @@ SIGNATURES = {
                                  _vp]),
     "sq_decode_attention_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
     "sq_layernorm": (_i, [_vp, _vp, _vp, _vp, _i, _i, ctypes.c_float, _vp]),
+    "sq_w4a16_ln_fusable": (_i, [_i, _i, _i, _i, _i]),
+    "sq_w4a16_gemm_ln_fused": (_i, [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
+                                    _vp, ctypes.c_size_t, _vp]),
     "sq_lut_attention_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, ctypes.c_float, _i, _vp]),
 }
 
@@ -209,11 +212,30 @@ def gemm_fused(x, w, zs, n, k, group_size, bias=None, residual=None, act=SQ_ACT_
     m = x.numel() // k
     if out is None:
         out = torch.empty((m, n), dtype=torch.float16, device=x.device)
-    if ws is None and use_workspace and 4 < m <= 1024:
+    if ws is None and use_workspace and 2 < m <= 1024:
         ws = workspace(m, n, k, x.device, stream)
     _check(lib().sq_w4a16_gemm_fused(_ptr(x), _ptr(w), _ptr(zs), _ptr(bias), _ptr(residual), _ptr(out), m, n, k,
                                      group_size, SQ_LAYOUT_L1, act, algo, _ptr(ws), 0 if ws is None else ws.numel(),
                                      _stream(stream)), "sq_w4a16_gemm_fused")
+    return out
+
+
+def gemm_ln_fused(x, ln_gamma, ln_beta, ln_eps, w, zs, n, k, group_size, bias=None, residual=None, act=SQ_ACT_NONE,
+                  out=None, stream=None, ws=None):
+    """y = act(LayerNorm(x) W_hat^T + bias) + residual through sq_w4a16_gemm_ln_fused (the normalisation inside the
+    linear's kernel where sq_w4a16_ln_fusable says so, the LayerNorm kernel into a scratch tensor otherwise)."""
+    m = x.numel() // k
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
+    scratch = None
+    if not lib().sq_w4a16_ln_fusable(m, n, k, group_size, SQ_LAYOUT_L1):
+        scratch = torch.empty((m, k), dtype=torch.float16, device=x.device)
+        if ws is None and 2 < m <= 1024:
+            ws = workspace(m, n, k, x.device, stream)
+    _check(lib().sq_w4a16_gemm_ln_fused(_ptr(x), _ptr(ln_gamma), _ptr(ln_beta), float(ln_eps), _ptr(scratch), _ptr(w),
+                                        _ptr(zs), _ptr(bias), _ptr(residual), _ptr(out), m, n, k, group_size, SQ_LAYOUT_L1,
+                                        act, _ptr(ws), 0 if ws is None else ws.numel(), _stream(stream)),
+           "sq_w4a16_gemm_ln_fused")
     return out
 
 

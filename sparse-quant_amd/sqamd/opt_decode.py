@@ -56,16 +56,22 @@ class DecoderLayer(nn.Module):
         self.fc1 = _random_walinear(hidden, ffn, g, dev, gen, scale_std, scale_min)
         self.fc2 = _random_walinear(ffn, hidden, g, dev, gen, scale_std, scale_min)
         self.qkv_proj = None
+        self.fuse_ln = True  # LayerNorm inside the q/k/v and fc1 launches
 
     def forward(self, x, kc, vc, pos0):
         """x [B, T, H]; kc, vc [B, heads, Lmax, hd]; writes cache rows pos0 .. pos0+T-1."""
         b, t, hdim = x.shape
-        h = _layernorm(self.ln1, x)
-        flat = h.reshape(1, b * t, hdim)  # the reference flattens to [1, bs*seq, K] as well
         if self.qkv_proj is not None:
-            qkv = self.qkv_proj(flat).view(b, t, 3, self.heads, self.hd)
+            # the first LayerNorm rides in the q/k/v launch (inside the kernel at decode batch sizes)
+            flat = x.reshape(1, b * t, hdim)  # the reference flattens to [1, bs*seq, K] as well
+            if self.fuse_ln:
+                qkv = self.qkv_proj(flat, pre_ln=self.ln1)
+            else:
+                qkv = self.qkv_proj(_layernorm(self.ln1, x).reshape(1, b * t, hdim))
+            qkv = qkv.view(b, t, 3, self.heads, self.hd)
             q, k, v = (qkv[:, :, j].transpose(1, 2) for j in range(3))
         else:
+            flat = _layernorm(self.ln1, x).reshape(1, b * t, hdim)
             q = self.q_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
             k = self.k_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
             v = self.v_proj(flat).view(b, t, self.heads, self.hd).transpose(1, 2)
@@ -81,8 +87,10 @@ class DecoderLayer(nn.Module):
             a = capi.decode_attention(q, kc, vc, pos0, 1.0 / math.sqrt(self.hd), k_new=k, v_new=v).view(1, b * t, hdim)
         # bias, ReLU and the two residual adds ride in the kernels' stores
         x = self.out_proj(a, residual=x.reshape(1, b * t, hdim)).view(b, t, hdim)
-        h = _layernorm(self.ln2, x).reshape(1, b * t, hdim)
-        h = self.fc1(h, act="relu")
+        if self.fuse_ln:
+            h = self.fc1(x.reshape(1, b * t, hdim), act="relu", pre_ln=self.ln2)  # the second LayerNorm rides in fc1
+        else:
+            h = self.fc1(_layernorm(self.ln2, x).reshape(1, b * t, hdim), act="relu")
         return self.fc2(h, residual=x.reshape(1, b * t, hdim)).view(b, t, hdim)
 
     def fuse_qkv(self):
@@ -145,6 +153,7 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
     max_len = prompt + new_tokens
     cache = model.new_cache(batch, max_len)
 
+    model(ids, cache, 0)  # untimed first pass: code objects, library handles and workspaces come into being here
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     logits = model(ids, cache, 0)
@@ -205,7 +214,8 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
         "batch": batch, "prompt": prompt, "new_tokens": new_tokens, "layers": layers,
         "launch": "hip-graph replay" if graph is not None else "eager",
         "fused": "bias+relu+residual in the GEMM store" + ("; q/k/v one launch" if fuse_qkv else "") +
-                 "; decode attention appends K/V in the same launch; one-launch LayerNorm",
+                 "; both LayerNorms inside the q/k/v and fc1 kernels at decode; decode attention appends K/V in the same "
+                 "launch",
         "prefill_ms": round(prefill_s * 1e3, 2),
         "prefill_tok_per_s": round(batch * prompt / prefill_s, 1),
         "decode_ms_per_step": round(decode_s * 1e3 / steps, 4),

@@ -49,10 +49,12 @@ class WALinear(nn.Module):
             self.register_buffer("bias", None)
 
     @torch.no_grad()
-    def forward(self, x, residual=None, act="none"):
+    def forward(self, x, residual=None, act="none", pre_ln=None):
         """y = act(x W_hat^T + bias) + residual.  With the defaults this is the reference's
         forward (gemm_awq_ut, then + bias); bias, activation and residual all ride in the
-        kernel's store instead of separate element-wise launches."""
+        kernel's store instead of separate element-wise launches.  pre_ln: an nn.LayerNorm (or
+        any object with weight, bias, eps) applied to x first, inside the same kernel where the
+        shape allows (up to 8 tokens, group size 128, 2048 < K <= 4096)."""
         weight = self.weight
         if self.w_bit == 2:
             if self.layout != "l1":
@@ -63,8 +65,14 @@ class WALinear(nn.Module):
         res3 = None
         if residual is not None:
             res3 = residual.reshape(x3.shape[0], x3.shape[1], self.out_features).contiguous()
-        y = quant.gemm_awq_fused_ut(x3.contiguous(), weight, self.zeros_scales, self.bias, res3, act,
-                                    self.out_features, self.group_size)
+        if pre_ln is not None:
+            if self.layout != "l1":
+                raise NotImplementedError("pre_ln is supported in layout 'l1' only")
+            y = quant.gemm_awq_ln_fused_ut(x3.contiguous(), pre_ln.weight, pre_ln.bias, pre_ln.eps, weight,
+                                           self.zeros_scales, self.bias, res3, act, self.out_features, self.group_size)
+        else:
+            y = quant.gemm_awq_fused_ut(x3.contiguous(), weight, self.zeros_scales, self.bias, res3, act,
+                                        self.out_features, self.group_size)
         return y.reshape(*lead, self.out_features)
 
     @staticmethod

@@ -69,7 +69,7 @@ def test_independent_linears_of_mixed_shapes(capi, m):
     torch.cuda.synchronize()
     for y, ref, sh in zip(ys, refs, shapes):
         assert rel_err(y.float().cpu().numpy(), ref) <= TOL, sh
-    assert seq.error_flag() == 0 and torch.count_nonzero(seq.ws).item() == 0
+    assert seq.error_flag() == 0 and capi.workspace_is_clean(seq.ws)  # counters; partial tiles may stay
     first = [y.clone() for y in ys]
     seq.run()
     torch.cuda.synchronize()
@@ -113,7 +113,7 @@ def test_dependent_chain_with_epilogues(capi, m, mode):
         assert rel_err(y[1].float().cpu().numpy(), r1.astype(np.float64)) <= TOL
         assert rel_err(y[2].float().cpu().numpy(), r2.astype(np.float64)) <= TOL
         assert rel_err(y[3].float().cpu().numpy(), r3) <= TOL
-    assert seq.error_flag() == 0 and torch.count_nonzero(seq.ws).item() == 0
+    assert seq.error_flag() == 0 and capi.workspace_is_clean(seq.ws)  # counters; partial tiles may stay
     # the same chain with one launch per linear (no workspace: the fallback inside the entry point)
     y2 = [torch.empty_like(t) for t in y]
     lin2 = [dict(l) for l in lin]
@@ -181,7 +181,7 @@ def test_opt67_layer_linears_in_one_launch(capi, m, mode):
         torch.cuda.synchronize()
         for y, f in zip(ys, first):
             assert torch.equal(y, f)
-    assert seq.error_flag() == 0 and torch.count_nonzero(seq.ws).item() == 0
+    assert seq.error_flag() == 0 and capi.workspace_is_clean(seq.ws)  # counters; partial tiles may stay
 
 
 @pytest.mark.parametrize("m", [5, 8, 16, 32])
