@@ -64,7 +64,7 @@ size_t skinny2_workspace_bytes(int M, int N, int K);
 hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                                 int g, int tune, Epilogue epi, hipStream_t st);
 // sq_skinny3.hip: M <= 16, group size 128, K % 128 == 0: the streaming decode kernel.  ws may be null when
-// K <= 4096 (no K split).  tune = rows per workgroup (1: 16, 4: 64) | ksplit << 4, 0 = heuristic.
+// K <= 4096 (no K split).  tune = rows per workgroup (1: 16, 3: 48, 4: 64) | ksplit << 4, 0 = heuristic.
 // hipErrorInvalidValue when the shape does not fit.
 // ln (may be null): LayerNorm of the activations inside the kernel (2048 < K <= 4096, at most 8 tokens).
 hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,

@@ -147,7 +147,7 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     __builtin_amdgcn_sched_barrier(0);  // nothing that waits for a load moves above the weight requests
     // 3. the wave's weight loads, in units of four (two row tiles x the two 64-byte halves of a 128-byte
     //    line back to back, so that the line is requested from L2 once), DEPTH units ahead of the arithmetic
-    constexpr int RTU = RT >= 2 ? 2 : 1;        // row tiles per unit
+    constexpr int RTU = RT % 2 == 0 ? 2 : 1;    // row tiles per unit
     constexpr int RG = RT / RTU;                // units per chunk pair
     constexpr int HN = CH == 1 ? 1 : 2;         // chunk slots per unit
     constexpr int NU = (CH == 1 ? 1 : CH / 2) * RG;
@@ -462,29 +462,47 @@ struct Sk3Plan {
     int rt, ch, ksplit;
 };
 
-Sk3Plan plan(int blocks64, int K, bool have_ws, int tune) {
+Sk3Plan plan(const int* rows, int count, int K, bool have_ws, int tune) {
     const int groups = K / 128;
     Sk3Plan p{4, 4, (groups + 31) / 32};
-    // Few rows: 16-row workgroups (four times as many) when 64-row ones would leave most CUs idle.
-    if (blocks64 * p.ksplit < 128) p.rt = 1;
-    if (tune & 0xF) p.rt = (tune & 0xF) == 1 ? 1 : 4;
     if ((tune >> 4) & 0xF) p.ksplit = (tune >> 4) & 0xF;
     const int cps = (groups + p.ksplit - 1) / p.ksplit;
     p.ch = cps <= 8 ? 1 : cps <= 16 ? 2 : 4;
-    if (cps > 32 || (p.ksplit > 1 && !have_ws) || p.ksplit > 8 || (p.ksplit - 1) * cps >= groups) p.ksplit = 0;  // does not fit
+    if (cps > 32 || (p.ksplit > 1 && !have_ws) || p.ksplit > 8 || (p.ksplit - 1) * cps >= groups) {
+        p.ksplit = 0;  // does not fit
+        return p;
+    }
+    // Rows per workgroup: 64, 48 or 16, whichever needs the least time by this count: rounds of 256 workgroups
+    // (one per CU) times the row tiles of a workgroup plus two for its activations (at 8 tokens the staged
+    // activations weigh as much as two row tiles of weights).  OPT-6.7B: 4096 rows -> 16 (256 workgroups),
+    // 12288 and 11008 -> 48 (256 and 230), 16384 -> 64 (256).  48-row workgroups only without a K split (their
+    // partial tiles do not fit the workspace layout) and with full-length K ranges.
+    int best = 1 << 30;
+    for (int rt : {4, 3, 1}) {
+        if (rt == 3 && (p.ksplit != 1 || p.ch != 4)) continue;
+        long blocks = 0;
+        for (int l = 0; l < count; l++) blocks += (rows[l] + 16 * rt - 1) / (16 * rt);
+        const long rounds = (blocks * p.ksplit + 255) / 256;
+        const long cost = rounds * (rt + 2);
+        if (cost < best) {
+            best = (int)cost;
+            p.rt = rt;
+        }
+    }
+    if (tune & 0xF) p.rt = (tune & 0xF) == 1 ? 1 : ((tune & 0xF) == 3 && p.ksplit == 1 && p.ch == 4) ? 3 : 4;
     return p;
 }
 
 }  // namespace
 
-// M <= 16, group size 128, K % 128 == 0.  tune = rows per workgroup (1: 16, 4: 64) | ksplit << 4, 0 = heuristic.
+// M <= 16, group size 128, K % 128 == 0.  tune = rows per workgroup (1: 16, 3: 48, 4: 64) | ksplit << 4, 0 = heuristic.
 // ln (may be null): LayerNorm of the activations inside the kernel; possible when a workgroup holds whole rows
 // (2048 < K <= 4096, no K split) of at most 8 tokens.  hipErrorInvalidValue when the shape does not fit (K range per workgroup beyond
 // 4096, a K split without a workspace, or a LayerNorm over rows the workgroup does not hold whole).
 hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                                 int tune, Epilogue epi, const LnPre* ln, hipStream_t st) {
     if (M < 1 || M > 16 || K % 128 != 0) return hipErrorInvalidValue;
-    const Sk3Plan p = plan((N + 63) / 64, K, ws != nullptr, tune);
+    const Sk3Plan p = plan(&N, 1, K, ws != nullptr, tune);
     if (p.ksplit == 0) return hipErrorInvalidValue;
     if (p.ksplit > 1 && (N + 16 * p.rt - 1) / (16 * p.rt) > 16384) return hipErrorInvalidValue;
     if (ln) {
@@ -492,10 +510,12 @@ hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, vo
 #define SQ_SK3_LN(MR, RT) return launch_cfg<MR, RT, 4, true>(x, w, zs, y, ws, M, N, K, 1, epi, *ln, st)
         if (M <= 4) {
             if (p.rt == 1) SQ_SK3_LN(4, 1);
+            if (p.rt == 3) SQ_SK3_LN(4, 3);
             SQ_SK3_LN(4, 4);
         }
         if (M > 8) return hipErrorInvalidValue;  // sixteen rows of statistics per thread do not fit the registers
         if (p.rt == 1) SQ_SK3_LN(8, 1);
+        if (p.rt == 3) SQ_SK3_LN(8, 3);
         SQ_SK3_LN(8, 4);
 #undef SQ_SK3_LN
     }
@@ -509,13 +529,16 @@ hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, vo
     } while (0)
     if (M <= 4) {
         if (p.rt == 1) SQ_SK3_CH(4, 1);
+        if (p.rt == 3) SQ_SK3(4, 3, 4);
         SQ_SK3_CH(4, 4);
     }
     if (M <= 8) {
         if (p.rt == 1) SQ_SK3_CH(8, 1);
+        if (p.rt == 3) SQ_SK3(8, 3, 4);
         SQ_SK3_CH(8, 4);
     }
     if (p.rt == 1) SQ_SK3_CH(16, 1);
+    if (p.rt == 3) SQ_SK3(16, 3, 4);
     SQ_SK3_CH(16, 4);
 #undef SQ_SK3_CH
 #undef SQ_SK3
@@ -526,12 +549,14 @@ hipError_t launch_skinny3_group(const SeqProblem* probs, int count, int M, void*
     if (count < 2 || count > GEMV_GROUP_MAX || M < 1 || M > 16) return hipErrorInvalidValue;
     const int K = probs[0].K;
     if (K % 128 != 0) return hipErrorInvalidValue;
+    int rows[GEMV_GROUP_MAX];
     int blocks64 = 0;
     for (int p = 0; p < count; p++) {
         if (probs[p].K != K || probs[p].group_size != 128) return hipErrorInvalidValue;
+        rows[p] = probs[p].N;
         blocks64 += (probs[p].N + 63) / 64;
     }
-    const Sk3Plan pl = plan(blocks64, K, ws != nullptr, 0);
+    const Sk3Plan pl = plan(rows, count, K, ws != nullptr, 0);
     if (pl.ksplit == 0) return hipErrorInvalidValue;
     if (pl.ksplit > 1 && (blocks64 * (4 / pl.rt) > 16384 || ws_bytes < skinny2_group_workspace_bytes(probs, count, M)))
         return hipErrorInvalidValue;
@@ -544,13 +569,16 @@ hipError_t launch_skinny3_group(const SeqProblem* probs, int count, int M, void*
     } while (0)
     if (M <= 4) {
         if (pl.rt == 1) SQ_SK3_CH(4, 1);
+        if (pl.rt == 3) SQ_SK3(4, 3, 4);
         SQ_SK3_CH(4, 4);
     }
     if (M <= 8) {
         if (pl.rt == 1) SQ_SK3_CH(8, 1);
+        if (pl.rt == 3) SQ_SK3(8, 3, 4);
         SQ_SK3_CH(8, 4);
     }
     if (pl.rt == 1) SQ_SK3_CH(16, 1);
+    if (pl.rt == 3) SQ_SK3(16, 3, 4);
     SQ_SK3_CH(16, 4);
 #undef SQ_SK3_CH
 #undef SQ_SK3

@@ -46,18 +46,20 @@ def linear(n, k, seed=0):
 
 
 def tunings(k):
-    """0 = heuristic; rows per workgroup (1: 16, 4: 64) | ksplit << 4 for every split whose K range fits."""
+    """0 = heuristic; rows per workgroup (1: 16, 3: 48, 4: 64) | ksplit << 4 for every split whose K range fits."""
     chunks = k // 128
     out = [0]
-    for rt in (1, 4):
+    for rt in (1, 3, 4):
         for ks in (1, 2, 3, 4, 8):
             cps = -(-chunks // ks)
+            if rt == 3 and (ks != 1 or cps <= 16):
+                continue  # 48-row workgroups: full-length K ranges without a split only
             if cps <= 32 and (ks - 1) * cps < chunks:
                 out.append(rt | (ks << 4))
     return out
 
 
-SHAPES = [(256, 1024), (264, 2048), (200, 1536), (520, 4096), (72, 4224), (1000, 5120), (264, 11008), (136, 16384)]
+SHAPES = [(256, 1024), (264, 2048), (200, 1536), (520, 4096), (1048, 3200), (72, 4224), (1000, 5120), (264, 11008), (136, 16384)]
 
 
 @pytest.mark.parametrize("n,k", SHAPES)
