@@ -28,7 +28,7 @@ namespace sq {
 namespace {
 
 constexpr int DA_WAVES = 8;
-constexpr int DA_U = 4;  // 128-bit loads in flight per wave
+constexpr int DA_U = 4;  // rows of a batch per row slot: 128-bit loads per wave and operand in one request (6 and 8: no faster)
 
 struct DecodeAttnArgs {
     const half_t* q;
@@ -54,7 +54,7 @@ struct DecodeAttnArgs {
 
 __device__ __forceinline__ float xor_sum(float v, int m) { return v + __shfl_xor(v, m, 64); }
 
-template <int D>
+template <int D, bool MASK>
 __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnArgs a) {
     constexpr int LPR = D / 8;    // lanes per cache row
     constexpr int RPI = 64 / LPR; // rows per load instruction
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: the stream's loop is then uniform control flow
     const int c = lane % LPR;
     const int r = lane / LPR;
     const int b = blockIdx.x / a.H;
@@ -101,12 +101,12 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
             dst[u] = *(const u32x4_t*)src;
         }
     };
-    auto store_fresh = [&](half_t* cache, int base, const u32x4_t (&src)[DA_U]) {
-        if (!append) return;
-#pragma unroll
-        for (int u = 0; u < DA_U; u++)
-            if (base + u * RPI + r == n0 && n0 < r1) *(u32x4_t*)(cache + (long)n0 * D) = src[u];
-    };
+    // The appended row goes into the cache once, up front, by the lanes of the workgroup whose share holds it
+    // (the stream below takes it from the new-row pointers and never reads it back).
+    if (append && n0 >= r0 && n0 < r1 && wave == 0 && r == 0) {
+        *(u32x4_t*)(kbase + (long)n0 * D) = *(const u32x4_t*)knrow;
+        *(u32x4_t*)(vbase + (long)n0 * D) = *(const u32x4_t*)vnrow;
+    }
 
     // Online softmax state of this lane's row slot (the LPR lanes of a slot hold the same m and l).
     float m = -INFINITY, l = 0.f;
@@ -114,20 +114,24 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = 0.f;
 
-    u32x4_t kcur[DA_U], vcur[DA_U], knxt[DA_U], vnxt[DA_U];
-    int base = r0 + wave * RPI * DA_U;
-    if (base < r1) {
-        load_rows(kbase, knrow, base, kcur);
-        load_rows(vbase, vnrow, base, vcur);
-    }
-    for (; base < r1; base += STEP) {
-        const bool more = base + STEP < r1;
-        if (more) {
-            load_rows(kbase, knrow, base + STEP, knxt);
-            load_rows(vbase, vnrow, base + STEP, vnxt);
-        }
-        store_fresh(kbase, base, kcur);
-        store_fresh(vbase, base, vcur);
+    // The stream.  No branch and no store inside the loop: the next batch of rows is always requested (row
+    // indices clamped to the share, so a batch past the end re-reads the last row and gets probability zero),
+    // which keeps the compiler's wait counts exact: the arithmetic of a batch waits for that batch only while
+    // the next one is in flight.
+    u32x4_t ka[DA_U], va[DA_U], kb[DA_U], vb[DA_U];
+    float ma[DA_U], mb_[DA_U];
+    auto load_mask = [&](int base, float (&dst)[DA_U]) {
+#pragma unroll
+        for (int u = 0; u < DA_U; u++) dst[u] = MASK ? (float)mrow[imin(base + u * RPI + r, r1 - 1)] : 0.f;
+    };
+    auto request = [&](int base, u32x4_t (&kd)[DA_U], u32x4_t (&vd)[DA_U], float (&md)[DA_U]) {
+        __builtin_amdgcn_sched_barrier(0);
+        load_rows(kbase, knrow, base, kd);
+        load_rows(vbase, vnrow, base, vd);
+        load_mask(base, md);
+        __builtin_amdgcn_sched_barrier(0);  // the requests go out here, ahead of the arithmetic that follows
+    };
+    auto consume = [&](int base, const u32x4_t (&kcur)[DA_U], const u32x4_t (&vcur)[DA_U], const float (&mcur)[DA_U]) {
         float sc[DA_U];
         float mx = m;
 #pragma unroll
@@ -141,8 +145,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
             s = xor_sum(s, 4);
             if (LPR == 16) s = xor_sum(s, 8);
             const int j = base + u * RPI + r;
-            s *= a.scale;
-            if (mrow && j < r1) s += (float)mrow[j];
+            s = s * a.scale + mcur[u];
             sc[u] = j < r1 ? s : -INFINITY;
             mx = fmaxf(mx, sc[u]);
         }
@@ -160,13 +163,19 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
             for (int i = 0; i < 8; i++) acc[i] += p * (float)vv[i];
         }
         m = mx;
-        if (more) {
-#pragma unroll
-            for (int u = 0; u < DA_U; u++) {
-                kcur[u] = knxt[u];
-                vcur[u] = vnxt[u];
-            }
-        }
+    };
+    // Two register sets take turns (a loop that copied "next" into "current" would have to wait for the
+    // requests it has just made); two batches per trip, one past the end of the share is all probability zero.
+    int base = r0 + wave * RPI * DA_U;
+    if (base < r1) {
+        request(base, ka, va, ma);
+        do {
+            request(base + STEP, kb, vb, mb_);
+            consume(base, ka, va, ma);
+            request(base + 2 * STEP, ka, va, ma);
+            consume(base + STEP, kb, vb, mb_);
+            base += 2 * STEP;
+        } while (base < r1);
     }
 
     // Merge the row slots of a wave (lanes with equal c), then the waves.
@@ -243,7 +252,10 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
 
 template <int D>
 hipError_t launch_d(const DecodeAttnArgs& a, int B, int nsplit, hipStream_t st) {
-    hipLaunchKernelGGL((decode_attn_kernel<D>), dim3(B * a.H, nsplit), dim3(64 * DA_WAVES), 0, st, a);
+    if (a.mask)
+        hipLaunchKernelGGL((decode_attn_kernel<D, true>), dim3(B * a.H, nsplit), dim3(64 * DA_WAVES), 0, st, a);
+    else
+        hipLaunchKernelGGL((decode_attn_kernel<D, false>), dim3(B * a.H, nsplit), dim3(64 * DA_WAVES), 0, st, a);
     return hipGetLastError();
 }
 
