@@ -82,10 +82,12 @@ int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y,
  * least sq_w4a16_workspace_bytes(M, N, K) bytes, be 16-byte aligned, and have its
  * first 64 KiB zeroed before the first call (every call leaves them zero); calls that
  * share a workspace must not overlap in time.  With SQ_ALGO_AUTO the split is taken
- * where it is the fastest: the split-K decode kernel for 5..32 tokens on weights of
- * 2^25 elements or more or with K > 8192 and for 17..32 tokens on any weight, the same
- * kernel in two blocks for 33..48 tokens on such weights, and a K split of the tiled
- * GEMM for larger M whose grid would leave most CUs idle.  A workspace that is NULL, misaligned or too small is ignored under
+ * where it is the fastest: the streaming decode kernel for 3..16 tokens at group size
+ * 128 when K exceeds 4096 (a shorter K needs no split and no workspace), the split-K
+ * decode kernel for 5..32 tokens otherwise on weights of 2^25 elements or more or with
+ * K > 8192 and for 17..32 tokens on any weight, the same kernel in two blocks for 33..48
+ * tokens on such weights, and a K split of the tiled GEMM for larger M whose grid would
+ * leave most CUs idle.  A workspace that is NULL, misaligned or too small is ignored under
  * SQ_ALGO_AUTO (the workspace-free kernels run); an explicit SQ_ALGO_SKINNY_WS then
  * returns SQ_ERR_WORKSPACE. */
 int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y,
@@ -173,8 +175,8 @@ int sq_w4a16_gemm_fused(const void* x, const void* w, const void* zs, const void
  *            depends on anything, kept for that case and for measurement.
  *   workspace  NULL, or sq_w4a16_gemv_sequence_workspace_bytes(linears, count, M) bytes, 16-byte
  *            aligned, its first 64 KiB zero before the first call (every call leaves them zero);
- *            calls that share it must be ordered.  Up to 4 tokens it is used by
- *            SQ_SEQ_ONE_LAUNCH only (256 bytes); with 5..32 tokens it is the split-K workspace of
+ *            calls that share it must be ordered.  With 1 or 2 tokens it is used by
+ *            SQ_SEQ_ONE_LAUNCH only (256 bytes); with 3..32 tokens it is the split-K workspace of
  *            sq_w4a16_gemm_ws, sized for the linears that may share a launch.
  *            Word 9 of it is a sticky error flag: it becomes 1 if a grid barrier ever ran out of
  *            polls (results of that call are then undefined).
