@@ -103,7 +103,8 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
         // one launch 8.6 against 12.1, fc2 12.7 against 14.6; against the GEMV on 4096 x 4096: 4.9 against 6.5.
         // With 3 or 4 tokens it also beats the GEMV on fc1 / fc2-class weights (9.7 against 10.7 us, 11.9 against
         // 13.6 us at 4 tokens); on 4096 x 4096 and with 1 or 2 tokens the GEMV stays ahead.
-        const bool stream_ok = (M > 4 || (M >= 3 && large)) && M <= 16 && group_size == 128 && K % 128 == 0 &&
+        const bool stream_ok = (M > 4 || (M >= 3 && large)) && M <= 16 && (group_size == 128 || group_size == 64) &&
+                               K % 128 == 0 &&
                                (K <= 4096 || (ws_ok && K <= 32768));
         if (stream_ok) {
             kernel = SQ_ALGO_STREAM;
@@ -150,10 +151,11 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
                 return SQ_ERR_WORKSPACE;
             return launch_code(sq::launch_skinny2_tuned(x, w, zs, y, workspace, M, N, K, group_size, tune, epi, st));
         case SQ_ALGO_STREAM: {
-            if (M > 16 || group_size != 128) return SQ_ERR_BAD_ALGO;
+            if (M > 16 || (group_size != 128 && group_size != 64)) return SQ_ERR_BAD_ALGO;
             const bool ws_fits = workspace && aligned16(workspace) &&
                                  workspace_bytes >= sq::skinny2_workspace_bytes(M, N, K);
-            const hipError_t e = sq::launch_skinny3_tuned(x, w, zs, y, ws_fits ? workspace : nullptr, M, N, K, tune, epi, nullptr, st);
+            const hipError_t e =
+                sq::launch_skinny3_tuned(x, w, zs, y, ws_fits ? workspace : nullptr, M, N, K, group_size, tune, epi, nullptr, st);
             return e == hipErrorInvalidValue ? SQ_ERR_WORKSPACE : launch_code(e);
         }
         case SQ_ALGO_GEMM:
@@ -499,7 +501,7 @@ int sq_w4a16_gemm_ln_fused(const void* x, const void* ln_gamma, const void* ln_b
         if (!x || !w || !zs || !y) return SQ_ERR_NULL_POINTER;
         if (!aligned16(x) || !aligned16(w) || !aligned16(zs) || !aligned16(y)) return SQ_ERR_MISALIGNED;
         const sq::LnPre ln{static_cast<const sq::half_t*>(ln_gamma), static_cast<const sq::half_t*>(ln_beta), ln_eps};
-        const hipError_t e = sq::launch_skinny3_tuned(x, w, zs, y, nullptr, M, N, K, 0, epi, &ln,
+        const hipError_t e = sq::launch_skinny3_tuned(x, w, zs, y, nullptr, M, N, K, group_size, 0, epi, &ln,
                                                       static_cast<hipStream_t>(stream));
         if (e != hipErrorInvalidValue) return launch_code(e);
     }

@@ -63,12 +63,12 @@ hipError_t launch_skinny_tuned(const void* x, const void* w, const void* zs, voi
 size_t skinny2_workspace_bytes(int M, int N, int K);
 hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                                 int g, int tune, Epilogue epi, hipStream_t st);
-// sq_skinny3.hip: M <= 16, group size 128, K % 128 == 0: the streaming decode kernel.  ws may be null when
+// sq_skinny3.hip: M <= 16, group size 128 or 64, K % 128 == 0: the streaming decode kernel.  ws may be null when
 // K <= 4096 (no K split).  tune = rows per workgroup (1: 16, 3: 48, 4: 64) | ksplit << 4, 0 = heuristic.
 // hipErrorInvalidValue when the shape does not fit.
 // ln (may be null): LayerNorm of the activations inside the kernel (2048 < K <= 4096, at most 8 tokens).
 hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
-                                int tune, Epilogue epi, const LnPre* ln, hipStream_t st);
+                                int g, int tune, Epilogue epi, const LnPre* ln, hipStream_t st);
 hipError_t launch_skinny3_group(const SeqProblem* probs, int count, int M, void* ws, size_t ws_bytes, hipStream_t st);
 // sq_gemm.hip: any M.  tune = 32-row tiles per workgroup (1,2,4) | ksplit << 8; ws may be null.
 size_t gemm_workspace_bytes(int M, int N, int K);

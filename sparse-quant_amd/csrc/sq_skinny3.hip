@@ -40,7 +40,6 @@ namespace {
 constexpr int SK3_COUNTER_BYTES = 65536;  // start of the workspace: one uint32 per row block
 constexpr int SK3_NWV = 8;
 constexpr int SK3_NT = 64 * SK3_NWV;
-constexpr int SK3_ZPITCH = 33;
 #ifndef SQ_SK3_DEPTH
 #define SQ_SK3_DEPTH 1
 #endif
@@ -50,15 +49,16 @@ constexpr int SK3_ZPITCH = 33;
 constexpr int SK3_DEPTH_PRE = SQ_SK3_DEPTH_PRE;  // units requested before the activations are parked
 constexpr int SK3_DEPTH = SQ_SK3_DEPTH;  // units of four weight loads requested ahead of the one being consumed
 
-template <int MROWS, int RT, int CH>
+template <int MROWS, int RT, int CH, int GPC = 1>
 struct Sk3Lds {
+    static constexpr int ZPITCH = 32 * GPC + 1;          // (zero, scale) pairs per staged row: GPC per chunk slot
     static constexpr int CHUNKS = SK3_NWV * CH;          // chunk slots of a workgroup
     static constexpr int XPITCH = CHUNKS * 256 + 16;     // bytes per staged token row
     static constexpr int X_BYTES = MROWS * XPITCH;
     static constexpr int TILE = RT * 4 * 64;             // floats a wave contributes: [rt][v][lane]
     static constexpr int RED_BYTES = SK3_NWV * TILE * 4;
     static constexpr int Z_OFF = X_BYTES > RED_BYTES ? X_BYTES : RED_BYTES;  // the partials reuse the activations' space
-    static constexpr int FLAG_OFF = Z_OFF + 16 * RT * SK3_ZPITCH * 4;
+    static constexpr int FLAG_OFF = Z_OFF + 16 * RT * ZPITCH * 4;
     static constexpr int LN_OFF = FLAG_OFF + 16;         // fused LayerNorm: mean and reciprocal deviation per token
     static constexpr int BYTES = LN_OFF + 2 * MROWS * 4;
 };
@@ -67,17 +67,20 @@ __device__ __forceinline__ void sk3_barrier() { asm volatile("s_waitcnt lgkmcnt(
 
 // rb = row block inside this linear; slot = index of the row block in the workspace, which differs from
 // rb when several linears share a launch.
-template <int MROWS, int RT, int CH, int DEPTH, bool LN>
+// GPC = groups per 128-wide chunk: 1 (group size 128: zero and scale applied per chunk in fp32) or 2 (group size 64:
+// per-weight dequantisation in fp16, as the reference computes W_hat).
+template <int MROWS, int RT, int CH, int DEPTH, bool LN, int GPC>
 __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ZS,
                                              const half_t* __restrict__ X, half_t* __restrict__ Y, float* part,
                                              unsigned* counters, int M, int N, int K, int ksplit, const Epilogue& epi,
                                              const LnPre& ln, int rb, int slot, int nslots) {
-    using L = Sk3Lds<MROWS, RT, CH>;
+    using L = Sk3Lds<MROWS, RT, CH, GPC>;
     constexpr int ROWS = 16 * RT;
+    constexpr int ZW = 32 * GPC;  // staged (zero, scale) pairs per row
     constexpr int TILE = L::TILE;
     constexpr int WPR = L::CHUNKS * 16;  // 128-bit words per staged token row
     constexpr int XPT = MROWS * WPR / SK3_NT;
-    constexpr int ZPT = (ROWS * 32 + SK3_NT - 1) / SK3_NT;
+    constexpr int ZPT = (ROWS * ZW + SK3_NT - 1) / SK3_NT;
     static_assert(CH == 1 || CH == 2 || CH == 4, "chunk slots per wave");
     static_assert(MROWS * WPR % SK3_NT == 0, "activation words divide over the threads");
     static_assert(!LN || WPR == SK3_NT, "fused LayerNorm: thread t holds columns 8t .. 8t+7 of every token");
@@ -95,10 +98,11 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     const int li = lane & 15;
     const int lj = lane >> 4;
     const int ks = blockIdx.y;
-    const int groups = K >> 7;  // group size 128: one (z, s) pair per chunk
-    const int cps = (groups + ksplit - 1) / ksplit;
+    const int chunks = K >> 7;
+    const int groups = chunks * GPC;  // (z, s) pairs per row
+    const int cps = (chunks + ksplit - 1) / ksplit;
     int c_begin = ks * cps;
-    int nc = imin(c_begin + cps, groups) - c_begin;
+    int nc = imin(c_begin + cps, chunks) - c_begin;
     if (nc <= 0) {  // an empty K range (the host does not create one) streams chunk 0 against zeros
         nc = 0;
         c_begin = 0;
@@ -109,9 +113,9 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
 #pragma unroll
     for (int p = 0; p < ZPT; p++) {
         const int idx = tid + p * SK3_NT;
-        const int r = (idx >> 5) % ROWS, col = idx & 31;
+        const int r = (idx / ZW) % ROWS, col = idx % ZW;
         const int row = imin(rb * ROWS + r, N - 1);
-        zreg[p] = ZS[(long)row * groups + c_begin + (col < nc ? col : 0)];
+        zreg[p] = ZS[(long)row * groups + c_begin * GPC + (col < nc * GPC ? col : 0)];
     }
     // 2. every activation of the K range (tokens beyond M and chunk slots beyond the range: zeros)
     u32x4_t xr[XPT];
@@ -241,7 +245,7 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
 #pragma unroll
     for (int p = 0; p < ZPT; p++) {
         const int idx = tid + p * SK3_NT;
-        if (idx < ROWS * 32) zsl[(idx >> 5) * SK3_ZPITCH + (idx & 31)] = zreg[p];
+        if (idx < ROWS * ZW) zsl[(idx / ZW) * L::ZPITCH + idx % ZW] = zreg[p];
     }
 #pragma unroll
     for (int p = 0; p < XPT; p++) {
@@ -279,29 +283,45 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
             half8_t xa[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) xa[t] = *(const half8_t*)(xrd + cl * 256 + 16 * t);
-            if (rg == 0) {
-                xsum[u] = (float4_t){0.f, 0.f, 0.f, 0.f};
-                x960[u] = (float4_t){0.f, 0.f, 0.f, 0.f};
+            if (GPC == 1) {
+                if (rg == 0) {
+                    xsum[u] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                    x960[u] = (float4_t){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    xsum[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t], ones, xsum[u], 0, 0, 0);
-                    x960[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t], m960, x960[u], 0, 0, 0);
+                    for (int t = 0; t < 4; t++) {
+                        xsum[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t], ones, xsum[u], 0, 0, 0);
+                        x960[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t], m960, x960[u], 0, 0, 0);
+                    }
                 }
-            }
 #pragma unroll
-            for (int r = 0; r < RTU; r++) {
-                const int rt = RTU * rg + r;
-                const half2_t zsv = bit_cast<half2_t>(zsl[(16 * rt + li) * SK3_ZPITCH + zcol]);
-                // shift-free unpack (1024 + q on four of every eight positions); the accumulator starts at
-                // -960 * (sum of x over those positions), which takes the extra bias out again
-                float4_t tmp = x960[u];
+                for (int r = 0; r < RTU; r++) {
+                    const int rt = RTU * rg + r;
+                    const half2_t zsv = bit_cast<half2_t>(zsl[(16 * rt + li) * L::ZPITCH + zcol]);
+                    // shift-free unpack (1024 + q on four of every eight positions); the accumulator starts at
+                    // -960 * (sum of x over those positions), which takes the extra bias out again
+                    float4_t tmp = x960[u];
 #pragma unroll
-                for (int t = 0; t < 4; t++)
-                    tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t], unpack8_mixed(wq[u][rt][t], nm), tmp, 0, 0, 0);
-                const float zf = (float)zsv.x;
-                const float sf = (float)zsv.y;
+                    for (int t = 0; t < 4; t++)
+                        tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t], unpack8_mixed(wq[u][rt][t], nm), tmp, 0, 0, 0);
+                    const float zf = (float)zsv.x;
+                    const float sf = (float)zsv.y;
 #pragma unroll
-                for (int v = 0; v < 4; v++) acc[rt][v] += sf * (tmp[v] - zf * xsum[u][v]);
+                    for (int v = 0; v < 4; v++) acc[rt][v] += sf * (tmp[v] - zf * xsum[u][v]);
+                }
+            } else {
+                // Group size 64: a matrix instruction spans both groups of the chunk (lanes lj = 0, 1 hold the
+                // first 64 columns, lj = 2, 3 the second), so zero and scale cannot be applied to its result;
+                // each lane dequantises its own weights instead (its row and its group are its own), bit-identical
+                // to the reference's fp16 (q - z) * s.
+#pragma unroll
+                for (int r = 0; r < RTU; r++) {
+                    const int rt = RTU * rg + r;
+                    const half2_t zsv = bit_cast<half2_t>(zsl[(16 * rt + li) * L::ZPITCH + zcol * GPC + (lj >> 1)]);
+                    const half2_t z64 = {zsv.x, zsv.x}, sc = {zsv.y, zsv.y};
+#pragma unroll
+                    for (int t = 0; t < 4; t++)
+                        acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[t], dequant8(wq[u][rt][t], z64, sc, nm), acc[rt], 0, 0, 0);
+                }
             }
         }
     }
@@ -367,12 +387,12 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     if (tid == 0) __hip_atomic_store(&counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int MROWS, int RT, int CH, bool LN>
+template <int MROWS, int RT, int CH, bool LN, int GPC>
 __global__ __launch_bounds__(SK3_NT) void skinny3_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ZS,
                                                          const half_t* __restrict__ X, half_t* __restrict__ Y,
                                                          float* part, unsigned* counters, int M, int N, int K,
                                                          int ksplit, Epilogue epi, LnPre ln) {
-    skinny3_body<MROWS, RT, CH, SK3_DEPTH, LN>(W, ZS, X, Y, part, counters, M, N, K, ksplit, epi, ln, blockIdx.x, blockIdx.x,
+    skinny3_body<MROWS, RT, CH, SK3_DEPTH, LN, GPC>(W, ZS, X, Y, part, counters, M, N, K, ksplit, epi, ln, blockIdx.x, blockIdx.x,
                                                gridDim.x);
 }
 
@@ -398,7 +418,7 @@ __global__ __launch_bounds__(SK3_NT) void skinny3_group_kernel(const Skinny3Grou
         if (q + 1 < grp.count && (int)blockIdx.x >= grp.blk_end[q]) p = q + 1;
     const int rb = blockIdx.x - (p > 0 ? grp.blk_end[p - 1] : 0);
     const Epilogue epi{grp.bias[p], grp.residual[p], grp.act[p]};
-    skinny3_body<MROWS, RT, CH, SK3_DEPTH, false>(grp.W[p], grp.ZS[p], grp.X[p], grp.Y[p], part, counters, M, grp.N[p], K,
+    skinny3_body<MROWS, RT, CH, SK3_DEPTH, false, 1>(grp.W[p], grp.ZS[p], grp.X[p], grp.Y[p], part, counters, M, grp.N[p], K,
                                                   ksplit, epi, LnPre{nullptr, nullptr, 0.f}, rb, blockIdx.x, gridDim.x);
 }
 
@@ -415,15 +435,15 @@ hipError_t allow_lds(Kern kern, int bytes, bool* done) {
     return hipSuccess;
 }
 
-template <int MROWS, int RT, int CH, bool LN>
+template <int MROWS, int RT, int CH, bool LN, int GPC = 1>
 hipError_t launch_cfg(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K, int ksplit,
                       Epilogue epi, LnPre ln, hipStream_t st) {
     static bool allowed[64];
-    constexpr int lds = Sk3Lds<MROWS, RT, CH>::BYTES;
-    const hipError_t e = allow_lds(skinny3_kernel<MROWS, RT, CH, LN>, lds, allowed);
+    constexpr int lds = Sk3Lds<MROWS, RT, CH, GPC>::BYTES;
+    const hipError_t e = allow_lds(skinny3_kernel<MROWS, RT, CH, LN, GPC>, lds, allowed);
     if (e != hipSuccess) return e;
     const dim3 grid((N + 16 * RT - 1) / (16 * RT), ksplit);
-    hipLaunchKernelGGL((skinny3_kernel<MROWS, RT, CH, LN>), grid, dim3(SK3_NT), lds, st, (const uint8_t*)w,
+    hipLaunchKernelGGL((skinny3_kernel<MROWS, RT, CH, LN, GPC>), grid, dim3(SK3_NT), lds, st, (const uint8_t*)w,
                        (const uint32_t*)zs, (const half_t*)x, (half_t*)y,
                        ws ? (float*)((char*)ws + SK3_COUNTER_BYTES) : nullptr, (unsigned*)ws, M, N, K, ksplit, epi, ln);
     return hipGetLastError();
@@ -495,16 +515,34 @@ Sk3Plan plan(const int* rows, int count, int K, bool have_ws, int tune) {
 
 }  // namespace
 
-// M <= 16, group size 128, K % 128 == 0.  tune = rows per workgroup (1: 16, 3: 48, 4: 64) | ksplit << 4, 0 = heuristic.
+// M <= 16, group size 128 or 64, K % 128 == 0.  tune = rows per workgroup (1: 16, 3: 48, 4: 64) | ksplit << 4, 0 = heuristic.
 // ln (may be null): LayerNorm of the activations inside the kernel; possible when a workgroup holds whole rows
 // (2048 < K <= 4096, no K split) of at most 8 tokens.  hipErrorInvalidValue when the shape does not fit (K range per workgroup beyond
 // 4096, a K split without a workspace, or a LayerNorm over rows the workgroup does not hold whole).
 hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
-                                int tune, Epilogue epi, const LnPre* ln, hipStream_t st) {
-    if (M < 1 || M > 16 || K % 128 != 0) return hipErrorInvalidValue;
-    const Sk3Plan p = plan(&N, 1, K, ws != nullptr, tune);
+                                int g, int tune, Epilogue epi, const LnPre* ln, hipStream_t st) {
+    if (M < 1 || M > 16 || K % 128 != 0 || (g != 128 && g != 64)) return hipErrorInvalidValue;
+    Sk3Plan p = plan(&N, 1, K, ws != nullptr, tune);
     if (p.ksplit == 0) return hipErrorInvalidValue;
+    if (g == 64 && p.rt == 3) p.rt = 4;  // group size 64: 16- and 64-row workgroups only
     if (p.ksplit > 1 && (N + 16 * p.rt - 1) / (16 * p.rt) > 16384) return hipErrorInvalidValue;
+    const LnPre none{nullptr, nullptr, 0.f};
+    if (g == 64) {
+        if (ln) return hipErrorInvalidValue;
+#define SQ_SK3_G64(MR, RT)                                                                                   \
+    do {                                                                                                     \
+        if (p.ch == 1) return launch_cfg<MR, RT, 1, false, 2>(x, w, zs, y, ws, M, N, K, p.ksplit, epi, none, st); \
+        if (p.ch == 2) return launch_cfg<MR, RT, 2, false, 2>(x, w, zs, y, ws, M, N, K, p.ksplit, epi, none, st); \
+        return launch_cfg<MR, RT, 4, false, 2>(x, w, zs, y, ws, M, N, K, p.ksplit, epi, none, st);                \
+    } while (0)
+        if (M <= 8) {
+            if (p.rt == 1) SQ_SK3_G64(8, 1);
+            SQ_SK3_G64(8, 4);
+        }
+        if (p.rt == 1) SQ_SK3_G64(16, 1);
+        SQ_SK3_G64(16, 4);
+#undef SQ_SK3_G64
+    }
     if (ln) {
         if (p.ksplit != 1 || p.ch != 4) return hipErrorInvalidValue;
 #define SQ_SK3_LN(MR, RT) return launch_cfg<MR, RT, 4, true>(x, w, zs, y, ws, M, N, K, 1, epi, *ln, st)
@@ -519,7 +557,6 @@ hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, vo
         SQ_SK3_LN(8, 4);
 #undef SQ_SK3_LN
     }
-    const LnPre none{nullptr, nullptr, 0.f};
 #define SQ_SK3(MR, RT, CH) return launch_cfg<MR, RT, CH, false>(x, w, zs, y, ws, M, N, K, p.ksplit, epi, none, st)
 #define SQ_SK3_CH(MR, RT)            \
     do {                             \

@@ -1,4 +1,4 @@
-"""GPU parity of the streaming decode kernel (SQ_ALGO_STREAM: up to 16 tokens, group size 128) against the
+"""GPU parity of the streaming decode kernel (SQ_ALGO_STREAM: up to 16 tokens, group size 128 or 64) against the
 CPU oracle, through the C ABI: every workgroup shape and K split it can be launched with, ragged row counts,
 K ranges that do not fill a workgroup's chunk slots, the fused epilogue, the grouped launch behind
 sq_w4a16_gemv_sequence, and the properties that do not depend on the size (determinism, exact doubling,
@@ -93,13 +93,40 @@ def test_stream_without_workspace_up_to_4096_columns(capi):
         capi.gemm(to_dev(orc.synth_x(8, 8192, seed=46)), d2["w_dev"], d2["zs_dev"], n, 8192, G, algo=capi.SQ_ALGO_STREAM)
 
 
+@pytest.mark.parametrize("n,k", [(256, 1024), (200, 1536), (520, 4096), (4096, 4096), (264, 8192)])
+@pytest.mark.parametrize("m", [3, 5, 8, 13, 16])
+def test_stream_group_size_64(capi, n, k, m):
+    """Group size 64 (two (zero, scale) pairs per 128-wide chunk): explicit kernel id with 16- and 64-row
+    workgroups and K splits, and the automatic dispatch, against the oracle."""
+    dd = orc.synth_linear(n, k, 64, seed=90)
+    w_hat = orc.dequant_l1(dd["w_l1"], dd["zs_l1"], 64)
+    wd, zd = to_dev(dd["w_l1"]), to_dev(dd["zs_l1"])
+    x = orc.synth_x(m, k, seed=91 + m)
+    rows = np.arange(n) if n <= 1024 else np.sort(np.random.default_rng(92).choice(n, size=256, replace=False))
+    y_ref = orc.gemm_ref(x, w_hat[rows])
+    xd = to_dev(x)
+    ws = capi.workspace(16, n, k, xd.device)
+    for tune in [t for t in tunings(k) if (t & 0xF) != 3]:
+        y = torch.full((m, n), float("nan"), dtype=torch.float16, device=DEV)
+        capi.gemm_ws(xd, wd, zd, n, k, 64, algo=capi.SQ_ALGO_STREAM | (tune << 8), out=y, ws=ws)
+        torch.cuda.synchronize()
+        got = y.float().cpu().numpy()[:, rows]
+        assert np.all(np.isfinite(got)), (m, n, k, hex(tune))
+        assert np.max(np.abs(got - y_ref)) <= TOL * np.max(np.abs(y_ref)), (m, n, k, hex(tune))
+    if m >= 5:  # the automatic choice at this group size too
+        y_auto = capi.gemm_ws(xd, wd, zd, n, k, 64, ws=ws)
+        y_stream = capi.gemm_ws(xd, wd, zd, n, k, 64, algo=capi.SQ_ALGO_STREAM, ws=ws)
+        assert torch.equal(y_auto, y_stream)
+    assert capi.workspace_is_clean(ws)
+
+
 def test_stream_rejects_what_it_cannot_run(capi):
     d = linear(256, 1024, seed=47)
     with pytest.raises(capi.SqError):  # more than 16 tokens
         capi.gemm(to_dev(orc.synth_x(17, 1024, seed=48)), d["w_dev"], d["zs_dev"], 256, 1024, G, algo=capi.SQ_ALGO_STREAM)
-    d64 = orc.synth_linear(256, 1024, 64, seed=49)
-    with pytest.raises(capi.SqError):  # group size 64
-        capi.gemm(to_dev(orc.synth_x(8, 1024, seed=50)), to_dev(d64["w_l1"]), to_dev(d64["zs_l1"]), 256, 1024, 64,
+    d32 = orc.synth_linear(256, 1024, 32, seed=49)
+    with pytest.raises(capi.SqError):  # group size 32
+        capi.gemm(to_dev(orc.synth_x(8, 1024, seed=50)), to_dev(d32["w_l1"]), to_dev(d32["zs_l1"]), 256, 1024, 32,
                   algo=capi.SQ_ALGO_STREAM)
 
 
