@@ -70,6 +70,11 @@ hipError_t launch_skinny2_tuned(const void* x, const void* w, const void* zs, vo
 hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                                 int g, int tune, Epilogue epi, const LnPre* ln, hipStream_t st);
 hipError_t launch_skinny3_group(const SeqProblem* probs, int count, int M, void* ws, size_t ws_bytes, hipStream_t st);
+// The same kernel family for 17..32 tokens (two token tiles, activations staged in two halves); group size 128 only.
+hipError_t launch_skinny3_wide(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
+                               Epilogue epi, hipStream_t st);
+hipError_t launch_skinny3_wide_group(const SeqProblem* probs, int count, int M, void* ws, size_t ws_bytes,
+                                     hipStream_t st);
 // sq_gemm.hip: any M.  tune = 32-row tiles per workgroup (1,2,4) | ksplit << 8; ws may be null.
 size_t gemm_workspace_bytes(int M, int N, int K);
 hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, size_t ws_bytes, int M,

@@ -387,6 +387,250 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     if (tid == 0) __hip_atomic_store(&counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// ---- 17..32 tokens ------------------------------------------------------------------------------------------
+// Two token tiles per matrix-instruction operand (every unpacked weight word meets both), group size 128, 64 weight
+// rows and a K range of up to 4096 columns per workgroup.  32 tokens x 4096 columns of activations are 256 KiB, so
+// they are staged in two halves of 2048 columns (sixteen chunk slots): the second half waits in registers, requested
+// right after the first is parked, while the first half's chunks are consumed; one pair of barriers swaps it in.
+// The weight stream does not stop for that: the unit that follows the swap is requested before it.
+struct Sk3WideLds {
+    static constexpr int PSLOTS = 16;                    // chunk slots per half
+    static constexpr int XPITCH = PSLOTS * 256 + 16;     // bytes per staged token row (16 mod 256)
+    static constexpr int X_BYTES = 32 * XPITCH;
+    static constexpr int TILE = 4 * 2 * 4 * 64;          // floats a wave contributes: [rt][mt][v][lane]
+    static constexpr int RED_BYTES = SK3_NWV * TILE * 4;
+    static constexpr int Z_OFF = X_BYTES > RED_BYTES ? X_BYTES : RED_BYTES;
+    static constexpr int ZPITCH = 33;
+    static constexpr int FLAG_OFF = Z_OFF + 64 * ZPITCH * 4;
+    static constexpr int BYTES = FLAG_OFF + 16;
+};
+
+__device__ __forceinline__ void skinny3_wide_body(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ZS,
+                                                  const half_t* __restrict__ X, half_t* __restrict__ Y, float* part,
+                                                  unsigned* counters, int M, int N, int K, int ksplit,
+                                                  const Epilogue& epi, int rb, int slot, int nslots) {
+    using L = Sk3WideLds;
+    constexpr int RT = 4, MT = 2, CH = 4, ROWS = 64, TILE = L::TILE;
+    constexpr int WPR = L::PSLOTS * 16;              // 128-bit words per staged token row and half
+    constexpr int XPT = 32 * WPR / SK3_NT;           // 16
+    constexpr int ZPT = ROWS * 32 / SK3_NT;          // 4
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t sk3_lds[];
+    uint8_t* xl = sk3_lds;
+    uint32_t* zsl = (uint32_t*)(sk3_lds + L::Z_OFF);
+    unsigned* last_flag = (unsigned*)(sk3_lds + L::FLAG_OFF);
+    float* red = (float*)sk3_lds;
+
+    const NibbleMasks nm = nibble_masks();
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int li = lane & 15;
+    const int lj = lane >> 4;
+    const int ks = blockIdx.y;
+    const int chunks = K >> 7;
+    const int cps = (chunks + ksplit - 1) / ksplit;
+    int c_begin = ks * cps;
+    int nc = imin(c_begin + cps, chunks) - c_begin;
+    if (nc <= 0) {
+        nc = 0;
+        c_begin = 0;
+    }
+
+    uint32_t zreg[ZPT];
+#pragma unroll
+    for (int p = 0; p < ZPT; p++) {
+        const int idx = tid + p * SK3_NT;
+        const int r = idx >> 5, col = idx & 31;
+        const int row = imin(rb * ROWS + r, N - 1);
+        zreg[p] = ZS[(long)row * chunks + c_begin + (col < nc ? col : 0)];
+    }
+    // one half of the activations: token idx / 256, 128-bit column idx % 256 of the half
+    auto load_x = [&](int half, u32x4_t (&xr)[XPT]) {
+#pragma unroll
+        for (int p = 0; p < XPT; p++) {
+            const int idx = tid + p * SK3_NT;
+            const int m = idx / WPR, col = half * WPR + idx % WPR;
+            const bool ok = (m < M) && (col < nc * 16);
+            const uint32_t keep = ok ? 0xffffffffu : 0u;
+            const u32x4_t v = *(const u32x4_t*)(X + (ok ? (long)m * K + c_begin * 128 + col * 8 : 0));
+            xr[p] = (u32x4_t){v.x & keep, v.y & keep, v.z & keep, v.w & keep};
+        }
+    };
+    auto park_x = [&](const u32x4_t (&xr)[XPT]) {
+#pragma unroll
+        for (int p = 0; p < XPT; p++) {
+            const int idx = tid + p * SK3_NT;
+            *(u32x4_t*)(xl + (idx / WPR) * L::XPITCH + (idx % WPR) * 16) = xr[p];
+        }
+    };
+    u32x4_t xr[XPT];
+    load_x(0, xr);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");  // every wave's activation requests precede every weight request
+    __builtin_amdgcn_sched_barrier(0);
+
+    // weight units: (chunk pair pr = half, row tiles 2 rg, 2 rg + 1) x the two 64-byte halves of a line
+    u32x4_t wq[CH][RT];
+    int slot_of[CH];
+#pragma unroll
+    for (int u = 0; u < CH; u++) slot_of[u] = 2 * (wave + SK3_NWV * (u >> 1)) + (u & 1);
+    const uint8_t* wrow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) wrow[rt] = W + (long)imin(rb * ROWS + 16 * rt + li, N - 1) * (K >> 1) + lj * 16;
+    auto issue_unit = [&](int un) {
+        const int pr = un >> 1, rg = un & 1;
+#pragma unroll
+        for (int r = 0; r < 2; r++)
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int cl = slot_of[2 * pr + h];
+                wq[2 * pr + h][2 * rg + r] = *(const u32x4_t*)(wrow[2 * rg + r] + (long)(c_begin + (cl < nc ? cl : 0)) * 64);
+            }
+    };
+    issue_unit(0);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int p = 0; p < ZPT; p++) {
+        const int idx = tid + p * SK3_NT;
+        zsl[(idx >> 5) * L::ZPITCH + (idx & 31)] = zreg[p];
+    }
+    park_x(xr);
+    sk3_barrier();
+    issue_unit(1);  // ahead of the second half's activation requests, so that the weight stream does not pause for them
+    __builtin_amdgcn_sched_barrier(0);
+    load_x(1, xr);  // the second half waits in registers while the first is consumed
+    __builtin_amdgcn_sched_barrier(0);
+
+    float4_t acc[RT][MT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) acc[rt][mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+    const half8_t ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f,
+                          (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
+    const half8_t m960 = {(half_t)-960.f, (half_t)-960.f, (half_t)0.f, (half_t)0.f,
+                          (half_t)-960.f, (half_t)-960.f, (half_t)0.f, (half_t)0.f};
+    const uint8_t* xrd = xl + li * L::XPITCH + lj * 64;
+#pragma unroll
+    for (int un = 0; un < 4; un++) {
+        if (un == 2) {  // swap the second half of the activations in
+            sk3_barrier();
+            park_x(xr);
+            sk3_barrier();
+        }
+        if (un > 0 && un + 1 < 4) {
+            issue_unit(un + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        const int pr = un >> 1, rg = un & 1;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int u = 2 * pr + h;
+            const int cl = slot_of[u];
+            const int zcol = cl < nc ? cl : 0;
+            half8_t xa[MT][4];
+            float4_t xsum[MT], x960[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) {
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+                    xa[mt][t] = *(const half8_t*)(xrd + 16 * mt * L::XPITCH + (cl - L::PSLOTS * pr) * 256 + 16 * t);
+                xsum[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                x960[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    xsum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][t], ones, xsum[mt], 0, 0, 0);
+                    x960[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][t], m960, x960[mt], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 2; r++) {
+                const int rt = 2 * rg + r;
+                const half2_t zsv = bit_cast<half2_t>(zsl[(16 * rt + li) * L::ZPITCH + zcol]);
+                const float zf = (float)zsv.x;
+                const float sf = (float)zsv.y;
+                half8_t wv[4];
+#pragma unroll
+                for (int t = 0; t < 4; t++) wv[t] = unpack8_mixed(wq[u][rt][t], nm);
+#pragma unroll
+                for (int mt = 0; mt < MT; mt++) {
+                    float4_t tmp = x960[mt];
+#pragma unroll
+                    for (int t = 0; t < 4; t++) tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][t], wv[t], tmp, 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < 4; v++) acc[rt][mt][v] += sf * (tmp[v] - zf * xsum[mt][v]);
+                }
+            }
+        }
+    }
+    sk3_barrier();  // every wave is done with the activations, which the partials now overwrite
+
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) red[wave * TILE + ((rt * MT + mt) * 4 + v) * 64 + lane] = acc[rt][mt][v];
+    sk3_barrier();
+
+    // Element t of the tile: lane l = t % 64, v, mt, rt -> token m = 16 mt + 4 (l / 16) + v, row n = 64 rb + 16 rt + l % 16.
+    if (ksplit == 1) {
+        for (int t = tid; t < TILE; t += SK3_NT) {
+            float sum = 0.f;
+#pragma unroll
+            for (int p = 0; p < SK3_NWV; p++) sum += red[p * TILE + t];
+            const int l = t & 63, v = (t >> 6) & 3, mt = (t >> 8) % MT, rt = (t >> 8) / MT;
+            const int m = 16 * mt + 4 * (l >> 4) + v;
+            const int n = rb * ROWS + 16 * rt + (l & 15);
+            if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum, m, n, N, epi);
+        }
+        return;
+    }
+    float* mine = part + ((long)ks * nslots + slot) * TILE;
+    for (int t4 = tid * 4; t4 < TILE; t4 += 4 * SK3_NT) {
+        float4_t sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int p = 0; p < SK3_NWV; p++) sum += *(const float4_t*)(&red[p * TILE + t4]);
+        store_coherent_x4(mine + t4, sum);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    sk3_barrier();
+    if (tid == 0) {
+        const unsigned old = __hip_atomic_fetch_add(&counters[slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *last_flag = (old == (unsigned)(ksplit - 1)) ? 1u : 0u;
+    }
+    sk3_barrier();
+    if (!*last_flag) return;
+    for (int t4 = tid * 4; t4 < TILE; t4 += 4 * SK3_NT) {
+        const float* src[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) src[q] = part + ((long)(q < ksplit ? q : 0) * nslots + slot) * TILE + t4;
+        float4_t pv[8];
+        load8_coherent_x4(src, pv);
+        float4_t sum = pv[0];
+#pragma unroll
+        for (int q = 1; q < 8; q++)
+            if (q < ksplit) sum += pv[q];  // fixed order
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int t = t4 + e;
+            const int l = t & 63, v = (t >> 6) & 3, mt = (t >> 8) % MT, rt = (t >> 8) / MT;
+            const int m = 16 * mt + 4 * (l >> 4) + v;
+            const int n = rb * ROWS + 16 * rt + (l & 15);
+            if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum[e], m, n, N, epi);
+        }
+    }
+    if (tid == 0) __hip_atomic_store(&counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__global__ __launch_bounds__(SK3_NT) void skinny3_wide_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ZS,
+                                                              const half_t* __restrict__ X, half_t* __restrict__ Y,
+                                                              float* part, unsigned* counters, int M, int N, int K,
+                                                              int ksplit, Epilogue epi) {
+    skinny3_wide_body(W, ZS, X, Y, part, counters, M, N, K, ksplit, epi, blockIdx.x, blockIdx.x, gridDim.x);
+}
+
 template <int MROWS, int RT, int CH, bool LN, int GPC>
 __global__ __launch_bounds__(SK3_NT) void skinny3_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ZS,
                                                          const half_t* __restrict__ X, half_t* __restrict__ Y,
@@ -420,6 +664,18 @@ __global__ __launch_bounds__(SK3_NT) void skinny3_group_kernel(const Skinny3Grou
     const Epilogue epi{grp.bias[p], grp.residual[p], grp.act[p]};
     skinny3_body<MROWS, RT, CH, SK3_DEPTH, false, 1>(grp.W[p], grp.ZS[p], grp.X[p], grp.Y[p], part, counters, M, grp.N[p], K,
                                                   ksplit, epi, LnPre{nullptr, nullptr, 0.f}, rb, blockIdx.x, gridDim.x);
+}
+
+__global__ __launch_bounds__(SK3_NT) void skinny3_wide_group_kernel(const Skinny3Group grp, float* part,
+                                                                    unsigned* counters, int M, int K, int ksplit) {
+    int p = 0;
+#pragma unroll
+    for (int q = 0; q < GEMV_GROUP_MAX - 1; q++)
+        if (q + 1 < grp.count && (int)blockIdx.x >= grp.blk_end[q]) p = q + 1;
+    const int rb = blockIdx.x - (p > 0 ? grp.blk_end[p - 1] : 0);
+    const Epilogue epi{grp.bias[p], grp.residual[p], grp.act[p]};
+    skinny3_wide_body(grp.W[p], grp.ZS[p], grp.X[p], grp.Y[p], part, counters, M, grp.N[p], K, ksplit, epi, rb, blockIdx.x,
+                      gridDim.x);
 }
 
 template <typename Kern>
@@ -579,6 +835,59 @@ hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, vo
     SQ_SK3_CH(16, 4);
 #undef SQ_SK3_CH
 #undef SQ_SK3
+}
+
+// 17..32 tokens (any M <= 32 works), group size 128, K % 128 == 0, 64-row workgroups.  hipErrorInvalidValue when the
+// shape does not fit: a K split without a workspace, or so few row blocks that most CUs would idle (the caller then
+// takes the split-K kernel, which splits K further).
+hipError_t launch_skinny3_wide(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
+                               Epilogue epi, hipStream_t st) {
+    if (M < 1 || M > 32 || K % 128 != 0) return hipErrorInvalidValue;
+    const int chunks = K / 128, ksplit = (chunks + 31) / 32, blocks = (N + 63) / 64;
+    const int cps = (chunks + ksplit - 1) / ksplit;
+    if (ksplit > 8 || (ksplit > 1 && !ws) || (ksplit - 1) * cps >= chunks || blocks > 16384 || blocks * ksplit < 128)
+        return hipErrorInvalidValue;
+    static bool allowed[64];
+    const hipError_t e = allow_lds(skinny3_wide_kernel, Sk3WideLds::BYTES, allowed);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(skinny3_wide_kernel, dim3(blocks, ksplit), dim3(SK3_NT), Sk3WideLds::BYTES, st, (const uint8_t*)w,
+                       (const uint32_t*)zs, (const half_t*)x, (half_t*)y,
+                       ws ? (float*)((char*)ws + SK3_COUNTER_BYTES) : nullptr, (unsigned*)ws, M, N, K, ksplit, epi);
+    return hipGetLastError();
+}
+
+hipError_t launch_skinny3_wide_group(const SeqProblem* probs, int count, int M, void* ws, size_t ws_bytes,
+                                     hipStream_t st) {
+    if (count < 2 || count > GEMV_GROUP_MAX || M < 1 || M > 32) return hipErrorInvalidValue;
+    const int K = probs[0].K;
+    if (K % 128 != 0) return hipErrorInvalidValue;
+    Skinny3Group g;
+    int blocks = 0;
+    for (int p = 0; p < GEMV_GROUP_MAX; p++) {
+        const SeqProblem& q = probs[p < count ? p : 0];
+        if (q.K != K || q.group_size != 128) return hipErrorInvalidValue;
+        g.W[p] = (const uint8_t*)q.w;
+        g.ZS[p] = (const uint32_t*)q.zs;
+        g.X[p] = (const half_t*)q.x;
+        g.Y[p] = (half_t*)q.y;
+        g.bias[p] = (const half_t*)q.bias;
+        g.residual[p] = (const half_t*)q.residual;
+        g.N[p] = q.N;
+        g.act[p] = q.act;
+        if (p < count) blocks += (q.N + 63) / 64;
+        g.blk_end[p] = blocks;
+    }
+    g.count = count;
+    const int chunks = K / 128, ksplit = (chunks + 31) / 32;
+    const int cps = (chunks + ksplit - 1) / ksplit;
+    if (ksplit > 8 || (ksplit - 1) * cps >= chunks || blocks > 16384 || blocks * ksplit < 128) return hipErrorInvalidValue;
+    if (ksplit > 1 && (!ws || ws_bytes < skinny2_group_workspace_bytes(probs, count, M))) return hipErrorInvalidValue;
+    static bool allowed[64];
+    const hipError_t e = allow_lds(skinny3_wide_group_kernel, Sk3WideLds::BYTES, allowed);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(skinny3_wide_group_kernel, dim3(blocks, ksplit), dim3(SK3_NT), Sk3WideLds::BYTES, st, g,
+                       ws ? (float*)((char*)ws + SK3_COUNTER_BYTES) : nullptr, (unsigned*)ws, M, K, ksplit);
+    return hipGetLastError();
 }
 
 // Grouped launch: count in 2..GEMV_GROUP_MAX linears with the same K, group size 128, 5 <= M <= 16.

@@ -122,7 +122,7 @@ def test_stream_group_size_64(capi, n, k, m):
 
 def test_stream_rejects_what_it_cannot_run(capi):
     d = linear(256, 1024, seed=47)
-    with pytest.raises(capi.SqError):  # more than 16 tokens
+    with pytest.raises(capi.SqError):  # more than 16 tokens on a weight too small for the two-tile variant
         capi.gemm(to_dev(orc.synth_x(17, 1024, seed=48)), d["w_dev"], d["zs_dev"], 256, 1024, G, algo=capi.SQ_ALGO_STREAM)
     d32 = orc.synth_linear(256, 1024, 32, seed=49)
     with pytest.raises(capi.SqError):  # group size 32
@@ -146,6 +146,34 @@ def test_stream_is_the_automatic_choice_at_full_size(capi, n, k, m):
     y_ref = orc.gemm_ref(x, d["w_hat"][rows])
     got = y_auto.float().cpu().numpy()[:, rows]
     assert np.max(np.abs(got - y_ref)) <= TOL * np.max(np.abs(y_ref))
+    assert capi.workspace_is_clean(ws)
+
+
+@pytest.mark.parametrize("n,k", [(8192, 1024), (8200, 3200), (16384, 4096), (4096, 16384), (4096, 11008)])
+@pytest.mark.parametrize("m", [17, 24, 31, 32])
+def test_stream_two_token_tiles(capi, n, k, m):
+    """17..32 tokens: activations staged in two halves under one weight stream; explicit kernel id and automatic
+    dispatch against the oracle on sampled rows, with bias, ReLU and residual on the way out."""
+    d = linear(n, k, seed=95)
+    rng = np.random.default_rng(96 + m)
+    x = orc.synth_x(m, k, seed=97 + m)
+    bias = rng.normal(0, 1.0, size=n).astype(np.float16)
+    res = rng.normal(0, 1.0, size=(m, n)).astype(np.float16)
+    rows = np.sort(rng.choice(n, size=256, replace=False))
+    rows[0], rows[-1] = 0, n - 1
+    plain = orc.gemm_ref(x, d["w_hat"][rows]).astype(np.float64)
+    ref = np.maximum(plain + bias[rows].astype(np.float64)[None, :], 0.0) + res[:, rows].astype(np.float64)
+    xd, bd, rd = to_dev(x), to_dev(bias), to_dev(res)
+    ws = capi.workspace(m, n, k, xd.device)
+    y = capi.gemm_fused(xd, d["w_dev"], d["zs_dev"], n, k, G, bias=bd, residual=rd, act=1, algo=capi.SQ_ALGO_STREAM, ws=ws)
+    y_auto = capi.gemm_fused(xd, d["w_dev"], d["zs_dev"], n, k, G, bias=bd, residual=rd, act=1, ws=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_auto)
+    got = y.float().cpu().numpy()[:, rows]
+    assert np.all(np.isfinite(got))
+    assert np.max(np.abs(got - ref)) <= TOL * np.max(np.abs(plain))
+    # fixed summation order: the same bits on a second call, counters back at zero
+    assert torch.equal(y, capi.gemm_fused(xd, d["w_dev"], d["zs_dev"], n, k, G, bias=bd, residual=rd, act=1, ws=ws))
     assert capi.workspace_is_clean(ws)
 
 
