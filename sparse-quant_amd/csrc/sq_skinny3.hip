@@ -1,4 +1,5 @@
-// Streaming skinny GEMM for up to 16 tokens, group size 128, layout L1: the decode kernel for small batches.
+// Streaming skinny GEMM for up to 32 tokens, group size 128 (64 up to 16 tokens), layout L1: the decode kernel for
+// small batches.
 //
 // The matrix instruction, the operand mapping and the per-chunk arithmetic are those of the split-K
 // decode kernel in sq_skinny2.hip (v_mfma_f32_16x16x32_f16, weights as the B operand straight from
@@ -40,14 +41,10 @@ namespace {
 constexpr int SK3_COUNTER_BYTES = 65536;  // start of the workspace: one uint32 per row block
 constexpr int SK3_NWV = 8;
 constexpr int SK3_NT = 64 * SK3_NWV;
-#ifndef SQ_SK3_DEPTH
-#define SQ_SK3_DEPTH 1
-#endif
-#ifndef SQ_SK3_DEPTH_PRE
-#define SQ_SK3_DEPTH_PRE 1
-#endif
-constexpr int SK3_DEPTH_PRE = SQ_SK3_DEPTH_PRE;  // units requested before the activations are parked
-constexpr int SK3_DEPTH = SQ_SK3_DEPTH;  // units of four weight loads requested ahead of the one being consumed
+// Units of weight loads requested before the activations are parked, and ahead of the unit being consumed (two
+// and three were measured: a wave that issues into a full memory queue stalls before it reaches the parking stores).
+constexpr int SK3_DEPTH_PRE = 1;
+constexpr int SK3_DEPTH = 1;
 
 template <int MROWS, int RT, int CH, int GPC = 1>
 struct Sk3Lds {
