@@ -491,6 +491,7 @@ def main():
         try:
             out["decode_batch"] = decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream)
             out["config1"] = config1_leg(torch, capi, dev, gen, stream)
+            out["layernorm_fused"] = ln_fused_leg(torch, capi, pool, shapes, g, dev, gen, stream)
             if m <= 4:
                 out["sequence"] = sequence_leg(torch, capi, pool, shapes, m, g, dev, gen, stream, bytes_per_step)
             out["fused_qkv"] = fused_qkv_leg(torch, capi, m, g, dev, gen, stream, args.layers, bytes_per_step)
@@ -722,6 +723,62 @@ def config1_leg(torch, capi, dev, gen, stream, g=64, n=4096, k=4096, copies=32):
         res["m%d" % m] = {"us": round(us, 3), "gbs": round(nbytes / us / 1e3, 1),
                           "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                           "parity_max_rel_err": round(err, 6)}
+    return res
+
+
+def ln_fused_leg(torch, capi, pool, shapes, g, dev, gen, stream, m=8):
+    """LayerNorm + fc1 at M = 8 (the shape of the end-to-end decode step): sq_layernorm followed by the linear (two
+    launches) against sq_w4a16_gemm_ln_fused (the normalisation inside the linear's kernel), cold weights, HIP-graph
+    replay; parity of the fused call against the oracle's LayerNorm (rounded to fp16) and product on sampled rows."""
+    import numpy as np
+    import w4a16_oracle as orc
+    idx = [i for i, (name, _, _) in enumerate(shapes) if name == "fc1"][0]
+    _, n, k = shapes[idx]
+    x = (torch.randn((m, k), device=dev, generator=gen) * 1.5 + 0.2).half()
+    gamma = (torch.randn(k, device=dev, generator=gen) * 0.2 + 1.0).half()
+    beta = (torch.randn(k, device=dev, generator=gen) * 0.2).half()
+    h = torch.empty_like(x)
+    y = torch.empty((m, n), dtype=torch.float16, device=dev)
+    torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
+    res = {"shape": "LayerNorm(8 x 4096) -> fc1 4096 -> 16384, group %d" % g}
+    with torch.cuda.stream(stream):
+        ws = capi.workspace(m, n, k, dev, stream)
+
+        def two():
+            for layer in pool:
+                capi.layernorm(x, gamma, beta, 1e-5, out=h, stream=stream)
+                capi.gemm_ws(h, layer[idx][0], layer[idx][1], n, k, g, out=y, stream=stream, ws=ws)
+
+        def fused():
+            for layer in pool:
+                capi.gemm_ln_fused(x, gamma, beta, 1e-5, layer[idx][0], layer[idx][1], n, k, g, out=y, stream=stream, ws=ws)
+
+        fused()
+        stream.synchronize()
+        w, zs = pool[-1][idx]
+        ridx = np.sort(np.random.default_rng(5).choice(n, size=64, replace=False))
+        hn = orc.layernorm_ref(x.cpu().numpy(), gamma.cpu().numpy(), beta.cpu().numpy(), 1e-5).astype(np.float16)
+        ref = orc.gemm_ref(hn, orc.dequant_l1(w.cpu().numpy()[ridx], zs.cpu().numpy()[ridx], g))
+        got = y.float().cpu().numpy()[:, ridx]
+        err = gate(float(np.max(np.abs(got - ref)) / np.max(np.abs(ref))) if np.all(np.isfinite(got)) else float("inf"),
+                   "LayerNorm inside fc1 at M=%d" % m)
+        res["parity_max_rel_err"] = round(err, 6)
+        for name, fn in (("layernorm_then_linear", two), ("layernorm_inside_linear", fused)):
+            fn()
+            stream.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                fn()
+            for _ in range(5):
+                graph.replay()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(50):
+                graph.replay()
+            e1.record(stream)
+            stream.synchronize()
+            res[name] = {"us": round(e0.elapsed_time(e1) * 1e3 / (50 * len(pool)), 2),
+                         "launches": 2 if fn is two else 1}
     return res
 
 
