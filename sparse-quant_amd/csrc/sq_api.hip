@@ -111,8 +111,15 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
         const int wide_ksplit = (K / 128 + 31) / 32;
         const bool wide_ok = M > 16 && M <= 32 && group_size == 128 && K % 128 == 0 && wide_ksplit <= 8 &&
                              (wide_ksplit == 1 || ws_ok) && (long)((N + 63) / 64) * wide_ksplit >= 128;
+        // more than 32 tokens at group size 128: the tiled kernel with both operands through LDS and K split
+        // through the workspace (4096 x 4096 at 48 tokens 14.5 us against 17.2 for two blocks of the split-K
+        // decode kernel, fc1 24.7 against 28.2, fc2 27.0 against 32.3; at 64 tokens 14.5 against 20.5 for the
+        // 16-column kernel)
+        const bool lds_ok = M > 32 && group_size == 128 && K % 256 == 0 && gemm_ws;
         if (stream_ok || wide_ok) {
             kernel = SQ_ALGO_STREAM;
+        } else if (lds_ok) {
+            kernel = SQ_ALGO_GEMM;
         } else if (ws_ok && M > 4 && M <= 32 && (large || M > 16 || K > 8192)) {
             kernel = SQ_ALGO_SKINNY_WS;
         } else if (ws_ok && M > 32 && M <= 48 && (large || K > 8192)) {

@@ -168,4 +168,32 @@ __device__ __forceinline__ void load8_coherent_x4(const float* const (&p)[8], fl
         : "memory");
 }
 
+// Sixteen coherent 128-bit loads in flight: p[i] points at the SECOND of two locations 4096 bytes
+// apart (v[2i] = p[i][-4096 bytes], v[2i+1] = p[i][0]); one asm block with its own wait, so that no
+// register holding a result can be touched before the data is there.
+__device__ __forceinline__ void load16_coherent_x4(const float* const (&p)[8], float4_t (&v)[16]) {
+    asm volatile(
+        "global_load_dwordx4 %0, %16, off offset:-4096 sc1\n\t"
+        "global_load_dwordx4 %1, %16, off sc1\n\t"
+        "global_load_dwordx4 %2, %17, off offset:-4096 sc1\n\t"
+        "global_load_dwordx4 %3, %17, off sc1\n\t"
+        "global_load_dwordx4 %4, %18, off offset:-4096 sc1\n\t"
+        "global_load_dwordx4 %5, %18, off sc1\n\t"
+        "global_load_dwordx4 %6, %19, off offset:-4096 sc1\n\t"
+        "global_load_dwordx4 %7, %19, off sc1\n\t"
+        "global_load_dwordx4 %8, %20, off offset:-4096 sc1\n\t"
+        "global_load_dwordx4 %9, %20, off sc1\n\t"
+        "global_load_dwordx4 %10, %21, off offset:-4096 sc1\n\t"
+        "global_load_dwordx4 %11, %21, off sc1\n\t"
+        "global_load_dwordx4 %12, %22, off offset:-4096 sc1\n\t"
+        "global_load_dwordx4 %13, %22, off sc1\n\t"
+        "global_load_dwordx4 %14, %23, off offset:-4096 sc1\n\t"
+        "global_load_dwordx4 %15, %23, off sc1\n\t"
+        "s_waitcnt vmcnt(0)"
+        : "=&v"(v[0]), "=&v"(v[1]), "=&v"(v[2]), "=&v"(v[3]), "=&v"(v[4]), "=&v"(v[5]), "=&v"(v[6]), "=&v"(v[7]),
+          "=&v"(v[8]), "=&v"(v[9]), "=&v"(v[10]), "=&v"(v[11]), "=&v"(v[12]), "=&v"(v[13]), "=&v"(v[14]), "=&v"(v[15])
+        : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3]), "v"(p[4]), "v"(p[5]), "v"(p[6]), "v"(p[7])
+        : "memory");
+}
+
 }  // namespace sq

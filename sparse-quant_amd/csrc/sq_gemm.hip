@@ -33,6 +33,98 @@ constexpr int GEMM_STAGES = 3;  // register stages; loads run GEMM_STAGES - 1 st
 
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
+// What follows the K loop in both tiled kernels: with K split over gridDim.z workgroups the
+// partial tiles meet in the workspace, then the epilogue and the fp16 stores.
+template <int MI>
+__device__ __forceinline__ void gemm_tail(float16_t (&acc)[MI][2], half_t* __restrict__ Y, int M, int N, int m0, int n0,
+                                          const Epilogue& epi, float* part, unsigned* counters) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int ln = lane & 31;
+    const int lc = lane >> 5;
+    const int ksplit = gridDim.z;
+    if (ksplit > 1) {
+        // Partial tiles meet in the workspace: 128-bit stores at the device-coherent cache level,
+        // one counter per output tile; the workgroup that arrives last adds the partials in a
+        // fixed order (bit-reproducible), stores the tile and resets the counter.
+        __shared__ unsigned last_flag;
+        constexpr int SLOTS = MI * 2 * 4;  // float4 per thread
+        const long tile = (long)blockIdx.y * gridDim.x + blockIdx.x;
+        const long ntile = (long)gridDim.x * gridDim.y;
+        float* mine = part + ((long)blockIdx.z * ntile + tile) * (SLOTS * 256 * 4);
+#pragma unroll
+        for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float4_t v4 = {acc[mi][ni][4 * q], acc[mi][ni][4 * q + 1], acc[mi][ni][4 * q + 2],
+                                         acc[mi][ni][4 * q + 3]};
+                    store_coherent_x4(mine + (((mi * 2 + ni) * 4 + q) * 256 + tid) * 4, v4);
+                }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned old = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_flag = (old == (unsigned)(ksplit - 1)) ? 1u : 0u;
+        }
+        __syncthreads();
+        if (!last_flag) return;
+        // The last arriver's loads are round trips to L2 that nothing hides: sixteen per thread in
+        // flight, i.e. 16 / NZ of its SLOTS per trip, NZ = the number of partials rounded up to 2, 4
+        // or 8 (sources past ksplit re-read the first partial and are not added).
+        const float* first = part + tile * (SLOTS * 256 * 4) + tid * 4;
+        const long zstride = ntile * (SLOTS * 256 * 4);
+        auto reduce = [&](auto NZ_) {
+            constexpr int NZ = decltype(NZ_)::value;
+            constexpr int PAIRS = 8 / NZ;  // pairs of slots per trip
+#pragma unroll
+            for (int s0 = 0; s0 < SLOTS; s0 += 2 * PAIRS) {
+                const float* src[8];
+                float4_t pv[16];
+#pragma unroll
+                for (int pr = 0; pr < PAIRS; pr++)
+#pragma unroll
+                    for (int z = 0; z < NZ; z++)
+                        src[pr * NZ + z] = first + (long)(z < ksplit ? z : 0) * zstride + (s0 + 2 * pr + 1) * 1024;
+                load16_coherent_x4(src, pv);
+#pragma unroll
+                for (int pr = 0; pr < PAIRS; pr++)
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        float4_t sum = pv[2 * (pr * NZ) + h];
+#pragma unroll
+                        for (int z = 1; z < NZ; z++)
+                            if (z < ksplit) sum += pv[2 * (pr * NZ + z) + h];
+                        const int slot = s0 + 2 * pr + h;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[slot >> 3][(slot >> 2) & 1][4 * (slot & 3) + e] = sum[e];
+                    }
+            }
+        };
+        if (ksplit <= 2)
+            reduce(std::integral_constant<int, 2>{});
+        else if (ksplit <= 4)
+            reduce(std::integral_constant<int, 4>{});
+        else
+            reduce(std::integral_constant<int, 8>{});
+        if (tid == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    // Epilogue: fp32 -> fp16, 32 consecutive columns per half-wave.
+#pragma unroll
+    for (int mi = 0; mi < MI; mi++)
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++) {
+            const int n = n0 + 32 * ni + ln;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int m = m0 + 32 * mi + 8 * (v >> 2) + 4 * lc + (v & 3);
+                if (m < M && n < N) Y[(long)m * N + n] = epilogue(acc[mi][ni][v], m, n, N, epi);
+            }
+        }
+}
+
 // Two waves per SIMD (two workgroups per CU): one wave alone cannot both issue the
 // unpack / LDS / load instructions of a step and keep the matrix pipe full.
 template <int MI>
@@ -192,78 +284,197 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         step(it + 5, std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
     }
 
-    if (ksplit > 1) {
-        // Partial tiles meet in the workspace: 128-bit stores at the device-coherent cache level,
-        // one counter per output tile; the workgroup that arrives last adds the partials in a
-        // fixed order (bit-reproducible), stores the tile and resets the counter.
-        __shared__ unsigned last_flag;
-        constexpr int SLOTS = MI * 2 * 4;  // float4 per thread
-        const long tile = (long)blockIdx.y * gridDim.x + blockIdx.x;
-        const long ntile = (long)gridDim.x * gridDim.y;
-        float* mine = part + ((long)blockIdx.z * ntile + tile) * (SLOTS * 256 * 4);
-#pragma unroll
-        for (int mi = 0; mi < MI; mi++)
-#pragma unroll
-            for (int ni = 0; ni < 2; ni++)
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const float4_t v4 = {acc[mi][ni][4 * q], acc[mi][ni][4 * q + 1], acc[mi][ni][4 * q + 2],
-                                         acc[mi][ni][4 * q + 3]};
-                    store_coherent_x4(mine + (((mi * 2 + ni) * 4 + q) * 256 + tid) * 4, v4);
-                }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (tid == 0) {
-            const unsigned old = __hip_atomic_fetch_add(&counters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            last_flag = (old == (unsigned)(ksplit - 1)) ? 1u : 0u;
-        }
-        __syncthreads();
-        if (!last_flag) return;
-#pragma unroll
-        for (int mi = 0; mi < MI; mi++)
-#pragma unroll
-            for (int ni = 0; ni < 2; ni++)
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    const float* src[8];
-#pragma unroll
-                    for (int z = 0; z < 8; z++)
-                        src[z] = part + ((long)(z < ksplit ? z : 0) * ntile + tile) * (SLOTS * 256 * 4) +
-                                 (((mi * 2 + ni) * 4 + q) * 256 + tid) * 4;
-                    float4_t pv[8];
-                    load8_coherent_x4(src, pv);
-                    float4_t sum = pv[0];
-#pragma unroll
-                    for (int z = 1; z < 8; z++)
-                        if (z < ksplit) sum += pv[z];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) acc[mi][ni][4 * q + e] = sum[e];
-                }
-        if (tid == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
+    gemm_tail<MI>(acc, Y, M, N, m0, n0, epi, part, counters);
+}
 
-    // Epilogue: fp32 -> fp16, 32 consecutive columns per half-wave.
+// One direct global -> LDS load: 16 (or 4) bytes per lane, lane l lands at lds_byte + 16 (4) * l.
+// Written as inline assembly on purpose: the compiler, when it knows of such a load, makes every
+// later LDS read wait for ALL outstanding vector memory loads unless it can prove the two apart,
+// which it cannot for stages picked at run time.  The kernel orders them itself (a counted
+// s_waitcnt and a barrier per step); the "memory" clobbers keep LDS reads from moving across.
+__device__ __forceinline__ void load_to_lds_x4(const void* g, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte) : "memory");
+}
+__device__ __forceinline__ void load_to_lds_x1(const void* g, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_byte) : "memory");
+}
+
+// Both operands through LDS, for group size 128 and K a multiple of 256.  The kernels above hand
+// every lane its own 16 bytes of a weight row (32 rows per wave-wide load) and 4 bytes of
+// zeros/scales, and the L1 takes lanes that are not neighbours in memory one at a time: about 1240
+// cache accesses per workgroup and K step, three per four cycles, which is what bounds those
+// kernels between decode and prefill.  Here every operand goes global -> LDS with direct loads
+// (no registers in between):
+//   * weights: a wave moves its own 64 rows x 32 bytes in two instructions whose neighbouring
+//     lanes are neighbours in memory; lane l of instruction i fetches half
+//     (l & 1) ^ ((row >> 3) & 1) of row 32 * i + l / 2, so that the operand reads (lane = row,
+//     128 bits) are bank-conflict free;
+//   * activations: the swizzled chunk order of the register-staged kernel, written by the load
+//     instead of a store;
+//   * zeros/scales: the two pairs of a group of four steps, one dword per lane and pair, once per
+//     four steps.
+// Three stages (two for zeros/scales), loads two steps ahead; one barrier per step, behind a
+// counted wait for the loads of the next step (the loads just issued stay in flight).  Same
+// operand mapping and arithmetic as gemm_kernel: bit-identical results.
+template <int MI>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_lds_kernel(
+    const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS, const half_t* __restrict__ X, half_t* __restrict__ Y,
+    int M, int N, int K, Epilogue epi, float* part, unsigned* counters) {
+    constexpr int BM = 32 * MI;
+    constexpr int XB = BM * 128;  // bytes of an activation stage
+    constexpr int WB = 256 * 32;  // bytes of a weight stage
+    constexpr int ZB = 256 * 8;   // bytes of a zeros/scales stage: 4 waves x 2 pairs x 64 rows
+    constexpr int W_OFF = 0, Z_OFF = 3 * WB, X_OFF = Z_OFF + 2 * ZB;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[X_OFF + 3 * XB];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
+
+    const NibbleMasks nm = nibble_masks();
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ln = lane & 31;
+    const int lc = lane >> 5;
+    const int m0 = blockIdx.y * BM;
+    const int n0 = blockIdx.x * GEMM_BN + 64 * wave;
+    const int groups = K >> 7;
+    const int nit = K / GEMM_BK;
+    // K split in whole four-step groups
+    const int ksplit = gridDim.z;
+    const int spz = ((nit + ksplit - 1) / ksplit + 3) & ~3;
+    const int it0 = blockIdx.z * spz;
+    const int it1 = imin(it0 + spz, nit);
+
+    const half_t* xsrc[MI];
+    int xchunk[MI];
+#pragma unroll
+    for (int p = 0; p < MI; p++) {
+        const int R = 32 * p + 8 * wave + (lane >> 3);
+        xchunk[p] = ((lane & 7) ^ swz(R)) * 8;
+        xsrc[p] = X + (long)imin(m0 + R, M - 1) * K;
+    }
+    const uint8_t* wld[2];
+    int whalf[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int r = 32 * i + (lane >> 1);
+        whalf[i] = 32 * ((lane & 1) ^ ((r >> 3) & 1));
+        wld[i] = W + (long)imin(n0 + r, N - 1) * (K >> 1);
+    }
+    const half2_t* zld = ZS + (long)imin(n0 + lane, N - 1) * groups;  // lane = row of the wave's 64
+    int woff[2], zoff[2];
+#pragma unroll
+    for (int ni = 0; ni < 2; ni++) {
+        woff[ni] = W_OFF + wave * 2048 + ((32 * ni + ln) * 2 + (lc ^ ((ln >> 3) & 1))) * 16;
+        zoff[ni] = Z_OFF + wave * 512 + (32 * ni + ln) * 4;
+    }
+    int xoff[4];
+#pragma unroll
+    for (int t = 0; t < 4; t++) xoff[t] = X_OFF + ln * 128 + (((4 * lc + t) ^ swz(ln)) * 16);
+
+    float16_t acc[MI][2];
 #pragma unroll
     for (int mi = 0; mi < MI; mi++)
 #pragma unroll
-        for (int ni = 0; ni < 2; ni++) {
-            const int n = n0 + 32 * ni + ln;
+        for (int ni = 0; ni < 2; ni++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int m = m0 + 32 * mi + 8 * (v >> 2) + 4 * lc + (v & 3);
-                if (m < M && n < N) Y[(long)m * N + n] = epilogue(acc[mi][ni][v], m, n, N, epi);
+            for (int v = 0; v < 16; v++) acc[mi][ni][v] = 0.f;
+
+    // Loads of step `it` into stage c (wave-uniform); a k past the end is clamped, its scale zeroed at use.
+    auto issue = [&](int it, int c) {
+#pragma unroll
+        for (int p = 0; p < MI; p++) {
+            const int kx = imin(it * GEMM_BK + xchunk[p], K - 8);
+            load_to_lds_x4(xsrc[p] + kx, lds0 + X_OFF + c * XB + (32 * p + 8 * wave) * 128);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int kc = imin(it * GEMM_BK + whalf[i], K - 32);
+            load_to_lds_x4(wld[i] + (kc >> 1), lds0 + W_OFF + c * WB + wave * 2048 + i * 1024);
+        }
+    };
+    // The two zeros/scales pairs of the four-step group that starts at step `it`, into stage zc.
+    auto issue_zs = [&](int it, int zc) {
+        const int gi = imin(it >> 1, groups - 2);
+        load_to_lds_x1(zld + gi, lds0 + Z_OFF + zc * ZB + wave * 512);
+        load_to_lds_x1(zld + gi + 1, lds0 + Z_OFF + zc * ZB + wave * 512 + 256);
+    };
+
+    // One K step: J = step within its group of four, c = its stage, cf = the stage read in the step
+    // before (free since that step's barrier), zc = the zeros/scales stage of its group.
+    auto step = [&](int it, int c, int cf, int zc, auto J_) {
+        constexpr int j = decltype(J_)::value;
+        issue(it + 2, cf);
+        if constexpr (j == 2) issue_zs(it + 2, zc ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        const bool kin = it < it1 && it * GEMM_BK + 32 * lc < K;  // false past the range: scale 0 -> W_hat 0
+        u32x4_t q[2];
+        half2_t z64[2], sc[2];
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++) {
+            q[ni] = *(const u32x4_t*)(lds + c * WB + woff[ni]);
+            const half2_t zsv = *(const half2_t*)(lds + zc * ZB + (j >> 1) * 256 + zoff[ni]);
+            const half_t sv = kin ? zsv.y : (half_t)0.f;
+            z64[ni] = (half2_t){zsv.x, zsv.x};
+            sc[ni] = (half2_t){sv, sv};
+        }
+        const uint8_t* xp = lds + c * XB;
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            half8_t bf[2];
+#pragma unroll
+            for (int ni = 0; ni < 2; ni++) bf[ni] = dequant8(q[ni][t], z64[ni], sc[ni], nm);
+#pragma unroll
+            for (int mi = 0; mi < MI; mi++) {
+                const half8_t a = *(const half8_t*)(xp + (32 * mi) * 128 + xoff[t]);
+#pragma unroll
+                for (int ni = 0; ni < 2; ni++)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, bf[ni], acc[mi][ni], 0, 0, 0);
             }
         }
+        __builtin_amdgcn_sched_barrier(0);
+        // the loads of step it + 1 (issued a step ago) have landed, this wave's operand reads are done:
+        // behind the barrier stage c is free and the next stage is complete
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(MI + 2 + (j == 2 ? 2 : 0)) : "memory");
+    };
+
+    issue_zs(it0, 0);
+    issue(it0, 0);
+    issue(it0 + 1, 1);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(MI + 2) : "memory");
+    const int end = it0 + (it1 - it0 + 3) / 4 * 4;  // padded with steps whose scale is 0 and whose loads are clamped
+    int c = 0, cp = 2, zc = 0;
+    auto advance = [&]() {
+        cp = c;
+        c = c == 2 ? 0 : c + 1;
+    };
+    for (int it = it0; it < end; it += 4) {
+        step(it, c, cp, zc, std::integral_constant<int, 0>{});
+        advance();
+        step(it + 1, c, cp, zc, std::integral_constant<int, 1>{});
+        advance();
+        step(it + 2, c, cp, zc, std::integral_constant<int, 2>{});
+        advance();
+        step(it + 3, c, cp, zc, std::integral_constant<int, 3>{});
+        advance();
+        zc ^= 1;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last two steps' loads ran ahead of the range
+    gemm_tail<MI>(acc, Y, M, N, m0, n0, epi, part, counters);
 }
 
 constexpr int GEMM_COUNTER_BYTES = 65536;  // start of the workspace: one uint32 per output tile
 
 template <int MI>
 static hipError_t launch_mi(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int gshift,
-                            Epilogue epi, void* ws, int ksplit, hipStream_t st) {
+                            Epilogue epi, void* ws, int ksplit, bool lds, hipStream_t st) {
     const dim3 grid((N + GEMM_BN - 1) / GEMM_BN, (M + 32 * MI - 1) / (32 * MI), ksplit);
     unsigned* counters = (unsigned*)ws;
     float* part = ws ? (float*)((char*)ws + GEMM_COUNTER_BYTES) : nullptr;
+    if (lds && gshift == 7 && K % 256 == 0) {
+        hipLaunchKernelGGL((gemm_lds_kernel<MI>), grid, dim3(256), 0, st, (const uint8_t*)w, (const half2_t*)zs,
+                           (const half_t*)x, (half_t*)y, M, N, K, epi, part, counters);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL((gemm_kernel<MI>), grid, dim3(256), 0, st, (const uint8_t*)w, (const half2_t*)zs,
                        (const half_t*)x, (half_t*)y, M, N, K, gshift, epi, part, counters);
     return hipGetLastError();
@@ -277,14 +488,48 @@ static hipError_t launch_mi(const void* x, const void* w, const void* zs, void* 
 // unsplit).  `pipe` receives the pipelined variant to use instead (-1 = none).
 struct GemmPlan {
     int mi, ksplit, pipe;
+    int lds = 0;  // 1: gemm_lds_kernel (group size 128, K a multiple of 256)
 };
-static GemmPlan plan_gemm(int M, int N, int K, bool have_ws) {
+// Group size 128 with K a multiple of 256 and more than 32 tokens: gemm_lds_kernel, whose choices
+// come from a sweep of tile height x split over 4096 x 4096, 16384 x 4096, 4096 x 16384,
+// 11008 x 4096, 4096 x 11008 and 12288 x 4096 at 48..4096 tokens (within a few percent of the best
+// swept configuration on all of them): 32-row tiles up to 64 tokens on narrow weights (up to 128
+// when K is short as well), 128-row tiles beyond 256 tokens when the weight is wide or K long and
+// always beyond 1024, 64-row tiles between; K split while the grid stays within one round of 256
+// workgroups and every part keeps 8 steps.  Only a long K whose 256 x 256 tiles fill whole rounds
+// stays with the pipelined kernel (4096 x 16384 at 4096 tokens: 497 against 530 us).
+static GemmPlan plan_gemm_lds(int M, long ncol, int nit, bool have_ws) {
+    GemmPlan p = {1, 1, -1};
+    const long t256 = ncol * ((M + 255) / 256);
+    const long rounds = (t256 + 255) / 256;
+    if (M > 1024 && nit >= 128 && t256 * 10 >= rounds * 256 * 9) {
+        p.pipe = 2;
+        return p;
+    }
+    p.lds = 1;
+    const bool wide_or_long = ncol >= 32 || nit >= 128;
+    if (M <= 64)
+        p.mi = ncol >= 32 ? 2 : 1;
+    else if (M <= 128)
+        p.mi = wide_or_long ? 2 : 1;
+    else if (M <= 256)
+        p.mi = 2;
+    else
+        p.mi = (wide_or_long || M > 1024) ? 4 : 2;
+    const long t = ncol * ((M + 32 * p.mi - 1) / (32 * p.mi));
+    if (have_ws && t <= 16384)
+        while (p.ksplit < 8 && t * p.ksplit * 2 <= 256 && nit / (p.ksplit * 2) >= 8) p.ksplit *= 2;
+    return p;
+}
+
+static GemmPlan plan_gemm(int M, int N, int K, int g, bool have_ws) {
     GemmPlan p = {1, 1, -1};
     const long ncol = (N + 255) / 256;
     auto ntiles = [&](int rows) { return ncol * ((M + rows - 1) / rows); };
     const long t256 = ntiles(256);
     const long rounds = (t256 + 255) / 256;
     const int nit = (K + GEMM_BK - 1) / GEMM_BK;
+    if (g == 128 && K % 256 == 0 && M > 32) return plan_gemm_lds(M, ncol, nit, have_ws);
     if (M > 64 && t256 * 10 >= rounds * 256 * 6) {
         p.pipe = 2;  // 256 x 256 tiles pay from about 60 % of the CUs (5120 x 13696 at M = 2048: 338 us against 390 us)
     } else if (M > 64 && ntiles(128) >= 160) {
@@ -307,29 +552,37 @@ static GemmPlan plan_gemm(int M, int N, int K, bool have_ws) {
     return p;
 }
 
-size_t gemm_workspace_bytes(int M, int N, int K) {
-    const GemmPlan p = plan_gemm(M, N, K, true);
+static size_t plan_bytes(const GemmPlan& p, int M, int N) {
     if (p.ksplit == 1) return 0;
     const long tiles = (long)((N + 255) / 256) * ((M + 32 * p.mi - 1) / (32 * p.mi));
     return (size_t)GEMM_COUNTER_BYTES + (size_t)p.ksplit * tiles * (32 * p.mi) * 256 * sizeof(float);
 }
 
+// The query does not know the group size: the larger of what the two planners would use.
+size_t gemm_workspace_bytes(int M, int N, int K) {
+    const size_t a = plan_bytes(plan_gemm(M, N, K, 128, true), M, N);
+    const size_t b = plan_bytes(plan_gemm(M, N, K, 0, true), M, N);
+    return a > b ? a : b;
+}
+
 // tune = 0 for the heuristic, else the number of 32-row tiles per workgroup (1, 2 or 4) | ksplit << 8
-// (needs ws), or 8 / 9 / 10 for the software-pipelined kernel (128 rows at two waves per SIMD, 128 rows
+// (needs ws) | 0x80 for the kernel with both operands through LDS (group size 128, K % 256 == 0), or 8 / 9 / 10 for the software-pipelined kernel (128 rows at two waves per SIMD, 128 rows
 // at one, 256 rows at one).  ws = null or too small: K is never split.
 hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, size_t ws_bytes, int M,
                              int N, int K, int g, int tune, Epilogue epi, hipStream_t st) {
     int gshift = 0;
     while ((1 << gshift) < g) gshift++;
-    int mi = tune & 0xFF;
+    int mi = tune & 0x3F;
     int ksplit = (tune >> 8) & 0xFF;
+    bool lds = (tune & 0x80) != 0;
     if (mi >= 8 && mi <= 10) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, mi - 8, epi, st);
     if (mi != 1 && mi != 2 && mi != 4) {
-        const bool have_ws = ws != nullptr && ws_bytes >= gemm_workspace_bytes(M, N, K);
-        const GemmPlan p = plan_gemm(M, N, K, have_ws);
+        const bool have_ws = ws != nullptr && ws_bytes >= plan_bytes(plan_gemm(M, N, K, g, true), M, N);
+        const GemmPlan p = plan_gemm(M, N, K, g, have_ws);
         if (p.pipe >= 0) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, p.pipe, epi, st);
         mi = p.mi;
         ksplit = p.ksplit;
+        lds = p.lds != 0;
     } else {
         if (ksplit != 2 && ksplit != 4 && ksplit != 8) ksplit = 1;
         const long tiles = (long)((N + 255) / 256) * ((M + 32 * mi - 1) / (32 * mi));
@@ -337,9 +590,9 @@ hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void*
         if (ksplit > 1 && (!ws || ws_bytes < need || tiles > 16384)) ksplit = 1;
     }
     switch (mi) {
-        case 1: return launch_mi<1>(x, w, zs, y, M, N, K, gshift, epi, ws, ksplit, st);
-        case 2: return launch_mi<2>(x, w, zs, y, M, N, K, gshift, epi, ws, ksplit, st);
-        default: return launch_mi<4>(x, w, zs, y, M, N, K, gshift, epi, ws, ksplit, st);
+        case 1: return launch_mi<1>(x, w, zs, y, M, N, K, gshift, epi, ws, ksplit, lds, st);
+        case 2: return launch_mi<2>(x, w, zs, y, M, N, K, gshift, epi, ws, ksplit, lds, st);
+        default: return launch_mi<4>(x, w, zs, y, M, N, K, gshift, epi, ws, ksplit, lds, st);
     }
 }
 
