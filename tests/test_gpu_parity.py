@@ -637,6 +637,51 @@ def test_gemm_split_k_every_tile_height(capi, mi, ksplit):
         assert torch.equal(y1, capi.gemm_ws(x, d["w_dev"], d["zs_dev"], n, k, g, algo=algo, ws=ws))
 
 
+@pytest.mark.parametrize("mi", [1, 2, 4])
+@pytest.mark.parametrize("ksplit", [1, 2, 4, 8])
+def test_gemm_operands_through_lds(capi, mi, ksplit):
+    # the tiled kernel whose weights, activations and zeros/scales all reach LDS by direct loads (group size 128,
+    # K a multiple of 256): parity against the oracle on ragged M and N, K = 256 x odd, K ranges of the split that
+    # are padded; bit-identical to the register-staged kernel at the same tile height and split; counters left clean
+    lds = 0x80
+    for (m, n, k) in [(33, 264, 768), (70, 520, 1280), (129, 4096, 4096), (200, 264, 2816), (300, 1000, 11008)]:
+        g = 128
+        d = linear(n, k, g, seed=71)
+        x = to_dev(orc.synth_x(m, k, seed=72))
+        ws = torch.zeros(64 * 1024 * 1024, dtype=torch.uint8, device=DEV)
+        tune = mi | (ksplit << 8)
+        y_lds = capi.gemm_ws(x, d["w_dev"], d["zs_dev"], n, k, g, algo=capi.SQ_ALGO_GEMM | ((tune | lds) << 8), ws=ws)
+        y_ref = orc.gemm_ref(x.cpu().numpy(), d["w_hat"])
+        assert np.max(np.abs(y_lds.float().cpu().numpy() - y_ref)) <= TOL * np.max(np.abs(y_ref)), (m, n, k)
+        assert torch.count_nonzero(ws[:65536]).item() == 0
+        if ksplit == 1:  # the split ranges of the two kernels differ (whole groups of four steps here)
+            y_reg = capi.gemm_ws(x, d["w_dev"], d["zs_dev"], n, k, g, algo=capi.SQ_ALGO_GEMM | (tune << 8), ws=ws)
+            assert torch.equal(y_lds, y_reg), (m, n, k)
+        assert torch.equal(y_lds, capi.gemm_ws(x, d["w_dev"], d["zs_dev"], n, k, g,
+                                               algo=capi.SQ_ALGO_GEMM | ((tune | lds) << 8), ws=ws))
+
+
+def test_gemm_lds_request_falls_back_where_it_does_not_apply(capi):
+    # other group sizes and a K that is no multiple of 256 run the register-staged kernel under the same request
+    for (m, n, k, g) in [(70, 264, 704, 64), (100, 520, 1056, 32), (65, 264, 640, 128)]:
+        check_gemm(capi, m, n, k, g, capi.SQ_ALGO_GEMM | ((2 | 0x80) << 8))
+
+
+@pytest.mark.parametrize("m", [33, 64, 100, 256, 1000, 2048])
+def test_gemm_lds_fused_epilogue(capi, m):
+    # bias, ReLU and residual through the automatic choice at group size 128 (the LDS kernel, K split for small m)
+    n, k, g = 1000, 2816, 128
+    d = linear(n, k, g, seed=81)
+    rng = np.random.default_rng(82)
+    x = orc.synth_x(m, k, seed=83)
+    bias = rng.normal(0, 2.0, size=n).astype(np.float16)
+    res = rng.normal(0, 2.0, size=(m, n)).astype(np.float16)
+    y = capi.gemm_fused(to_dev(x), d["w_dev"], d["zs_dev"], n, k, g, bias=to_dev(bias), residual=to_dev(res), act=1)
+    y_ref = fused_ref(x, d["w_hat"], bias, res, 1)
+    scale = np.max(np.abs(orc.gemm_ref(x, d["w_hat"])))
+    assert np.max(np.abs(y.float().cpu().numpy() - y_ref)) <= TOL * scale
+
+
 def test_mfma_probe_reports_one_instruction_per_32_cycles(capi):
     data = torch.randn(5120, device=DEV).half()
     ticks = capi.mfma_probe(data, 4, 2000)
