@@ -579,11 +579,12 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
             del wd
     tf = flops_total / time_total / 1e6
     tfd = flops_total / dense_time_total / 1e6
-    # the other two token counts of the same configuration, aggregate only
+    # other token counts of the same configuration (64..1024: the range between decode and prefill), aggregate
+    # and per-linear time
     other = {}
     torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
     with torch.cuda.stream(stream):
-        for m2 in (512, 4096):
+        for m2 in (64, 128, 256, 512, 1024, 4096):
             fl2, t2 = 0.0, 0.0
             per = {}
             for w, zs, name, n, k in work:

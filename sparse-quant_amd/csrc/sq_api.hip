@@ -106,11 +106,10 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
         const bool stream_ok = (M > 4 || (M >= 3 && large)) && M <= 16 && (group_size == 128 || group_size == 64) &&
                                K % 128 == 0 &&
                                (K <= 4096 || (ws_ok && K <= 32768));
-        // 17..32 tokens at group size 128: the two-tile variant of the streaming kernel where 64-row blocks fill
-        // at least half the chip (fc1 at 32 tokens 15.8 against 17.9 us, q/k/v 13.3 against 15.6, fc2 17.3 against 19.1)
-        const int wide_ksplit = (K / 128 + 31) / 32;
-        const bool wide_ok = M > 16 && M <= 32 && group_size == 128 && K % 128 == 0 && wide_ksplit <= 8 &&
-                             (wide_ksplit == 1 || ws_ok) && (long)((N + 63) / 64) * wide_ksplit >= 128;
+        // 17..32 tokens at group size 128: the two-tile variant of the streaming kernel where 64-row blocks (times the
+        // K split) fill at least half the chip (fc1 at 32 tokens 16.5 against 17.2 us, q/k/v-sized 14.3 against 15.5,
+        // fc2 18.1 against 19.0)
+        const bool wide_ok = M > 16 && M <= 32 && group_size == 128 && sq::skinny3_wide_applies(N, K, ws_ok);
         // more than 32 tokens at group size 128: the tiled kernel with both operands through LDS and K split
         // through the workspace (4096 x 4096 at 48 tokens 14.5 us against 17.2 for two blocks of the split-K
         // decode kernel, fc1 24.7 against 28.2, fc2 27.0 against 32.3; at 64 tokens 14.5 against 20.5 for the

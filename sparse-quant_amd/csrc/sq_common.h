@@ -168,6 +168,18 @@ __device__ __forceinline__ void load8_coherent_x4(const float* const (&p)[8], fl
         : "memory");
 }
 
+// One direct global -> LDS load: 16 (or 4) bytes per lane, lane l lands at lds_byte + 16 (4) * l.
+// Written as inline assembly on purpose: the compiler, when it knows of such a load, makes every
+// later LDS read wait for ALL outstanding vector memory loads unless it can prove the two apart,
+// which it cannot for stages picked at run time.  The kernel orders them itself (a counted
+// s_waitcnt and a barrier per step); the "memory" clobbers keep LDS reads from moving across.
+__device__ __forceinline__ void load_to_lds_x4(const void* g, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte) : "memory");
+}
+__device__ __forceinline__ void load_to_lds_x1(const void* g, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_byte) : "memory");
+}
+
 // Sixteen coherent 128-bit loads in flight: p[i] points at the SECOND of two locations 4096 bytes
 // apart (v[2i] = p[i][-4096 bytes], v[2i+1] = p[i][0]); one asm block with its own wait, so that no
 // register holding a result can be touched before the data is there.

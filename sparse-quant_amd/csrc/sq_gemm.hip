@@ -287,18 +287,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     gemm_tail<MI>(acc, Y, M, N, m0, n0, epi, part, counters);
 }
 
-// One direct global -> LDS load: 16 (or 4) bytes per lane, lane l lands at lds_byte + 16 (4) * l.
-// Written as inline assembly on purpose: the compiler, when it knows of such a load, makes every
-// later LDS read wait for ALL outstanding vector memory loads unless it can prove the two apart,
-// which it cannot for stages picked at run time.  The kernel orders them itself (a counted
-// s_waitcnt and a barrier per step); the "memory" clobbers keep LDS reads from moving across.
-__device__ __forceinline__ void load_to_lds_x4(const void* g, uint32_t lds_byte) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte) : "memory");
-}
-__device__ __forceinline__ void load_to_lds_x1(const void* g, uint32_t lds_byte) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_byte) : "memory");
-}
-
 // Both operands through LDS, for group size 128 and K a multiple of 256.  The kernels above hand
 // every lane its own 16 bytes of a weight row (32 rows per wave-wide load) and 4 bytes of
 // zeros/scales, and the L1 takes lanes that are not neighbours in memory one at a time: about 1240

@@ -73,6 +73,7 @@ hipError_t launch_skinny3_group(const SeqProblem* probs, int count, int M, void*
 // The same kernel family for 17..32 tokens (two token tiles, activations staged in two halves); group size 128 only.
 hipError_t launch_skinny3_wide(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                                Epilogue epi, hipStream_t st);
+bool skinny3_wide_applies(int N, int K, bool have_ws);
 hipError_t launch_skinny3_wide_group(const SeqProblem* probs, int count, int M, void* ws, size_t ws_bytes,
                                      hipStream_t st);
 // sq_gemm.hip: any M.  tune = 32-row tiles per workgroup (1,2,4) | ksplit << 8; ws may be null.

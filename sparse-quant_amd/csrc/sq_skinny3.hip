@@ -384,44 +384,65 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     if (tid == 0) __hip_atomic_store(&counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// ---- 17..32 tokens ------------------------------------------------------------------------------------------
-// Two token tiles per matrix-instruction operand (every unpacked weight word meets both), group size 128, 64 weight
-// rows and a K range of up to 4096 columns per workgroup.  32 tokens x 4096 columns of activations are 256 KiB, so
-// they are staged in two halves of 2048 columns (sixteen chunk slots): the second half waits in registers, requested
-// right after the first is parked, while the first half's chunks are consumed; one pair of barriers swaps it in.
-// The weight stream does not stop for that: the unit that follows the swap is requested before it.
+// 17..32 tokens: two token tiles per operand (every unpacked weight word meets both), 64-row workgroups, a wave owns
+// the same four chunk slots as above.  A wave needs the activations of ITS chunks only (32 tokens x 256 bytes per
+// chunk), so nothing about them is shared: each wave moves them global -> LDS itself with direct loads (no
+// registers, no workgroup barrier) through a private ring of two chunks, the third and fourth chunk requested as
+// soon as the first and second are consumed.  The row of a token is stored with its sixteen 16-byte pieces XORed by
+// the token index, which makes the 128-bit operand reads (lane = token) conflict-free.  All sixteen weight words of
+// the wave are requested at the start, in the order of use and interleaved with the activation chunks, and every
+// wait names the number of younger requests that may stay in flight (the vector memory counter retires in order).
+// The loads are inline assembly: the compiler then inserts no waits of its own, which could only be conservative
+// here (it cannot see the direct loads).  A timeline of the previous form (activations staged by the whole
+// workgroup in two halves through registers) showed 12 of its 15.5 us waiting: 1.9 us to issue the first half's
+// requests (a CU takes a few dozen wave-wide requests at a time), 4 us from the first barrier to the end of the first
+// unit (the second half's requests had to be issued before its arithmetic could start), 1.5 us for the swap.
+//
+// RT row tiles per workgroup and CH chunk slots per wave (a workgroup covers 8 CH chunks of K); launched with 4 and 4.
+template <int RT, int CH>
 struct Sk3WideLds {
-    static constexpr int PSLOTS = 16;                    // chunk slots per half
-    static constexpr int XPITCH = PSLOTS * 256 + 16;     // bytes per staged token row (16 mod 256)
-    static constexpr int X_BYTES = 32 * XPITCH;
-    static constexpr int TILE = 4 * 2 * 4 * 64;          // floats a wave contributes: [rt][mt][v][lane]
-    static constexpr int RED_BYTES = SK3_NWV * TILE * 4;
-    static constexpr int Z_OFF = X_BYTES > RED_BYTES ? X_BYTES : RED_BYTES;
-    static constexpr int ZPITCH = 33;
-    static constexpr int FLAG_OFF = Z_OFF + 64 * ZPITCH * 4;
+    static constexpr int XSLOT = 32 * 256;               // one chunk of 32 tokens
+    static constexpr int XWAVE = 2 * XSLOT;              // a wave's ring
+    static constexpr int TILE = RT * 2 * 4 * 64;         // floats a wave contributes: [rt][mt][v][lane]; they overwrite its ring
+    static constexpr int ZCOLS = 8 * CH;                 // chunk slots of a workgroup
+    static constexpr int Z_OFF = SK3_NWV * XWAVE;        // zeros/scales of the row block: 16 RT rows x ZCOLS
+    static constexpr int FLAG_OFF = Z_OFF + 16 * RT * ZCOLS * 4;
     static constexpr int BYTES = FLAG_OFF + 16;
 };
 
+// Wait until at most N younger requests are outstanding.  Names a chunk's weight words, so that no use of them can be
+// scheduled ahead of the wait (they are loaded by inline assembly: the compiler does not know they arrive later).
+template <int N, int RT>
+__device__ __forceinline__ void sk3_wait_words(u32x4_t (&w)[RT]) {
+    static_assert(RT == 4 || RT == 8, "row tiles per workgroup");
+    if constexpr (RT == 4)
+        asm volatile("s_waitcnt vmcnt(%4)" : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]) : "n"(N) : "memory");
+    else
+        asm volatile("s_waitcnt vmcnt(%8)"
+                     : "+v"(w[0]), "+v"(w[1]), "+v"(w[2]), "+v"(w[3]), "+v"(w[4]), "+v"(w[5]), "+v"(w[6]), "+v"(w[7])
+                     : "n"(N)
+                     : "memory");
+}
+
+template <int RT, int CH>
 __device__ __forceinline__ void skinny3_wide_body(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ZS,
                                                   const half_t* __restrict__ X, half_t* __restrict__ Y, float* part,
                                                   unsigned* counters, int M, int N, int K, int ksplit,
                                                   const Epilogue& epi, int rb, int slot, int nslots) {
-    using L = Sk3WideLds;
-    constexpr int RT = 4, MT = 2, CH = 4, ROWS = 64, TILE = L::TILE;
-    constexpr int WPR = L::PSLOTS * 16;              // 128-bit words per staged token row and half
-    constexpr int XPT = 32 * WPR / SK3_NT;           // 16
-    constexpr int ZPT = ROWS * 32 / SK3_NT;          // 4
+    using L = Sk3WideLds<RT, CH>;
+    constexpr int MT = 2, ROWS = 16 * RT, TILE = L::TILE, ZC = L::ZCOLS;
+    static_assert(CH == 2 || CH == 4, "chunk slots per wave");
+    static_assert(L::XWAVE >= TILE * 4, "a wave's partial tile fits its ring");
 
     extern __shared__ __attribute__((aligned(16))) uint8_t sk3_lds[];
-    uint8_t* xl = sk3_lds;
-    uint32_t* zsl = (uint32_t*)(sk3_lds + L::Z_OFF);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)sk3_lds;
+    const uint32_t* zsl = (const uint32_t*)(sk3_lds + L::Z_OFF);
     unsigned* last_flag = (unsigned*)(sk3_lds + L::FLAG_OFF);
-    float* red = (float*)sk3_lds;
 
     const NibbleMasks nm = nibble_masks();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int li = lane & 15;
     const int lj = lane >> 4;
     const int ks = blockIdx.y;
@@ -433,71 +454,60 @@ __device__ __forceinline__ void skinny3_wide_body(const uint8_t* __restrict__ W,
         nc = 0;
         c_begin = 0;
     }
+    uint8_t* xw = sk3_lds + wave * L::XWAVE;
+    const uint32_t xw0 = lds0 + wave * L::XWAVE;
 
-    uint32_t zreg[ZPT];
+    // chunk slots of this wave; one past the range reads chunk c_begin and gets scale 0
+    int cl[CH], cg[CH];
 #pragma unroll
-    for (int p = 0; p < ZPT; p++) {
-        const int idx = tid + p * SK3_NT;
-        const int r = idx >> 5, col = idx & 31;
-        const int row = imin(rb * ROWS + r, N - 1);
-        zreg[p] = ZS[(long)row * chunks + c_begin + (col < nc ? col : 0)];
+    for (int u = 0; u < CH; u++) {
+        cl[u] = 2 * (wave + SK3_NWV * (u >> 1)) + (u & 1);
+        cg[u] = c_begin + (cl[u] < nc ? cl[u] : 0);
     }
-    // one half of the activations: token idx / 256, 128-bit column idx % 256 of the half
-    auto load_x = [&](int half, u32x4_t (&xr)[XPT]) {
+    // Instruction i of a chunk moves tokens 4 i .. 4 i + 3: lane l fetches, for ring position l % 16 of token
+    // 4 i + l / 16, the piece (l % 16) ^ (token % 16).  Tokens past M re-read the last one (never stored).
+    const half_t* xrow[8];
 #pragma unroll
-        for (int p = 0; p < XPT; p++) {
-            const int idx = tid + p * SK3_NT;
-            const int m = idx / WPR, col = half * WPR + idx % WPR;
-            const bool ok = (m < M) && (col < nc * 16);
-            const uint32_t keep = ok ? 0xffffffffu : 0u;
-            const u32x4_t v = *(const u32x4_t*)(X + (ok ? (long)m * K + c_begin * 128 + col * 8 : 0));
-            xr[p] = (u32x4_t){v.x & keep, v.y & keep, v.z & keep, v.w & keep};
-        }
+    for (int i = 0; i < 8; i++) {
+        const int t = 4 * i + lj;
+        xrow[i] = X + (long)imin(t, M - 1) * K + ((li ^ (t & 15)) * 8);
+    }
+    auto dma_x = [&](int u) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) load_to_lds_x4(xrow[i] + (long)cg[u] * 128, xw0 + (u & 1) * L::XSLOT + i * 1024);
     };
-    auto park_x = [&](const u32x4_t (&xr)[XPT]) {
-#pragma unroll
-        for (int p = 0; p < XPT; p++) {
-            const int idx = tid + p * SK3_NT;
-            *(u32x4_t*)(xl + (idx / WPR) * L::XPITCH + (idx % WPR) * 16) = xr[p];
-        }
-    };
-    u32x4_t xr[XPT];
-    load_x(0, xr);
-    __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_barrier" ::: "memory");  // every wave's activation requests precede every weight request
-    __builtin_amdgcn_sched_barrier(0);
-
-    // weight units: (chunk pair pr = half, row tiles 2 rg, 2 rg + 1) x the two 64-byte halves of a line
-    u32x4_t wq[CH][RT];
-    int slot_of[CH];
-#pragma unroll
-    for (int u = 0; u < CH; u++) slot_of[u] = 2 * (wave + SK3_NWV * (u >> 1)) + (u & 1);
     const uint8_t* wrow[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) wrow[rt] = W + (long)imin(rb * ROWS + 16 * rt + li, N - 1) * (K >> 1) + lj * 16;
-    auto issue_unit = [&](int un) {
-        const int pr = un >> 1, rg = un & 1;
+    u32x4_t wq[CH][RT];
+    auto load_w = [&](int u) {
 #pragma unroll
-        for (int r = 0; r < 2; r++)
-#pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const int cl = slot_of[2 * pr + h];
-                wq[2 * pr + h][2 * rg + r] = *(const u32x4_t*)(wrow[2 * rg + r] + (long)(c_begin + (cl < nc ? cl : 0)) * 64);
-            }
+        for (int rt = 0; rt < RT; rt++)
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(wq[u][rt]) : "v"(wrow[rt] + (long)cg[u] * 64) : "memory");
     };
-    issue_unit(0);
-    __builtin_amdgcn_sched_barrier(0);
+    // zeros/scales of the row block, by the whole workgroup: ZQ instructions per wave, 64 consecutive (row, chunk
+    // slot) pairs each
+    constexpr int ZQ = RT * CH / 4;
 #pragma unroll
-    for (int p = 0; p < ZPT; p++) {
-        const int idx = tid + p * SK3_NT;
-        zsl[(idx >> 5) * L::ZPITCH + (idx & 31)] = zreg[p];
+    for (int q = 0; q < ZQ; q++) {
+        const int idx = (wave * ZQ + q) * 64 + lane;
+        const int r = idx / ZC, col = idx % ZC;
+        const int row = imin(rb * ROWS + r, N - 1);
+        load_to_lds_x1(ZS + (long)row * chunks + c_begin + (col < nc ? col : 0), lds0 + L::Z_OFF + (wave * ZQ + q) * 256);
     }
-    park_x(xr);
-    sk3_barrier();
-    issue_unit(1);  // ahead of the second half's activation requests, so that the weight stream does not pause for them
-    __builtin_amdgcn_sched_barrier(0);
-    load_x(1, xr);  // the second half waits in registers while the first is consumed
-    __builtin_amdgcn_sched_barrier(0);
+    dma_x(0);
+    load_w(0);
+    // The one thing the waves share are the zeros/scales: meet as soon as they have landed (the twelve requests
+    // behind them stay in flight), before the bulk of the requests is issued.  Issuing takes a wave 2..8 us here
+    // (a CU takes a few dozen wave-wide requests at a time); with the barrier behind all of it every wave would
+    // start its arithmetic when the slowest has finished issuing.
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(8 + RT) : "memory");
+    dma_x(1);
+    load_w(1);
+    if constexpr (CH == 4) {
+        load_w(2);
+        load_w(3);
+    }
 
     float4_t acc[RT][MT];
 #pragma unroll
@@ -508,75 +518,83 @@ __device__ __forceinline__ void skinny3_wide_body(const uint8_t* __restrict__ W,
                           (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
     const half8_t m960 = {(half_t)-960.f, (half_t)-960.f, (half_t)0.f, (half_t)0.f,
                           (half_t)-960.f, (half_t)-960.f, (half_t)0.f, (half_t)0.f};
-    const uint8_t* xrd = xl + li * L::XPITCH + lj * 64;
+
+    auto consume = [&](int u) {
+        const uint8_t* xs = xw + (u & 1) * L::XSLOT + li * 256;
+        const bool valid = cl[u] < nc;
+        const int zcol = valid ? cl[u] : 0;
+        half8_t xa[MT][4];
+        float4_t xsum[MT], x960[MT];
 #pragma unroll
-    for (int un = 0; un < 4; un++) {
-        if (un == 2) {  // swap the second half of the activations in
-            sk3_barrier();
-            park_x(xr);
-            sk3_barrier();
-        }
-        if (un > 0 && un + 1 < 4) {
-            issue_unit(un + 1);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        const int pr = un >> 1, rg = un & 1;
+        for (int mt = 0; mt < MT; mt++) {
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const int u = 2 * pr + h;
-            const int cl = slot_of[u];
-            const int zcol = cl < nc ? cl : 0;
-            half8_t xa[MT][4];
-            float4_t xsum[MT], x960[MT];
+            for (int t = 0; t < 4; t++) xa[mt][t] = *(const half8_t*)(xs + 16 * mt * 256 + (((4 * lj + t) ^ li) * 16));
+            xsum[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+            x960[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                xsum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][t], ones, xsum[mt], 0, 0, 0);
+                x960[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][t], m960, x960[mt], 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            const half2_t zsv = bit_cast<half2_t>(zsl[(16 * rt + li) * ZC + zcol]);
+            const float zf = (float)zsv.x;
+            const float sf = valid ? (float)zsv.y : 0.f;
+            half8_t wv[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) wv[t] = unpack8_mixed(wq[u][rt][t], nm);
 #pragma unroll
             for (int mt = 0; mt < MT; mt++) {
+                float4_t tmp = x960[mt];
 #pragma unroll
-                for (int t = 0; t < 4; t++)
-                    xa[mt][t] = *(const half8_t*)(xrd + 16 * mt * L::XPITCH + (cl - L::PSLOTS * pr) * 256 + 16 * t);
-                xsum[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
-                x960[mt] = (float4_t){0.f, 0.f, 0.f, 0.f};
+                for (int t = 0; t < 4; t++) tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][t], wv[t], tmp, 0, 0, 0);
 #pragma unroll
-                for (int t = 0; t < 4; t++) {
-                    xsum[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][t], ones, xsum[mt], 0, 0, 0);
-                    x960[mt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][t], m960, x960[mt], 0, 0, 0);
-                }
-            }
-#pragma unroll
-            for (int r = 0; r < 2; r++) {
-                const int rt = 2 * rg + r;
-                const half2_t zsv = bit_cast<half2_t>(zsl[(16 * rt + li) * L::ZPITCH + zcol]);
-                const float zf = (float)zsv.x;
-                const float sf = (float)zsv.y;
-                half8_t wv[4];
-#pragma unroll
-                for (int t = 0; t < 4; t++) wv[t] = unpack8_mixed(wq[u][rt][t], nm);
-#pragma unroll
-                for (int mt = 0; mt < MT; mt++) {
-                    float4_t tmp = x960[mt];
-#pragma unroll
-                    for (int t = 0; t < 4; t++) tmp = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt][t], wv[t], tmp, 0, 0, 0);
-#pragma unroll
-                    for (int v = 0; v < 4; v++) acc[rt][mt][v] += sf * (tmp[v] - zf * xsum[mt][v]);
-                }
+                for (int v = 0; v < 4; v++) acc[rt][mt][v] += sf * (tmp[v] - zf * xsum[mt][v]);
             }
         }
-    }
-    sk3_barrier();  // every wave is done with the activations, which the partials now overwrite
+    };
 
+    if constexpr (CH == 4) {
+        // requests so far, oldest first: zeros/scales, x0 8, w0 RT, x1 8, w1 RT, w2 RT, w3 RT
+        sk3_wait_words<8 + 3 * RT>(wq[0]);  // x0, w0 are there
+        consume(0);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // ring position 0 has been read
+        dma_x(2);
+        sk3_wait_words<8 + 2 * RT>(wq[1]);  // x1, w1 (w2, w3, x2 may be outstanding)
+        consume(1);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        dma_x(3);
+        sk3_wait_words<8>(wq[2]);  // w2, w3, x2 (x3 may be outstanding)
+        consume(2);
+        sk3_wait_words<0>(wq[3]);
+        consume(3);
+    } else {
+        // zeros/scales, x0 8, w0 RT, x1 8, w1 RT: both chunks fit the ring
+        sk3_wait_words<8 + RT>(wq[0]);
+        consume(0);
+        sk3_wait_words<0>(wq[1]);
+        consume(1);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's ring is free: its partial tile goes there
+
+    float* mine_lds = (float*)xw;
 #pragma unroll
     for (int rt = 0; rt < RT; rt++)
 #pragma unroll
         for (int mt = 0; mt < MT; mt++)
 #pragma unroll
-            for (int v = 0; v < 4; v++) red[wave * TILE + ((rt * MT + mt) * 4 + v) * 64 + lane] = acc[rt][mt][v];
+            for (int v = 0; v < 4; v++) mine_lds[((rt * MT + mt) * 4 + v) * 64 + lane] = acc[rt][mt][v];
     sk3_barrier();
+    auto red = [&](int p, int t) -> const float* { return (const float*)(sk3_lds + p * L::XWAVE) + t; };
 
     // Element t of the tile: lane l = t % 64, v, mt, rt -> token m = 16 mt + 4 (l / 16) + v, row n = 64 rb + 16 rt + l % 16.
     if (ksplit == 1) {
         for (int t = tid; t < TILE; t += SK3_NT) {
             float sum = 0.f;
 #pragma unroll
-            for (int p = 0; p < SK3_NWV; p++) sum += red[p * TILE + t];
+            for (int p = 0; p < SK3_NWV; p++) sum += *red(p, t);
             const int l = t & 63, v = (t >> 6) & 3, mt = (t >> 8) % MT, rt = (t >> 8) / MT;
             const int m = 16 * mt + 4 * (l >> 4) + v;
             const int n = rb * ROWS + 16 * rt + (l & 15);
@@ -588,7 +606,7 @@ __device__ __forceinline__ void skinny3_wide_body(const uint8_t* __restrict__ W,
     for (int t4 = tid * 4; t4 < TILE; t4 += 4 * SK3_NT) {
         float4_t sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int p = 0; p < SK3_NWV; p++) sum += *(const float4_t*)(&red[p * TILE + t4]);
+        for (int p = 0; p < SK3_NWV; p++) sum += *(const float4_t*)red(p, t4);
         store_coherent_x4(mine + t4, sum);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -621,11 +639,12 @@ __device__ __forceinline__ void skinny3_wide_body(const uint8_t* __restrict__ W,
     if (tid == 0) __hip_atomic_store(&counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+template <int RT, int CH>
 __global__ __launch_bounds__(SK3_NT) void skinny3_wide_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ ZS,
                                                               const half_t* __restrict__ X, half_t* __restrict__ Y,
                                                               float* part, unsigned* counters, int M, int N, int K,
                                                               int ksplit, Epilogue epi) {
-    skinny3_wide_body(W, ZS, X, Y, part, counters, M, N, K, ksplit, epi, blockIdx.x, blockIdx.x, gridDim.x);
+    skinny3_wide_body<RT, CH>(W, ZS, X, Y, part, counters, M, N, K, ksplit, epi, blockIdx.x, blockIdx.x, gridDim.x);
 }
 
 template <int MROWS, int RT, int CH, bool LN, int GPC>
@@ -663,6 +682,7 @@ __global__ __launch_bounds__(SK3_NT) void skinny3_group_kernel(const Skinny3Grou
                                                   ksplit, epi, LnPre{nullptr, nullptr, 0.f}, rb, blockIdx.x, gridDim.x);
 }
 
+template <int RT, int CH>
 __global__ __launch_bounds__(SK3_NT) void skinny3_wide_group_kernel(const Skinny3Group grp, float* part,
                                                                     unsigned* counters, int M, int K, int ksplit) {
     int p = 0;
@@ -671,8 +691,8 @@ __global__ __launch_bounds__(SK3_NT) void skinny3_wide_group_kernel(const Skinny
         if (q + 1 < grp.count && (int)blockIdx.x >= grp.blk_end[q]) p = q + 1;
     const int rb = blockIdx.x - (p > 0 ? grp.blk_end[p - 1] : 0);
     const Epilogue epi{grp.bias[p], grp.residual[p], grp.act[p]};
-    skinny3_wide_body(grp.W[p], grp.ZS[p], grp.X[p], grp.Y[p], part, counters, M, grp.N[p], K, ksplit, epi, rb, blockIdx.x,
-                      gridDim.x);
+    skinny3_wide_body<RT, CH>(grp.W[p], grp.ZS[p], grp.X[p], grp.Y[p], part, counters, M, grp.N[p], K, ksplit, epi, rb,
+                              blockIdx.x, gridDim.x);
 }
 
 template <typename Kern>
@@ -837,17 +857,34 @@ hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, vo
 // 17..32 tokens (any M <= 32 works), group size 128, K % 128 == 0, 64-row workgroups.  hipErrorInvalidValue when the
 // shape does not fit: a K split without a workspace, or so few row blocks that most CUs would idle (the caller then
 // takes the split-K kernel, which splits K further).
+// The two-tile kernel runs 64 rows x 4096 columns per workgroup (RT 4, CH 4); a longer K is split over workgroups
+// through the workspace.  Measured and dropped at 32 tokens: 128 rows x 2048 columns (a third fewer requests per
+// unit of work, but every K is then split: fc1 19.0 against 16.5 us, q/k/v-sized weights 16.8 against 14.3) and
+// 64 rows x 2048 columns (4096 x 4096, where the 4096-column shape has too few workgroups: 10.2 us, the split-K
+// kernel's 10.1).  blocks64 = 64-row blocks of all linears of the launch together.
+static bool wide_fits(long blocks64, int K, bool have_ws, int* ksplit) {
+    if (K <= 0 || K % 128 != 0) return false;
+    const int chunks = K / 128, ks = (chunks + 31) / 32;
+    const int cps = (chunks + ks - 1) / ks;
+    *ksplit = ks;
+    return ks <= 8 && (ks == 1 || have_ws) && (ks - 1) * cps < chunks && blocks64 <= 16384 && blocks64 * ks >= 128;
+}
+
+bool skinny3_wide_applies(int N, int K, bool have_ws) {
+    int ks;
+    return wide_fits((N + 63) / 64, K, have_ws, &ks);
+}
+
+// ws = the caller's workspace or null (then K is never split); it must hold skinny2_workspace_bytes(M, N, K).
 hipError_t launch_skinny3_wide(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                                Epilogue epi, hipStream_t st) {
-    if (M < 1 || M > 32 || K % 128 != 0) return hipErrorInvalidValue;
-    const int chunks = K / 128, ksplit = (chunks + 31) / 32, blocks = (N + 63) / 64;
-    const int cps = (chunks + ksplit - 1) / ksplit;
-    if (ksplit > 8 || (ksplit > 1 && !ws) || (ksplit - 1) * cps >= chunks || blocks > 16384 || blocks * ksplit < 128)
-        return hipErrorInvalidValue;
+    int ksplit;
+    if (M < 1 || M > 32 || !wide_fits((N + 63) / 64, K, ws != nullptr, &ksplit)) return hipErrorInvalidValue;
     static bool allowed[64];
-    const hipError_t e = allow_lds(skinny3_wide_kernel, Sk3WideLds::BYTES, allowed);
+    constexpr int lds = Sk3WideLds<4, 4>::BYTES;
+    const hipError_t e = allow_lds(skinny3_wide_kernel<4, 4>, lds, allowed);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(skinny3_wide_kernel, dim3(blocks, ksplit), dim3(SK3_NT), Sk3WideLds::BYTES, st, (const uint8_t*)w,
+    hipLaunchKernelGGL((skinny3_wide_kernel<4, 4>), dim3((N + 63) / 64, ksplit), dim3(SK3_NT), lds, st, (const uint8_t*)w,
                        (const uint32_t*)zs, (const half_t*)x, (half_t*)y,
                        ws ? (float*)((char*)ws + SK3_COUNTER_BYTES) : nullptr, (unsigned*)ws, M, N, K, ksplit, epi);
     return hipGetLastError();
@@ -857,7 +894,6 @@ hipError_t launch_skinny3_wide_group(const SeqProblem* probs, int count, int M, 
                                      hipStream_t st) {
     if (count < 2 || count > GEMV_GROUP_MAX || M < 1 || M > 32) return hipErrorInvalidValue;
     const int K = probs[0].K;
-    if (K % 128 != 0) return hipErrorInvalidValue;
     Skinny3Group g;
     int blocks = 0;
     for (int p = 0; p < GEMV_GROUP_MAX; p++) {
@@ -875,14 +911,14 @@ hipError_t launch_skinny3_wide_group(const SeqProblem* probs, int count, int M, 
         g.blk_end[p] = blocks;
     }
     g.count = count;
-    const int chunks = K / 128, ksplit = (chunks + 31) / 32;
-    const int cps = (chunks + ksplit - 1) / ksplit;
-    if (ksplit > 8 || (ksplit - 1) * cps >= chunks || blocks > 16384 || blocks * ksplit < 128) return hipErrorInvalidValue;
-    if (ksplit > 1 && (!ws || ws_bytes < skinny2_group_workspace_bytes(probs, count, M))) return hipErrorInvalidValue;
+    const bool have_ws = ws && ws_bytes >= skinny2_group_workspace_bytes(probs, count, M);
+    int ksplit;
+    if (!wide_fits(blocks, K, have_ws, &ksplit)) return hipErrorInvalidValue;
     static bool allowed[64];
-    const hipError_t e = allow_lds(skinny3_wide_group_kernel, Sk3WideLds::BYTES, allowed);
+    constexpr int lds = Sk3WideLds<4, 4>::BYTES;
+    const hipError_t e = allow_lds(skinny3_wide_group_kernel<4, 4>, lds, allowed);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(skinny3_wide_group_kernel, dim3(blocks, ksplit), dim3(SK3_NT), Sk3WideLds::BYTES, st, g,
+    hipLaunchKernelGGL((skinny3_wide_group_kernel<4, 4>), dim3(blocks, ksplit), dim3(SK3_NT), lds, st, g,
                        ws ? (float*)((char*)ws + SK3_COUNTER_BYTES) : nullptr, (unsigned*)ws, M, K, ksplit);
     return hipGetLastError();
 }
