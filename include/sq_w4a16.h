@@ -49,8 +49,9 @@ extern "C" {
 #define SQ_ALGO_GEMM 4           /* any M: LDS-tiled MFMA GEMM */
 #define SQ_ALGO_SKINNY_WS 5      /* M <= 32: 64-row tiles, K split over workgroups through a workspace
                                     (sq_w4a16_gemm_ws only) */
-#define SQ_ALGO_STREAM 6         /* M <= 16, group size 128 or 64: weight loads a fixed distance ahead of the arithmetic,
-                                  * activations staged in LDS first; K beyond 4096 is split through the workspace */
+#define SQ_ALGO_STREAM 6         /* M <= 16 at group size 128 or 64, M <= 32 at group size 128: weight loads a fixed
+                                  * distance ahead of the arithmetic, activations staged in LDS first; K beyond 4096
+                                  * is split through the workspace */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int sq_version(void);
