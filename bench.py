@@ -222,6 +222,8 @@ def main():
                          "sq_w4a16_gemv_sequence")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the M=2048 TFLOP/s leg")
+    ap.add_argument("--prefill-other-tokens", default="64,128,256,512,1024,4096",
+                    help="token counts the prefill leg also measures (comma separated; a counter run names fewer)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the fused-QKV, LUT-attention and end-to-end OPT-6.7B legs")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -485,7 +487,8 @@ def main():
         out["calibration"] = {"kernel": "torch elementwise copy", "bytes_read": 256 << 20, "bytes_written": 256 << 20,
                               "launches": 5}
     if not args.no_prefill:
-        out["prefill"] = prefill_leg(torch, capi, pool[0], shapes, g, dev, gen, stream)
+        other_tokens = tuple(int(t) for t in args.prefill_other_tokens.split(",") if t.strip())
+        out["prefill"] = prefill_leg(torch, capi, pool[0], shapes, g, dev, gen, stream, other_tokens=other_tokens)
     if not args.no_extras:
         # Additional, separately labelled legs; none of them feeds `value`.
         try:
@@ -508,7 +511,7 @@ def main():
     print(json.dumps(out))
 
 
-def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10):
+def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10, other_tokens=(512, 4096)):
     """TFLOP/s of the M=2048 linears of the same layer (the prefill configuration).
 
     Reported beside each figure: the library's dense fp16 GEMM (torch.matmul, no int4 work at all) on
@@ -584,7 +587,7 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
     other = {}
     torch.cuda.synchronize()  # tensors made on the default stream are complete before this stream reads them
     with torch.cuda.stream(stream):
-        for m2 in (64, 128, 256, 512, 1024, 4096):
+        for m2 in other_tokens:
             fl2, t2 = 0.0, 0.0
             per = {}
             for w, zs, name, n, k in work:
