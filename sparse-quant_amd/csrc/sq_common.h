@@ -179,6 +179,16 @@ __device__ __forceinline__ void load_to_lds_x4(const void* g, uint32_t lds_byte)
 __device__ __forceinline__ void load_to_lds_x1(const void* g, uint32_t lds_byte) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_byte) : "memory");
 }
+// The same with the address split into a wave-uniform base and a 32-bit byte offset per lane: a loop that
+// walks along K then advances one scalar instead of one 64-bit sum per lane and load.
+__device__ __forceinline__ void load_to_lds_x4(const void* base, uint32_t lane_byte, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_byte), "s"(base), "s"(lds_byte)
+                 : "memory");
+}
+__device__ __forceinline__ void load_to_lds_x1(const void* base, uint32_t lane_byte, uint32_t lds_byte) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(lane_byte), "s"(base), "s"(lds_byte)
+                 : "memory");
+}
 
 // Sixteen coherent 128-bit loads in flight: p[i] points at the SECOND of two locations 4096 bytes
 // apart (v[2i] = p[i][-4096 bytes], v[2i+1] = p[i][0]); one asm block with its own wait, so that no

@@ -332,23 +332,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     const int it0 = blockIdx.z * spz;
     const int it1 = imin(it0 + spz, nit);
 
-    const half_t* xsrc[MI];
-    int xchunk[MI];
+    // Every address is a wave-uniform base that walks along K plus a byte offset per lane that never changes
+    // (the launcher keeps operands whose offsets would not fit 32 bits away from this kernel).
+    uint32_t xlane[MI];
 #pragma unroll
     for (int p = 0; p < MI; p++) {
         const int R = 32 * p + 8 * wave + (lane >> 3);
-        xchunk[p] = ((lane & 7) ^ swz(R)) * 8;
-        xsrc[p] = X + (long)imin(m0 + R, M - 1) * K;
+        xlane[p] = (uint32_t)(((long)imin(m0 + R, M - 1) * K + ((lane & 7) ^ swz(R)) * 8) * 2);
     }
-    const uint8_t* wld[2];
-    int whalf[2];
+    uint32_t wlane[2];
 #pragma unroll
     for (int i = 0; i < 2; i++) {
         const int r = 32 * i + (lane >> 1);
-        whalf[i] = 32 * ((lane & 1) ^ ((r >> 3) & 1));
-        wld[i] = W + (long)imin(n0 + r, N - 1) * (K >> 1);
+        wlane[i] = (uint32_t)((long)imin(n0 + r, N - 1) * (K >> 1) + 16 * ((lane & 1) ^ ((r >> 3) & 1)));
     }
-    const half2_t* zld = ZS + (long)imin(n0 + lane, N - 1) * groups;  // lane = row of the wave's 64
+    const uint32_t zlane = (uint32_t)((long)imin(n0 + lane, N - 1) * groups * 4);  // lane = row of the wave's 64
     int woff[2], zoff[2];
 #pragma unroll
     for (int ni = 0; ni < 2; ni++) {
@@ -367,24 +365,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[mi][ni][v] = 0.f;
 
-    // Loads of step `it` into stage c (wave-uniform); a k past the end is clamped, its scale zeroed at use.
+    // Loads of step `it` into stage c (both wave-uniform); a step past the end re-reads the last one, its scale
+    // is zeroed at use.
     auto issue = [&](int it, int c) {
+        const int itc = imin(it, nit - 1);
+        const uint8_t* xb = (const uint8_t*)X + (long)itc * (GEMM_BK * 2);
+        const uint8_t* wb = W + (long)itc * (GEMM_BK / 2);
 #pragma unroll
-        for (int p = 0; p < MI; p++) {
-            const int kx = imin(it * GEMM_BK + xchunk[p], K - 8);
-            load_to_lds_x4(xsrc[p] + kx, lds0 + X_OFF + c * XB + (32 * p + 8 * wave) * 128);
-        }
+        for (int p = 0; p < MI; p++) load_to_lds_x4(xb, xlane[p], lds0 + X_OFF + c * XB + (32 * p + 8 * wave) * 128);
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int kc = imin(it * GEMM_BK + whalf[i], K - 32);
-            load_to_lds_x4(wld[i] + (kc >> 1), lds0 + W_OFF + c * WB + wave * 2048 + i * 1024);
-        }
+        for (int i = 0; i < 2; i++) load_to_lds_x4(wb, wlane[i], lds0 + W_OFF + c * WB + wave * 2048 + i * 1024);
     };
     // The two zeros/scales pairs of the four-step group that starts at step `it`, into stage zc.
     auto issue_zs = [&](int it, int zc) {
-        const int gi = imin(it >> 1, groups - 2);
-        load_to_lds_x1(zld + gi, lds0 + Z_OFF + zc * ZB + wave * 512);
-        load_to_lds_x1(zld + gi + 1, lds0 + Z_OFF + zc * ZB + wave * 512 + 256);
+        const half2_t* zb = ZS + imin(it >> 1, groups - 2);
+        load_to_lds_x1(zb, zlane, lds0 + Z_OFF + zc * ZB + wave * 512);
+        load_to_lds_x1(zb + 1, zlane, lds0 + Z_OFF + zc * ZB + wave * 512 + 256);
     };
 
     // One K step: J = step within its group of four, c = its stage, cf = the stage read in the step
@@ -458,7 +454,9 @@ static hipError_t launch_mi(const void* x, const void* w, const void* zs, void* 
     const dim3 grid((N + GEMM_BN - 1) / GEMM_BN, (M + 32 * MI - 1) / (32 * MI), ksplit);
     unsigned* counters = (unsigned*)ws;
     float* part = ws ? (float*)((char*)ws + GEMM_COUNTER_BYTES) : nullptr;
-    if (lds && gshift == 7 && K % 256 == 0) {
+    // the LDS kernel addresses its operands with 32-bit byte offsets per lane
+    const bool fits32 = (long)M * K * 2 < (1L << 32) && (long)N * (K / 2) < (1L << 32);
+    if (lds && gshift == 7 && K % 256 == 0 && fits32) {
         hipLaunchKernelGGL((gemm_lds_kernel<MI>), grid, dim3(256), 0, st, (const uint8_t*)w, (const half2_t*)zs,
                            (const half_t*)x, (half_t*)y, M, N, K, epi, part, counters);
         return hipGetLastError();
