@@ -524,16 +524,21 @@ def prefill_leg(torch, capi, layer, shapes, g, dev, gen, stream, m=2048, reps=10
     side = torch.cuda.Stream(device=dev)
 
     def timed(fn):
-        for _ in range(3):
-            fn()
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        for _ in range(reps):
-            fn()
-        e1.record(stream)
-        stream.synchronize()
-        return e0.elapsed_time(e1) * 1e3 / reps
+        # A first estimate from a few launches, then a warm-up of about 20 ms and a timed window of about 40 ms
+        # (at least `reps` launches): after an idle gap the clocks take milliseconds to settle, and a window of a
+        # few launches reads up to 20 % low.
+        def window(n):
+            e0 = torch.cuda.Event(enable_timing=True)
+            e1 = torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(n):
+                fn()
+            e1.record(stream)
+            stream.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / n
+        est = max(window(3), 1.0)
+        window(max(3, min(2000, int(20000.0 / est))))
+        return window(max(reps, min(4000, int(40000.0 / est))))
 
     def clock_under(fn, us):
         n = max(8, int(3000.0 / us))           # about 3 ms of load on either side of the probe
