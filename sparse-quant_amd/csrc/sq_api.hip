@@ -110,11 +110,11 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
         // K split) fill at least half the chip (fc1 at 32 tokens 16.5 against 17.2 us, q/k/v-sized 14.3 against 15.5,
         // fc2 18.1 against 19.0)
         const bool wide_ok = M > 16 && M <= 32 && group_size == 128 && sq::skinny3_wide_applies(N, K, ws_ok);
-        // more than 32 tokens at group size 128: the tiled kernel with both operands through LDS and K split
+        // more than 32 tokens at group size 32, 64 or 128: the tiled kernel with both operands through LDS and K split
         // through the workspace (4096 x 4096 at 48 tokens 14.5 us against 17.2 for two blocks of the split-K
         // decode kernel, fc1 24.7 against 28.2, fc2 27.0 against 32.3; at 64 tokens 14.5 against 20.5 for the
         // 16-column kernel)
-        const bool lds_ok = M > 32 && group_size == 128 && K % 256 == 0 && gemm_ws;
+        const bool lds_ok = M > 32 && (group_size == 128 || group_size == 64 || group_size == 32) && K % 256 == 0 && gemm_ws;
         if (stream_ok || wide_ok) {
             kernel = SQ_ALGO_STREAM;
         } else if (lds_ok) {

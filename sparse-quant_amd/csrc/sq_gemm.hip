@@ -287,7 +287,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     gemm_tail<MI>(acc, Y, M, N, m0, n0, epi, part, counters);
 }
 
-// Both operands through LDS, for group size 128 and K a multiple of 256.  The kernels above hand
+// Both operands through LDS, for group sizes 32, 64 and 128 and K a multiple of 256.  The kernels above hand
 // every lane its own 16 bytes of a weight row (32 rows per wave-wide load) and 4 bytes of
 // zeros/scales, and the L1 takes lanes that are not neighbours in memory one at a time: about 1240
 // cache accesses per workgroup and K step, three per four cycles, which is what bounds those
@@ -299,12 +299,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 //     128 bits) are bank-conflict free;
 //   * activations: the swizzled chunk order of the register-staged kernel, written by the load
 //     instead of a store;
-//   * zeros/scales: the two pairs of a group of four steps, one dword per lane and pair, once per
-//     four steps.
+//   * zeros/scales: the two pairs of 2 g columns (four steps at group size 128, two at 64, one
+//     at 32), one dword per lane and pair.
 // Three stages (two for zeros/scales), loads two steps ahead; one barrier per step, behind a
 // counted wait for the loads of the next step (the loads just issued stay in flight).  Same
 // operand mapping and arithmetic as gemm_kernel: bit-identical results.
-template <int MI>
+template <int MI, int GS>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void gemm_lds_kernel(
     const uint8_t* __restrict__ W, const half2_t* __restrict__ ZS, const half_t* __restrict__ X, half_t* __restrict__ Y,
     int M, int N, int K, Epilogue epi, float* part, unsigned* counters) {
@@ -312,7 +312,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     constexpr int XB = BM * 128;  // bytes of an activation stage
     constexpr int WB = 256 * 32;  // bytes of a weight stage
     constexpr int ZB = 256 * 8;   // bytes of a zeros/scales stage: 4 waves x 2 pairs x 64 rows
-    constexpr int W_OFF = 0, Z_OFF = 3 * WB, X_OFF = Z_OFF + 2 * ZB;
+    // GS = log2 of the group size (5, 6, 7).  A zeros/scales stage always holds the two pairs of
+    // 2 g columns, i.e. of P = g / 32 steps: it is refilled every P steps, and with P = 1 it rotates
+    // with the operand stages (three of them) instead of alternating.
+    constexpr int P = 1 << (GS - 5);
+    constexpr int NZST = P == 1 ? 3 : 2;
+    static_assert(GS >= 5 && GS <= 7, "group sizes 32, 64, 128");
+    constexpr int W_OFF = 0, Z_OFF = 3 * WB, X_OFF = Z_OFF + NZST * ZB;
     __shared__ __attribute__((aligned(1024))) uint8_t lds[X_OFF + 3 * XB];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
 
@@ -324,7 +330,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     const int lc = lane >> 5;
     const int m0 = blockIdx.y * BM;
     const int n0 = blockIdx.x * GEMM_BN + 64 * wave;
-    const int groups = K >> 7;
+    const int groups = K >> GS;
     const int nit = K / GEMM_BK;
     // K split in whole four-step groups
     const int ksplit = gridDim.z;
@@ -351,7 +357,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 #pragma unroll
     for (int ni = 0; ni < 2; ni++) {
         woff[ni] = W_OFF + wave * 2048 + ((32 * ni + ln) * 2 + (lc ^ ((ln >> 3) & 1))) * 16;
-        zoff[ni] = Z_OFF + wave * 512 + (32 * ni + ln) * 4;
+        zoff[ni] = Z_OFF + wave * 512 + (32 * ni + ln) * 4 + (GS == 5 ? lc * 256 : 0);  // g = 32: the pair of the lane's half
     }
     int xoff[4];
 #pragma unroll
@@ -376,19 +382,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 #pragma unroll
         for (int i = 0; i < 2; i++) load_to_lds_x4(wb, wlane[i], lds0 + W_OFF + c * WB + wave * 2048 + i * 1024);
     };
-    // The two zeros/scales pairs of the four-step group that starts at step `it`, into stage zc.
+    // The two zeros/scales pairs of the P steps that start at step `it`, into stage zc.
     auto issue_zs = [&](int it, int zc) {
-        const half2_t* zb = ZS + imin(it >> 1, groups - 2);
+        const half2_t* zb = ZS + imin((it * GEMM_BK) >> GS, groups - 2);
         load_to_lds_x1(zb, zlane, lds0 + Z_OFF + zc * ZB + wave * 512);
         load_to_lds_x1(zb + 1, zlane, lds0 + Z_OFF + zc * ZB + wave * 512 + 256);
     };
 
     // One K step: J = step within its group of four, c = its stage, cf = the stage read in the step
-    // before (free since that step's barrier), zc = the zeros/scales stage of its group.
+    // before (free since that step's barrier), zc = the zeros/scales stage of steps 0 and 1 of the four.
     auto step = [&](int it, int c, int cf, int zc, auto J_) {
         constexpr int j = decltype(J_)::value;
+        constexpr bool fill = (j + 2) % P == 0;  // step it + 2 starts a zeros/scales group
+        const int zcur = P == 1 ? c : (P == 2 ? zc ^ (j >> 1) : zc);
         issue(it + 2, cf);
-        if constexpr (j == 2) issue_zs(it + 2, zc ^ 1);
+        if constexpr (fill) issue_zs(it + 2, P == 1 ? cf : zcur ^ 1);
         __builtin_amdgcn_sched_barrier(0);
         const bool kin = it < it1 && it * GEMM_BK + 32 * lc < K;  // false past the range: scale 0 -> W_hat 0
         u32x4_t q[2];
@@ -396,7 +404,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 #pragma unroll
         for (int ni = 0; ni < 2; ni++) {
             q[ni] = *(const u32x4_t*)(lds + c * WB + woff[ni]);
-            const half2_t zsv = *(const half2_t*)(lds + zc * ZB + (j >> 1) * 256 + zoff[ni]);
+            const half2_t zsv = *(const half2_t*)(lds + zcur * ZB + (P == 4 ? (j >> 1) : (P == 2 ? (j & 1) : 0)) * 256 + zoff[ni]);
             const half_t sv = kin ? zsv.y : (half_t)0.f;
             z64[ni] = (half2_t){zsv.x, zsv.x};
             sc[ni] = (half2_t){sv, sv};
@@ -418,13 +426,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         __builtin_amdgcn_sched_barrier(0);
         // the loads of step it + 1 (issued a step ago) have landed, this wave's operand reads are done:
         // behind the barrier stage c is free and the next stage is complete
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(MI + 2 + (j == 2 ? 2 : 0)) : "memory");
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(MI + 2 + (fill ? 2 : 0)) : "memory");
     };
 
     issue_zs(it0, 0);
     issue(it0, 0);
+    if constexpr (P == 1) issue_zs(it0 + 1, 1);
     issue(it0 + 1, 1);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(MI + 2) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(MI + 2 + (P == 1 ? 2 : 0)) : "memory");
     const int end = it0 + (it1 - it0 + 3) / 4 * 4;  // padded with steps whose scale is 0 and whose loads are clamped
     int c = 0, cp = 2, zc = 0;
     auto advance = [&]() {
@@ -440,7 +449,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         advance();
         step(it + 3, c, cp, zc, std::integral_constant<int, 3>{});
         advance();
-        zc ^= 1;
+        if constexpr (P == 4) zc ^= 1;
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last two steps' loads ran ahead of the range
     gemm_tail<MI>(acc, Y, M, N, m0, n0, epi, part, counters);
@@ -456,9 +465,16 @@ static hipError_t launch_mi(const void* x, const void* w, const void* zs, void* 
     float* part = ws ? (float*)((char*)ws + GEMM_COUNTER_BYTES) : nullptr;
     // the LDS kernel addresses its operands with 32-bit byte offsets per lane
     const bool fits32 = (long)M * K * 2 < (1L << 32) && (long)N * (K / 2) < (1L << 32);
-    if (lds && gshift == 7 && K % 256 == 0 && fits32) {
-        hipLaunchKernelGGL((gemm_lds_kernel<MI>), grid, dim3(256), 0, st, (const uint8_t*)w, (const half2_t*)zs,
-                           (const half_t*)x, (half_t*)y, M, N, K, epi, part, counters);
+    if (lds && gshift >= 5 && gshift <= 7 && K % 256 == 0 && fits32) {
+        if (gshift == 7)
+            hipLaunchKernelGGL((gemm_lds_kernel<MI, 7>), grid, dim3(256), 0, st, (const uint8_t*)w, (const half2_t*)zs,
+                               (const half_t*)x, (half_t*)y, M, N, K, epi, part, counters);
+        else if (gshift == 6)
+            hipLaunchKernelGGL((gemm_lds_kernel<MI, 6>), grid, dim3(256), 0, st, (const uint8_t*)w, (const half2_t*)zs,
+                               (const half_t*)x, (half_t*)y, M, N, K, epi, part, counters);
+        else
+            hipLaunchKernelGGL((gemm_lds_kernel<MI, 5>), grid, dim3(256), 0, st, (const uint8_t*)w, (const half2_t*)zs,
+                               (const half_t*)x, (half_t*)y, M, N, K, epi, part, counters);
         return hipGetLastError();
     }
     hipLaunchKernelGGL((gemm_kernel<MI>), grid, dim3(256), 0, st, (const uint8_t*)w, (const half2_t*)zs,
@@ -474,21 +490,22 @@ static hipError_t launch_mi(const void* x, const void* w, const void* zs, void* 
 // unsplit).  `pipe` receives the pipelined variant to use instead (-1 = none).
 struct GemmPlan {
     int mi, ksplit, pipe;
-    int lds = 0;  // 1: gemm_lds_kernel (group size 128, K a multiple of 256)
+    int lds = 0;  // 1: gemm_lds_kernel (group size 32, 64 or 128, K a multiple of 256)
 };
-// Group size 128 with K a multiple of 256 and more than 32 tokens: gemm_lds_kernel, whose choices
+// Group size 32, 64 or 128 with K a multiple of 256 and more than 32 tokens: gemm_lds_kernel, whose choices
 // come from a sweep of tile height x split over 4096 x 4096, 16384 x 4096, 4096 x 16384,
 // 11008 x 4096, 4096 x 11008 and 12288 x 4096 at 48..4096 tokens (within a few percent of the best
 // swept configuration on all of them): 32-row tiles up to 64 tokens on narrow weights (up to 128
 // when K is short as well), 128-row tiles beyond 256 tokens when the weight is wide or K long and
 // always beyond 1024, 64-row tiles between; K split while the grid stays within one round of 256
 // workgroups and every part keeps 8 steps.  Only a long K whose 256 x 256 tiles fill whole rounds
-// stays with the pipelined kernel (4096 x 16384 at 4096 tokens: 497 against 530 us).
-static GemmPlan plan_gemm_lds(int M, long ncol, int nit, bool have_ws) {
+// stays with the pipelined kernel (4096 x 16384 at 4096 tokens: 497 against 530 us); at group size 32, where
+// this kernel refills its zeros/scales every step, any K does (fc1 at 2048 tokens: 285 against 302 us).
+static GemmPlan plan_gemm_lds(int M, long ncol, int nit, int g, bool have_ws) {
     GemmPlan p = {1, 1, -1};
     const long t256 = ncol * ((M + 255) / 256);
     const long rounds = (t256 + 255) / 256;
-    if (M > 1024 && nit >= 128 && t256 * 10 >= rounds * 256 * 9) {
+    if (M > 1024 && (nit >= 128 || g == 32) && t256 * 10 >= rounds * 256 * 9) {
         p.pipe = 2;
         return p;
     }
@@ -515,7 +532,7 @@ static GemmPlan plan_gemm(int M, int N, int K, int g, bool have_ws) {
     const long t256 = ntiles(256);
     const long rounds = (t256 + 255) / 256;
     const int nit = (K + GEMM_BK - 1) / GEMM_BK;
-    if (g == 128 && K % 256 == 0 && M > 32) return plan_gemm_lds(M, ncol, nit, have_ws);
+    if ((g == 128 || g == 64 || g == 32) && K % 256 == 0 && M > 32) return plan_gemm_lds(M, ncol, nit, g, have_ws);
     if (M > 64 && t256 * 10 >= rounds * 256 * 6) {
         p.pipe = 2;  // 256 x 256 tiles pay from about 60 % of the CUs (5120 x 13696 at M = 2048: 338 us against 390 us)
     } else if (M > 64 && ntiles(128) >= 160) {
@@ -552,7 +569,7 @@ size_t gemm_workspace_bytes(int M, int N, int K) {
 }
 
 // tune = 0 for the heuristic, else the number of 32-row tiles per workgroup (1, 2 or 4) | ksplit << 8
-// (needs ws) | 0x80 for the kernel with both operands through LDS (group size 128, K % 256 == 0), or 8 / 9 / 10 for the software-pipelined kernel (128 rows at two waves per SIMD, 128 rows
+// (needs ws) | 0x80 for the kernel with both operands through LDS (group size 32..128, K % 256 == 0), or 8 / 9 / 10 for the software-pipelined kernel (128 rows at two waves per SIMD, 128 rows
 // at one, 256 rows at one).  ws = null or too small: K is never split.
 hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, size_t ws_bytes, int M,
                              int N, int K, int g, int tune, Epilogue epi, hipStream_t st) {

@@ -640,12 +640,13 @@ def test_gemm_split_k_every_tile_height(capi, mi, ksplit):
 @pytest.mark.parametrize("mi", [1, 2, 4])
 @pytest.mark.parametrize("ksplit", [1, 2, 4, 8])
 def test_gemm_operands_through_lds(capi, mi, ksplit):
-    # the tiled kernel whose weights, activations and zeros/scales all reach LDS by direct loads (group size 128,
-    # K a multiple of 256): parity against the oracle on ragged M and N, K = 256 x odd, K ranges of the split that
+    # the tiled kernel whose weights, activations and zeros/scales all reach LDS by direct loads (group sizes 32, 64,
+    # 128; K a multiple of 256): parity against the oracle on ragged M and N, K = 256 x odd, K ranges of the split that
     # are padded; bit-identical to the register-staged kernel at the same tile height and split; counters left clean
     lds = 0x80
-    for (m, n, k) in [(33, 264, 768), (70, 520, 1280), (129, 4096, 4096), (200, 264, 2816), (300, 1000, 11008)]:
-        g = 128
+    for (m, n, k, g) in [(33, 264, 768, 128), (70, 520, 1280, 128), (129, 4096, 4096, 128), (200, 264, 2816, 128),
+                         (300, 1000, 11008, 128), (70, 520, 1280, 64), (129, 1000, 2816, 64), (300, 264, 768, 64),
+                         (70, 520, 1280, 32), (129, 1000, 2816, 32), (300, 264, 768, 32)]:
         d = linear(n, k, g, seed=71)
         x = to_dev(orc.synth_x(m, k, seed=72))
         ws = torch.zeros(64 * 1024 * 1024, dtype=torch.uint8, device=DEV)
@@ -662,7 +663,7 @@ def test_gemm_operands_through_lds(capi, mi, ksplit):
 
 
 def test_gemm_lds_request_falls_back_where_it_does_not_apply(capi):
-    # other group sizes and a K that is no multiple of 256 run the register-staged kernel under the same request
+    # a K that is no multiple of 256 runs the register-staged kernel under the same request
     for (m, n, k, g) in [(70, 264, 704, 64), (100, 520, 1056, 32), (65, 264, 640, 128)]:
         check_gemm(capi, m, n, k, g, capi.SQ_ALGO_GEMM | ((2 | 0x80) << 8))
 
