@@ -431,7 +431,7 @@ __device__ __forceinline__ void skinny3_wide_body(const uint8_t* __restrict__ W,
                                                   const Epilogue& epi, int rb, int slot, int nslots) {
     using L = Sk3WideLds<RT, CH>;
     constexpr int MT = 2, ROWS = 16 * RT, TILE = L::TILE, ZC = L::ZCOLS;
-    static_assert(CH == 2 || CH == 4, "chunk slots per wave");
+    static_assert(CH == 4, "the request schedule below is written for four chunk slots per wave");
     static_assert(L::XWAVE >= TILE * 4, "a wave's partial tile fits its ring");
 
     extern __shared__ __attribute__((aligned(16))) uint8_t sk3_lds[];
@@ -504,10 +504,8 @@ __device__ __forceinline__ void skinny3_wide_body(const uint8_t* __restrict__ W,
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(8 + RT) : "memory");
     dma_x(1);
     load_w(1);
-    if constexpr (CH == 4) {
-        load_w(2);
-        load_w(3);
-    }
+    load_w(2);
+    load_w(3);
 
     float4_t acc[RT][MT];
 #pragma unroll
@@ -556,27 +554,19 @@ __device__ __forceinline__ void skinny3_wide_body(const uint8_t* __restrict__ W,
         }
     };
 
-    if constexpr (CH == 4) {
-        // requests so far, oldest first: zeros/scales, x0 8, w0 RT, x1 8, w1 RT, w2 RT, w3 RT
-        sk3_wait_words<8 + 3 * RT>(wq[0]);  // x0, w0 are there
-        consume(0);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // ring position 0 has been read
-        dma_x(2);
-        sk3_wait_words<8 + 2 * RT>(wq[1]);  // x1, w1 (w2, w3, x2 may be outstanding)
-        consume(1);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        dma_x(3);
-        sk3_wait_words<8>(wq[2]);  // w2, w3, x2 (x3 may be outstanding)
-        consume(2);
-        sk3_wait_words<0>(wq[3]);
-        consume(3);
-    } else {
-        // zeros/scales, x0 8, w0 RT, x1 8, w1 RT: both chunks fit the ring
-        sk3_wait_words<8 + RT>(wq[0]);
-        consume(0);
-        sk3_wait_words<0>(wq[1]);
-        consume(1);
-    }
+    // requests so far, oldest first: zeros/scales, x0 8, w0 RT, x1 8, w1 RT, w2 RT, w3 RT
+    sk3_wait_words<8 + 3 * RT>(wq[0]);  // x0, w0 are there
+    consume(0);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // ring position 0 has been read
+    dma_x(2);
+    sk3_wait_words<8 + 2 * RT>(wq[1]);  // x1, w1 (w2, w3, x2 may be outstanding)
+    consume(1);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    dma_x(3);
+    sk3_wait_words<8>(wq[2]);  // w2, w3, x2 (x3 may be outstanding)
+    consume(2);
+    sk3_wait_words<0>(wq[3]);
+    consume(3);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's ring is free: its partial tile goes there
 
     float* mine_lds = (float*)xw;
