@@ -301,7 +301,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 //     instead of a store;
 //   * zeros/scales: the two pairs of 2 g columns (four steps at group size 128, two at 64, one
 //     at 32), one dword per lane and pair.
-// Three stages (two for zeros/scales), loads two steps ahead; one barrier per step, behind a
+// Three stages (two for zeros/scales, three at group size 32), loads two steps ahead; one barrier per step, behind a
 // counted wait for the loads of the next step (the loads just issued stay in flight).  Same
 // operand mapping and arithmetic as gemm_kernel: bit-identical results.
 template <int MI, int GS>
