@@ -101,6 +101,29 @@ def _ext():
     return quant
 
 
+def test_host_side_queries_need_no_gpu(built_lib):
+    # Workspace sizes and the LayerNorm-fusion query are host arithmetic: what a binding may call at load time.
+    from sqamd import capi
+    L = capi.lib()
+    counters = 65536
+    # decode batches: counters + 8 K ranges x 64-row blocks x (4 row tiles x token tiles x 4 x 64 lanes) floats
+    assert L.sq_w4a16_workspace_bytes(1, 4096, 4096) == counters + 8 * 64 * (4 * 1 * 4 * 64) * 4
+    assert L.sq_w4a16_workspace_bytes(32, 16384, 4096) == counters + 8 * 256 * (4 * 2 * 4 * 64) * 4
+    # beyond 32 tokens: the larger of that and the tiled kernel's K split (64-row x 256-column tiles, four parts)
+    assert L.sq_w4a16_workspace_bytes(64, 16384, 4096) == counters + 4 * 64 * 64 * 256 * 4
+    # a grid that fills the chip splits nothing: only the decode kernels' share remains
+    assert L.sq_w4a16_workspace_bytes(2048, 16384, 4096) == L.sq_w4a16_workspace_bytes(32, 16384, 4096)
+    assert L.sq_w4a16_workspace_bytes(0, 4096, 4096) == 0
+    sizes = [L.sq_w4a16_workspace_bytes(m, 4096, 16384) for m in (1, 16, 17, 32, 33, 64, 512, 1024)]
+    assert all(b >= counters for b in sizes) and sizes[0] <= sizes[1] <= sizes[2] == sizes[3]
+    fus = L.sq_w4a16_ln_fusable
+    assert fus(8, 16384, 4096, 128, capi.SQ_LAYOUT_L1) == 1 and fus(1, 12288, 4096, 128, capi.SQ_LAYOUT_L1) == 1
+    for bad in ((9, 16384, 4096, 128, capi.SQ_LAYOUT_L1), (8, 16384, 2048, 128, capi.SQ_LAYOUT_L1),
+                (8, 16384, 8192, 128, capi.SQ_LAYOUT_L1), (8, 16384, 4096, 64, capi.SQ_LAYOUT_L1),
+                (8, 16384, 4096, 128, capi.SQ_LAYOUT_L2), (0, 16384, 4096, 128, capi.SQ_LAYOUT_L1)):
+        assert fus(*bad) == 0, bad
+
+
 def test_quant_module_surface():
     quant = _ext()
     for name in ("gemm_awq_ut", "dequant", "transpose_merge_zeros_scales", "convert_ours_to_awq",
