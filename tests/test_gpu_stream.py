@@ -152,8 +152,9 @@ def test_stream_is_the_automatic_choice_at_full_size(capi, n, k, m):
 @pytest.mark.parametrize("n,k", [(8192, 1024), (8200, 3200), (16384, 4096), (4096, 16384), (4096, 11008)])
 @pytest.mark.parametrize("m", [17, 24, 31, 32])
 def test_stream_two_token_tiles(capi, n, k, m):
-    """17..32 tokens: activations staged in two halves under one weight stream; explicit kernel id and automatic
-    dispatch against the oracle on sampled rows, with bias, ReLU and residual on the way out."""
+    """17..32 tokens: two token tiles per weight word, every wave moving the activations of its own chunks into LDS
+    (short K ranges leave chunk slots empty, long ones are split through the workspace, ragged N and K); explicit
+    kernel id and automatic dispatch against the oracle on sampled rows, with bias, ReLU and residual on the way out."""
     d = linear(n, k, seed=95)
     rng = np.random.default_rng(96 + m)
     x = orc.synth_x(m, k, seed=97 + m)
