@@ -242,6 +242,17 @@ int sq_repack_l2_to_l1(const void* w_l2, const void* zs_l2, void* w_l1, void* zs
  * (reference: test/muxi/module/qlinear/qlinear.py:93-103). */
 int sq_convert_2bit_to_4bit(const void* src, void* dst, int N, int K, void* stream);
 
+/* Layout L2 with 2-bit storage: int32 [K, N/8] (4-bit words) -> int32 [K, N/16] and back, with
+ * the arithmetic the reference's Python performs.  Shifts bind tighter than `&` in its
+ * expressions, so a pair of words (a, b) is stored as (a & 0xFFFF0000) + (b & 0x0000FFFF) and a
+ * stored word w expands to (w & 0x33333333, w & 0x33333333): the two are not inverses, and the
+ * library reproduces them bit for bit so that a 2-bit layer computes what it computes there.
+ * Replace convert_4bit_to_2bit / convert_2bit_to_4bit
+ * (reference: test/nvidia/utils/quant_dequant_nvidia.py:34-43 and :45-54; called from
+ * test/nvidia/module/qlinear/qlinear.py:58-62).  N must be a multiple of 16. */
+int sq_l2_convert_4bit_to_2bit(const void* src, void* dst, int K, int N, void* stream);
+int sq_l2_convert_2bit_to_4bit(const void* src, void* dst, int K, int N, void* stream);
+
 /* LUT block-sparse attention, prefill: out[z,h,m,:] = softmax over the keys of the
  * blocks lut[h][m/64][0..nnz) of (q k^T * sm_scale) (optionally causal) times v.
  * q, k, v, out fp16 [Z, H, S, D] contiguous, D in {64, 128}; lut int32 or int64

@@ -25,6 +25,10 @@ Pinning status of every function (what, other than this file, fixes it):
   gemm_ref              textbook matmul; float64 cross-check; one-hot rows
   rtn_quantize          closed form on hand-computed vectors
   convert_2bit_to_4bit  exhaustive over the 256 byte values
+  convert_4bit_to_2bit_l2 / convert_2bit_to_4bit_l2
+                        closed-form masks vs the sixteen terms of each loop evaluated
+                        one by one with Python's operator precedence; one-hot words
+                        (which of the 64 input bits survive, and where); hand vector
 No function here is "parity unpinned".
 """
 import numpy as np
@@ -301,6 +305,36 @@ def convert_2bit_to_4bit_l1(w2):
     first = ((b & 0xC0) >> 2) + ((b & 0x30) >> 4)
     second = ((b & 0x0C) << 2) + (b & 0x03)
     return np.stack([first, second], axis=-1).reshape(b.shape[0], b.shape[1] * 2).astype(np.uint8)
+
+
+def convert_4bit_to_2bit_l2(w4):
+    """int32 [K, N/8] -> int32 [K, N/16], the tensor-core layout's 2-bit storage.
+
+    Follows test/nvidia/utils/quant_dequant_nvidia.py:34-43 as Python evaluates it: the words are
+    taken in pairs (a, b) in row-major order, and each of the eight loop trips adds
+    `a & (0x30000000 >> 4*(i-1)) << 2*i` and `b & (0x30000000 >> 4*(i-1)) >> 16 - 2*i`.  `<<` and
+    `>>` bind tighter than `&`, so the shifts apply to the mask, not to the masked word: the masks
+    of a are 0xC0000000, 0x30000000, ... 0x00030000 (together 0xFFFF0000), those of b are 0xC000,
+    0x3000, ... 0x3 (together 0x0000FFFF), and the sum is (a & 0xFFFF0000) + (b & 0x0000FFFF).
+    """
+    w = np.ascontiguousarray(w4).view(np.uint32)
+    pairs = w.reshape(-1, 2)
+    out = (pairs[:, 0] & np.uint32(0xFFFF0000)) + (pairs[:, 1] & np.uint32(0x0000FFFF))
+    return out.astype(np.uint32).view(np.int32).reshape(w.shape[0], w.shape[1] // 2)
+
+
+def convert_2bit_to_4bit_l2(w2):
+    """int32 [K, N/16] -> int32 [K, N/8].
+
+    Follows test/nvidia/utils/quant_dequant_nvidia.py:45-54 as Python evaluates it: for a stored
+    word w the first output word sums `w & (0xC0000000 >> 2*(i-1)) >> 2*i`, whose masks are
+    0x30000000, 0x03000000, ... 0x3, the second sums `w & (0x0000C000 >> 2*(i-1)) << 16 - 2*i`
+    with the same eight masks: both are w & 0x33333333.
+    """
+    w = np.ascontiguousarray(w2).view(np.uint32)
+    m = (w & np.uint32(0x33333333)).reshape(-1)
+    out = np.stack([m, m], axis=1)
+    return out.view(np.int32).reshape(w.shape[0], w.shape[1] * 2)
 
 
 # ---------------------------------------------------------------------------

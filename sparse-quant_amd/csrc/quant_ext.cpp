@@ -370,18 +370,46 @@ void convert_awq_to_lmdeploy(at::Tensor qweight, at::Tensor qweight_dst, int in_
                    "convert_awq_to_lmdeploy");
 }
 
-// uint8 [N, K/4] 2-bit packed -> uint8 [N, K/2] 4-bit packed (layout L1).
+// 2-bit storage -> the 4-bit words the GEMM reads.  uint8 [N, K/4] -> uint8 [N, K/2] in layout L1;
+// int32 [K, N/16] -> int32 [K, N/8] in layout L2 (there with the reference's own word arithmetic).
 at::Tensor convert_2bit_to_4bit(at::Tensor qweight_2bit) {
     SQ_CHECK_DEVICE(qweight_2bit);
     SQ_CHECK_CONTIGUOUS(qweight_2bit);
-    SQ_CHECK_DTYPE(qweight_2bit, at::kByte);
     SQ_CHECK_DIMS(qweight_2bit, 2);
+    TORCH_CHECK(qweight_2bit.dtype() == at::kByte || qweight_2bit.dtype() == at::kInt,
+                "Tensor qweight_2bit must have dtype uint8 (layout L1) or int32 (layout L2)");
     c10::DeviceGuard guard(qweight_2bit.device());
+    if (qweight_2bit.dtype() == at::kInt) {
+        const int K = (int)qweight_2bit.size(0);
+        const int N = (int)qweight_2bit.size(1) * 16;
+        at::Tensor out = torch::empty({K, N / 8}, qweight_2bit.options());
+        raise_if_error(
+            sq_l2_convert_2bit_to_4bit(qweight_2bit.data_ptr(), out.data_ptr(), K, N, current_stream(qweight_2bit)),
+            "convert_2bit_to_4bit");
+        return out;
+    }
     const int N = (int)qweight_2bit.size(0);
     const int K = (int)qweight_2bit.size(1) * 4;
     at::Tensor out = torch::empty({N, K / 2}, qweight_2bit.options());
     raise_if_error(sq_convert_2bit_to_4bit(qweight_2bit.data_ptr(), out.data_ptr(), N, K, current_stream(qweight_2bit)),
                    "convert_2bit_to_4bit");
+    return out;
+}
+
+// int32 [K, N/8] -> int32 [K, N/16] (layout L2, the reference's word arithmetic).
+at::Tensor convert_4bit_to_2bit(at::Tensor qweight_4bit) {
+    SQ_CHECK_DEVICE(qweight_4bit);
+    SQ_CHECK_CONTIGUOUS(qweight_4bit);
+    SQ_CHECK_DTYPE(qweight_4bit, at::kInt);
+    SQ_CHECK_DIMS(qweight_4bit, 2);
+    TORCH_CHECK(qweight_4bit.size(1) % 2 == 0, "qweight_4bit needs an even number of words per row");
+    c10::DeviceGuard guard(qweight_4bit.device());
+    const int K = (int)qweight_4bit.size(0);
+    const int N = (int)qweight_4bit.size(1) * 8;
+    at::Tensor out = torch::empty({K, N / 16}, qweight_4bit.options());
+    raise_if_error(
+        sq_l2_convert_4bit_to_2bit(qweight_4bit.data_ptr(), out.data_ptr(), K, N, current_stream(qweight_4bit)),
+        "convert_4bit_to_2bit");
     return out;
 }
 
@@ -417,6 +445,7 @@ PYBIND11_MODULE(quant, m) {
           py::arg("bias") = py::none(), py::arg("residual") = py::none(), py::arg("act") = "none", py::arg("N"),
           py::arg("group_size"));
     m.def("convert_2bit_to_4bit", &convert_2bit_to_4bit);
+    m.def("convert_4bit_to_2bit", &convert_4bit_to_2bit);
     m.def("clear_repack_cache", &clear_repack_cache);
     m.def("repack_cache_size", &repack_cache_size);
     m.def("version", []() { return sq_version(); });

@@ -447,6 +447,18 @@ int sq_convert_2bit_to_4bit(const void* src, void* dst, int N, int K, void* stre
     return launch_code(sq::launch_2bit_to_4bit(src, dst, N, K, static_cast<hipStream_t>(stream)));
 }
 
+int sq_l2_convert_4bit_to_2bit(const void* src, void* dst, int K, int N, void* stream) {
+    if (N <= 0 || K <= 0 || N % 16 != 0) return SQ_ERR_BAD_SHAPE;
+    if (!src || !dst) return SQ_ERR_NULL_POINTER;
+    return launch_code(sq::launch_l2_4bit_to_2bit(src, dst, K, N, static_cast<hipStream_t>(stream)));
+}
+
+int sq_l2_convert_2bit_to_4bit(const void* src, void* dst, int K, int N, void* stream) {
+    if (N <= 0 || K <= 0 || N % 16 != 0) return SQ_ERR_BAD_SHAPE;
+    if (!src || !dst) return SQ_ERR_NULL_POINTER;
+    return launch_code(sq::launch_l2_2bit_to_4bit(src, dst, K, N, static_cast<hipStream_t>(stream)));
+}
+
 int sq_lut_attention_fwd(const void* q, const void* k, const void* v, void* out, const void* lut, int lut_elem_bytes,
                          int Z, int H, int S, int D, int nnz, float sm_scale, int causal, void* stream) {
     if (Z <= 0 || H <= 0 || S <= 0 || nnz <= 0 || (D != 64 && D != 128)) return SQ_ERR_BAD_SHAPE;

@@ -21,6 +21,8 @@ hipError_t launch_awq_to_lmdeploy(const void* src, void* dst, int K, int N, hipS
 hipError_t launch_l2_to_l1(const void* w_l2, const void* zs_l2, void* w_l1, void* zs_l1, int N, int K, int g,
                            hipStream_t st);
 hipError_t launch_2bit_to_4bit(const void* src, void* dst, int N, int K, hipStream_t st);
+hipError_t launch_l2_4bit_to_2bit(const void* src, void* dst, int K, int N, hipStream_t st);
+hipError_t launch_l2_2bit_to_4bit(const void* src, void* dst, int K, int N, hipStream_t st);
 
 // The *_tuned launchers take a kernel-specific tuning word (0 = built-in heuristic).
 // sq_gemv2.hip: M <= 8, streaming formulation.  tune = waves per workgroup (1,2,4,8).

@@ -128,6 +128,26 @@ __global__ void w2_to_w4_kernel(const uint8_t* __restrict__ src, uint8_t* __rest
     }
 }
 
+// Tensor-core layout, 2-bit storage, with the arithmetic the reference's Python performs
+// (reference: test/nvidia/utils/quant_dequant_nvidia.py:34-54).  `<<` and `>>` bind tighter than `&`
+// there, so the eight masks of each loop add up to one constant: a pair of 4-bit words (a, b) is
+// stored as (a & 0xFFFF0000) + (b & 0x0000FFFF), and a stored word w expands to the pair
+// (w & 0x33333333, w & 0x33333333).  Mirrored bit for bit; it is not an inverse pair.
+__global__ void l2_w4_to_w2_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, long total) {
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride)
+        dst[i] = (src[2 * i] & 0xFFFF0000u) + (src[2 * i + 1] & 0x0000FFFFu);
+}
+
+__global__ void l2_w2_to_w4_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, long total) {
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const uint32_t w = src[i] & 0x33333333u;
+        dst[2 * i] = w;
+        dst[2 * i + 1] = w;
+    }
+}
+
 hipError_t launch_transpose_merge_zeros_scales(const void* zeros, const void* scales, void* zs, int K, int N, int g,
                                                hipStream_t st) {
     const long total = (long)(K / g) * N;
@@ -163,6 +183,20 @@ hipError_t launch_2bit_to_4bit(const void* src, void* dst, int N, int K, hipStre
     const long total = (long)N * (K / 4);
     hipLaunchKernelGGL(w2_to_w4_kernel, flat_grid(total, 256), dim3(256), 0, st, (const uint8_t*)src,
                        (uint8_t*)dst, total);
+    return hipGetLastError();
+}
+
+hipError_t launch_l2_4bit_to_2bit(const void* src, void* dst, int K, int N, hipStream_t st) {
+    const long total = (long)K * (N / 16);
+    hipLaunchKernelGGL(l2_w4_to_w2_kernel, flat_grid(total, 256), dim3(256), 0, st, (const uint32_t*)src,
+                       (uint32_t*)dst, total);
+    return hipGetLastError();
+}
+
+hipError_t launch_l2_2bit_to_4bit(const void* src, void* dst, int K, int N, hipStream_t st) {
+    const long total = (long)K * (N / 16);
+    hipLaunchKernelGGL(l2_w2_to_w4_kernel, flat_grid(total, 256), dim3(256), 0, st, (const uint32_t*)src,
+                       (uint32_t*)dst, total);
     return hipGetLastError();
 }
 

@@ -38,6 +38,8 @@ SIGNATURES = {
     "sq_convert_awq_to_lmdeploy": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_repack_l2_to_l1": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "sq_convert_2bit_to_4bit": (_i, [_vp, _vp, _i, _i, _vp]),
+    "sq_l2_convert_4bit_to_2bit": (_i, [_vp, _vp, _i, _i, _vp]),
+    "sq_l2_convert_2bit_to_4bit": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_decode_attention": (_i, [_vp] * 7 + [_i] * 4 + [ctypes.c_long] * 7 + [_i, _vp, ctypes.c_float, _vp, ctypes.c_size_t,
                                  _vp]),
     "sq_decode_attention_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
@@ -311,6 +313,24 @@ def convert_2bit_to_4bit(w2, stream=None):
     out = torch.empty((n, k4 * 2), dtype=torch.uint8, device=w2.device)
     _check(lib().sq_convert_2bit_to_4bit(_ptr(w2), _ptr(out), n, k4 * 4, _stream(stream)),
            "sq_convert_2bit_to_4bit")
+    return out
+
+
+def l2_convert_4bit_to_2bit(w4, stream=None):
+    """int32 [K, N/8] -> int32 [K, N/16]."""
+    k, n8 = w4.shape
+    out = torch.empty((k, n8 // 2), dtype=torch.int32, device=w4.device)
+    _check(lib().sq_l2_convert_4bit_to_2bit(_ptr(w4), _ptr(out), k, n8 * 8, _stream(stream)),
+           "sq_l2_convert_4bit_to_2bit")
+    return out
+
+
+def l2_convert_2bit_to_4bit(w2, stream=None):
+    """int32 [K, N/16] -> int32 [K, N/8]."""
+    k, n16 = w2.shape
+    out = torch.empty((k, n16 * 2), dtype=torch.int32, device=w2.device)
+    _check(lib().sq_l2_convert_2bit_to_4bit(_ptr(w2), _ptr(out), k, n16 * 16, _stream(stream)),
+           "sq_l2_convert_2bit_to_4bit")
     return out
 
 

@@ -57,9 +57,19 @@ class WALinear(nn.Module):
         shape allows (up to 8 tokens, group size 128, 2048 < K <= 4096)."""
         weight = self.weight
         if self.w_bit == 2:
-            if self.layout != "l1":
-                raise NotImplementedError("2-bit weights are supported in layout 'l1' only")
-            weight = quant.convert_2bit_to_4bit(weight)
+            # uint8 [N, K/4] or int32 [K, N/16] -> the 4-bit words of the same layout, as the
+            # reference's forward does on every call (test/muxi/module/qlinear/qlinear.py:61-62,
+            # test/nvidia/module/qlinear/qlinear.py:58-61).
+            # The int32 expansion is kept while the stored words do not change, so that the
+            # one-time conversion of that layout behind gemm_awq_ut is not repeated per call.
+            if self.layout == "l1":
+                weight = quant.convert_2bit_to_4bit(weight)
+            else:
+                key = (weight.data_ptr(), weight._version)
+                if getattr(self, "_expanded_key", None) != key:
+                    self._expanded = quant.convert_2bit_to_4bit(weight)
+                    self._expanded_key = key
+                weight = self._expanded
         lead = x.shape[:-1]
         x3 = x.reshape(1, -1, x.shape[-1]) if x.dim() != 3 else x
         res3 = None

@@ -106,14 +106,14 @@ def quant_lmdeploy(weight, input_features, output_features, group_size=128, n_bi
 
     Same three-step chain as the reference: "ours" bytes (even k in the high
     nibble) -> AWQ order -> tensor-core tile order, plus the transposed merge of
-    zeros and scales; every step is a kernel of the `quant` extension.  Only n_bit = 4: the
-    reference's int32 2-bit repacking (convert_4bit_to_2bit, :34-43) keeps, as Python evaluates its
-    shifts and masks, only half of each pair of words, so there is no 2-bit format to be compatible with.
+    zeros and scales; every step is a kernel of the `quant` extension.  n_bit = 2 quantises to
+    four levels and passes the words through convert_4bit_to_2bit as the reference does (:29-30),
+    which returns int32 [K, N/16].
     """
     import quant
 
-    if n_bit != 4:
-        raise NotImplementedError("the tensor-core layout stores 4-bit weights only")
+    if n_bit not in (2, 4):
+        raise ValueError("n_bit must be 2 or 4")
     w = _as(weight, compute_dtype)
     q, scales, zeros = quantize_tensor(w, n_bit, group_size)
     g = group_size
@@ -128,4 +128,24 @@ def quant_lmdeploy(weight, input_features, output_features, group_size=128, n_bi
     quant.convert_ours_to_awq(ours, awq, input_features, output_features)
     qweight = torch.empty((input_features, output_features // 8), dtype=torch.int32, device=dev)
     quant.convert_awq_to_lmdeploy(awq, qweight, input_features, output_features)
+    if n_bit == 2:
+        qweight = convert_4bit_to_2bit(qweight)
     return qweight, zeros_scales, w_fp16
+
+
+def convert_4bit_to_2bit(qweight_4bit):
+    """int32 [K, N/8] -> int32 [K, N/16], bit for bit what the reference's function of this name
+    returns (test/nvidia/utils/quant_dequant_nvidia.py:34-43).  Its shifts bind tighter than its
+    `&`, so the eight masks per word add up to a constant: a pair of words (a, b) becomes
+    (a & 0xFFFF0000) + (b & 0x0000FFFF), not a 2-bit compaction of both."""
+    import quant
+
+    return quant.convert_4bit_to_2bit(qweight_4bit.contiguous())
+
+
+def convert_2bit_to_4bit(qweight_2bit):
+    """int32 [K, N/16] -> int32 [K, N/8] (:45-54 of the same file): every stored word w yields the
+    pair (w & 0x33333333, w & 0x33333333).  uint8 input is the L1 expansion instead."""
+    import quant
+
+    return quant.convert_2bit_to_4bit(qweight_2bit.contiguous())

@@ -91,6 +91,10 @@ def test_argument_errors_come_before_any_launch(built_lib):
     assert L.sq_repack_l2_to_l1(p, p, p, p, 64, 128, 64, None) == capi.SQ_ERR_BAD_GROUP
     assert L.sq_convert_2bit_to_4bit(p, None, 8, 64, None) == capi.SQ_ERR_NULL_POINTER
     assert L.sq_convert_2bit_to_4bit(p, p, 8, 62, None) == capi.SQ_ERR_BAD_SHAPE
+    for fn in (L.sq_l2_convert_4bit_to_2bit, L.sq_l2_convert_2bit_to_4bit):
+        assert fn(p, None, 8, 64, None) == capi.SQ_ERR_NULL_POINTER
+        assert fn(p, p, 8, 24, None) == capi.SQ_ERR_BAD_SHAPE
+        assert fn(p, p, 0, 64, None) == capi.SQ_ERR_BAD_SHAPE
 
 
 def _ext():

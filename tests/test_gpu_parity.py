@@ -247,6 +247,21 @@ def test_two_bit_expansion(capi):
     assert np.array_equal(out, orc.convert_2bit_to_4bit_l1(w2))
 
 
+def test_two_bit_int32_layout_words(capi):
+    """Layout L2 with 2-bit storage: the packer and the expander against the oracle's
+    restatement of the reference's word arithmetic, bit for bit."""
+    rng = np.random.default_rng(29)
+    for k, n in ((32, 64), (96, 1040), (1, 16)):
+        w4 = rng.integers(0, 2**32, size=(k, n // 8), dtype=np.uint64).astype(np.uint32).view(np.int32)
+        packed = capi.l2_convert_4bit_to_2bit(to_dev(w4))
+        assert packed.dtype == torch.int32 and tuple(packed.shape) == (k, n // 16)
+        assert np.array_equal(packed.cpu().numpy(), orc.convert_4bit_to_2bit_l2(w4))
+        w2 = rng.integers(0, 2**32, size=(k, n // 16), dtype=np.uint64).astype(np.uint32).view(np.int32)
+        wide = capi.l2_convert_2bit_to_4bit(to_dev(w2))
+        assert wide.dtype == torch.int32 and tuple(wide.shape) == (k, n // 8)
+        assert np.array_equal(wide.cpu().numpy(), orc.convert_2bit_to_4bit_l2(w2))
+
+
 # ------------------------------------------------------------------ the `quant` extension and WALinear
 def test_quant_extension_matches_reference_recipe():
     """The reference's own kernel check: allclose(x @ W_hat.T, gemm_awq_ut(...), atol = rtol = 2e-2)
@@ -339,6 +354,45 @@ def test_walinear_module():
     x = torch.randn((1, 4, k), dtype=torch.float16, device=DEV)
     ref = torch.matmul(x.float(), qf.dequant_to_fp16(lin.weight.data, 2, 64).float().t()) + lin.bias.float()
     assert (q2(x).float() - ref).abs().max() <= TOL * ref.abs().max()
+
+
+def test_walinear_two_bit_int32_layout():
+    """A 2-bit layer in layout L2 computes what the reference's module computes: four-level codes
+    packed into the tensor-core layout, the reference's 4-bit -> 2-bit -> 4-bit word arithmetic
+    (which returns half of the codes in their neighbours' places), then the 4-bit GEMM on the result.
+    Expected value from the oracle's chain on the same fp16 weight."""
+    import quant
+    from sqamd.qlinear import WALinear
+    from sqamd import quant_funcs as qf
+    rng = np.random.default_rng(31)
+    k, n, g = 512, 256, 128
+    w = (rng.normal(0, 0.05, size=(n, k))).astype(np.float16)
+    bias = rng.normal(0, 0.1, size=n).astype(np.float16)
+    lin = torch.nn.Linear(k, n, bias=True, device=DEV, dtype=torch.float16)
+    lin.weight.data.copy_(torch.from_numpy(w))
+    lin.bias.data.copy_(torch.from_numpy(bias))
+    layer = WALinear.from_float(lin, {"n_bit": 2, "group_size": g}, None, layout="l2")
+    assert layer.weight.dtype == torch.int32 and tuple(layer.weight.shape) == (k, n * 2 // 32)
+    # the packer's side of the chain
+    q, s, z = orc.rtn_quantize(w, 2, g, dtype=np.float16)
+    assert q.max() <= 3
+    stored = orc.convert_4bit_to_2bit_l2(orc.pack_l2(q))
+    assert np.array_equal(layer.weight.cpu().numpy(), stored)
+    zs = orc.transpose_merge_zeros_scales(z.astype(np.float16), s.astype(np.float16), k, n, g)
+    assert np.array_equal(layer.zeros_scales.cpu().numpy().view(np.uint16), zs.view(np.uint16))
+    # the module's side: expand, then the 4-bit GEMM
+    w4 = orc.convert_2bit_to_4bit_l2(stored)
+    assert np.array_equal(qf.convert_2bit_to_4bit(layer.weight).cpu().numpy(), w4)
+    x = rng.normal(0, 0.5, size=(2, 3, k)).astype(np.float16)
+    want = orc.gemm_l2(x.reshape(-1, k), w4, zs, g, k, n)[0].astype(np.float64) + bias.astype(np.float64)
+    fresh = WALinear(k, n, w_bit=2, group_size=g, bias=True, dev=DEV, layout="l2")
+    fresh.load_state_dict(layer.state_dict())
+    for _ in range(2):  # the second call reuses the kept expansion
+        got = fresh(to_dev(x)).cpu().numpy().astype(np.float64).reshape(-1, n)
+        assert np.abs(got - want).max() <= TOL * np.abs(want).max()
+    # half of the codes are not where a lossless 2-bit format would put them
+    assert not np.array_equal(w4, orc.pack_l2(q))
+    quant.clear_repack_cache()
 
 
 # ------------------------------------------------------------------ workspace-backed split-K kernel (5 <= M <= 32)

@@ -320,6 +320,79 @@ def test_two_bit_kat_and_exhaustive():
         assert out[v, 0] == (a | (bb << 4)) and out[v, 1] == (c | (d << 4))
 
 
+def _int32_sum(terms):
+    """Sum as torch's int32 `+=` gives it: modulo 2**32."""
+    return sum(terms) & 0xFFFFFFFF
+
+
+def _pack_pair_termwise(a, b):
+    """The sixteen terms of the packer's loop, each parenthesised the way Python's grammar
+    groups it (multiplication, then +/-, then shifts left to right, then &)."""
+    terms = []
+    for i in range(1, 9):
+        terms.append(a & ((0x30000000 >> (4 * (i - 1))) << (2 * i)))
+        terms.append(b & ((0x30000000 >> (4 * (i - 1))) >> (16 - 2 * i)))
+    return _int32_sum(terms)
+
+
+def _expand_termwise(w):
+    first, second = [], []
+    for i in range(1, 9):
+        first.append(w & ((0xC0000000 >> (2 * (i - 1))) >> (2 * i)))
+        second.append(w & ((0x0000C000 >> (2 * (i - 1))) << (16 - 2 * i)))
+    return _int32_sum(first), _int32_sum(second)
+
+
+def test_two_bit_int32_layout_words():
+    """The int32-layout 2-bit pair computes what the reference's expressions compute under
+    Python's precedence: checked term by term, on one-hot words and on a hand vector."""
+    # Python really groups the unparenthesised source text this way.
+    a, b, i = 0x89ABCDEF, 0x13579BDF, 3
+    assert (a & (0x30000000 >> 4 * (i - 1)) << 2 * i) == (a & ((0x30000000 >> (4 * (i - 1))) << (2 * i)))
+    assert (b & (0x30000000 >> 4 * (i - 1)) >> 16 - 2 * i) == (b & ((0x30000000 >> (4 * (i - 1))) >> (16 - 2 * i)))
+    assert (a & (0xC0000000 >> 2 * (i - 1)) >> 2 * i) == (a & ((0xC0000000 >> (2 * (i - 1))) >> (2 * i)))
+    assert (b & (0x0000C000 >> 2 * (i - 1)) << 16 - 2 * i) == (b & ((0x0000C000 >> (2 * (i - 1))) << (16 - 2 * i)))
+
+    k = KAT["two_bit_int32"]
+    w4 = np.array([k["words_4bit"]], dtype=np.uint32).view(np.int32)
+    packed = orc.convert_4bit_to_2bit_l2(w4)
+    assert packed.view(np.uint32).tolist() == [k["words_2bit"]]
+    assert orc.convert_2bit_to_4bit_l2(packed).view(np.uint32).tolist() == [k["words_expanded"]]
+
+    rng = np.random.default_rng(23)
+    w = rng.integers(0, 2**32, size=(6, 8), dtype=np.uint64).astype(np.uint32)
+    got = orc.convert_4bit_to_2bit_l2(w.view(np.int32)).view(np.uint32)
+    assert got.shape == (6, 4)
+    flat = w.reshape(-1, 2)
+    want = [_pack_pair_termwise(int(p[0]), int(p[1])) for p in flat]
+    assert got.reshape(-1).tolist() == want
+    back = orc.convert_2bit_to_4bit_l2(got.view(np.int32)).view(np.uint32)
+    assert back.shape == (6, 8)
+    want_back = [x for v in got.reshape(-1) for x in _expand_termwise(int(v))]
+    assert back.reshape(-1).tolist() == want_back
+
+    # One-hot inputs: a bit of the first word survives iff it is in the upper half, a bit of the
+    # second iff it is in the lower half, and it stays where it was.
+    for bit in range(32):
+        one = np.uint32(1 << bit)
+        pa = orc.convert_4bit_to_2bit_l2(np.array([[one, 0]], dtype=np.uint32).view(np.int32)).view(np.uint32)[0, 0]
+        pb = orc.convert_4bit_to_2bit_l2(np.array([[0, one]], dtype=np.uint32).view(np.int32)).view(np.uint32)[0, 0]
+        assert pa == (one if bit >= 16 else 0) and pb == (one if bit < 16 else 0)
+        e = orc.convert_2bit_to_4bit_l2(np.array([[one]], dtype=np.uint32).view(np.int32)).view(np.uint32)[0]
+        keep = one if (bit % 4) < 2 else 0
+        assert e.tolist() == [keep, keep]
+    # Words holding 2-bit codes (every nibble <= 3): the upper four codes of the first word and the
+    # lower four of the second come back; the other eight are replaced by their neighbours'.
+    codes = rng.integers(0, 4, size=(5, 4, 8), dtype=np.uint32)
+    words = (codes << (4 * np.arange(8, dtype=np.uint32))).sum(axis=2).astype(np.uint32)
+    rt = orc.convert_2bit_to_4bit_l2(orc.convert_4bit_to_2bit_l2(words.view(np.int32))).view(np.uint32)
+    rt_codes = (rt[..., None] >> (4 * np.arange(8, dtype=np.uint32))) & 15
+    pairs = codes.reshape(5, 2, 2, 8)
+    rtp = rt_codes.reshape(5, 2, 2, 8)
+    assert np.array_equal(rtp[:, :, 0, 4:], pairs[:, :, 0, 4:]) and np.array_equal(rtp[:, :, 1, :4], pairs[:, :, 1, :4])
+    assert np.array_equal(rtp[:, :, 0, :4], pairs[:, :, 1, :4]) and np.array_equal(rtp[:, :, 1, 4:], pairs[:, :, 0, 4:])
+
+
 # ---- LayerNorm restatement ----
 
 def test_layernorm_closed_forms():
