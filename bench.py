@@ -495,6 +495,7 @@ def main():
             out["decode_batch"] = decode_batch_leg(torch, capi, pool, shapes, g, dev, gen, stream)
             out["config1"] = config1_leg(torch, capi, dev, gen, stream)
             out["layernorm_fused"] = ln_fused_leg(torch, capi, pool, shapes, g, dev, gen, stream)
+            out["gated_mlp"] = gated_mlp_leg(torch, capi, g, dev, gen, stream)
             if m <= 4:
                 out["sequence"] = sequence_leg(torch, capi, pool, shapes, m, g, dev, gen, stream, bytes_per_step)
             out["fused_qkv"] = fused_qkv_leg(torch, capi, m, g, dev, gen, stream, args.layers, bytes_per_step)
@@ -788,6 +789,71 @@ def ln_fused_leg(torch, capi, pool, shapes, g, dev, gen, stream, m=8):
             stream.synchronize()
             res[name] = {"us": round(e0.elapsed_time(e1) * 1e3 / (50 * len(pool)), 2),
                          "launches": 2 if fn is two else 1}
+    return res
+
+
+def gated_mlp_leg(torch, capi, g, dev, gen, stream, n=11008, k=4096, tokens=(1, 8, 2048), copies=8):
+    """Front half of a Llama-7B MLP, silu(x W_gate^T) * (x W_up^T) with both weights 11008 x 4096: sq_w4a16_gemm_silu_dot
+    (two launches, SiLU and product in the second one's store) against two plain linears followed by torch's silu and
+    multiply (four launches), cold weights (rotating pool), HIP-graph replay; parity against the oracle's float64
+    formula on sampled output rows."""
+    import numpy as np
+    import w4a16_oracle as orc
+    pool = [(make_linear(n, k, g, dev, gen), make_linear(n, k, g, dev, gen)) for _ in range(copies)]
+    res = {"shape": "gate, up %d x %d, group %d" % (n, k, g), "pool_mb": round(copies * 2 * n * k / 2 / 1e6)}
+    for m in tokens:
+        x = torch.randn((m, k), device=dev, generator=gen).half()
+        y = torch.empty((m, n), dtype=torch.float16, device=dev)
+        a = torch.empty((m, n), dtype=torch.float16, device=dev)
+        b = torch.empty((m, n), dtype=torch.float16, device=dev)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            ws = capi.workspace(m, n, k, dev, stream) if 2 < m <= 1024 else None
+
+            def fused():
+                for (wg, zg), (wu, zu) in pool:
+                    capi.gemm_silu_dot(x, wg, zg, wu, zu, n, k, g, out=y, stream=stream, ws=ws, up_out=b)
+
+            def unfused():
+                for (wg, zg), (wu, zu) in pool:
+                    capi.gemm_ws(x, wg, zg, n, k, g, out=a, stream=stream, ws=ws)
+                    capi.gemm_ws(x, wu, zu, n, k, g, out=b, stream=stream, ws=ws)
+                    torch.mul(torch.nn.functional.silu(a), b, out=y)
+
+            fused()
+            stream.synchronize()
+            (wg, zg), (wu, zu) = pool[-1]
+            rng = np.random.default_rng(m)
+            ridx = np.sort(rng.choice(n, size=64, replace=False))
+            tidx = np.arange(m) if m <= 32 else np.sort(rng.choice(m, size=32, replace=False))
+            want = orc.silu_dot_ref(x.cpu().numpy()[tidx], orc.dequant_l1(wg.cpu().numpy()[ridx], zg.cpu().numpy()[ridx], g),
+                                    orc.dequant_l1(wu.cpu().numpy()[ridx], zu.cpu().numpy()[ridx], g))
+            got = y.float().cpu().numpy()[tidx][:, ridx]
+            err = gate(float(np.max(np.abs(got - want)) / np.max(np.abs(want))) if np.all(np.isfinite(got)) else float("inf"),
+                       "gated MLP at M=%d" % m)
+            entry = {"parity_max_rel_err": round(err, 6)}
+            for name, fn in (("silu_dot_in_the_store", fused), ("two_linears_then_torch", unfused)):
+                fn()
+                stream.synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=stream):
+                    fn()
+                reps = 20 if m <= 64 else 3
+                for _ in range(reps):
+                    graph.replay()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(2 * reps):
+                    graph.replay()
+                e1.record(stream)
+                stream.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / (2 * reps * copies)
+                entry[name] = {"us": round(us, 2), "launches": 2 if fn is fused else 4}
+                if m >= 512:
+                    entry[name]["tflops"] = round(4.0 * m * n * k / us * 1e-6, 1)
+                else:
+                    entry[name]["gbs"] = round(2 * algorithmic_bytes(m, n, k, g) / us * 1e-3, 1)
+            res["m%d" % m] = entry
     return res
 
 

@@ -140,7 +140,7 @@ size_t sq_w4a16_workspace_bytes(int M, int N, int K);
 /* The same product with the element-wise tail of the linear folded into the kernel's
  * store: Y = act(X * W_hat^T + bias) + residual, computed on the fp32 accumulator and
  * rounded to fp16 once.  bias fp16 [N] or NULL; residual fp16 [M, N] or NULL (must not
- * overlap y); act SQ_ACT_NONE or SQ_ACT_RELU.  workspace may be NULL (then the
+ * overlap y); act SQ_ACT_NONE, SQ_ACT_RELU or SQ_ACT_SILU (v / (1 + exp(-v))).  workspace may be NULL (then the
  * workspace-free kernels are used); otherwise as for sq_w4a16_gemm_ws.  Replaces the
  * separate `out + bias` of WALinear.forward (reference:
  * test/nvidia/module/qlinear/qlinear.py:69-70), the ReLU after fc1 and the residual
@@ -150,10 +150,26 @@ size_t sq_w4a16_workspace_bytes(int M, int N, int K);
  * is not part of it (quantization/nvidia/script/gemm_awq_test.py). */
 #define SQ_ACT_NONE 0
 #define SQ_ACT_RELU 1
+#define SQ_ACT_SILU 2
 int sq_w4a16_gemm_fused(const void* x, const void* w, const void* zs, const void* bias,
                         const void* residual, void* y, int M, int N, int K, int group_size,
                         int layout, int act, int algo, void* workspace, size_t workspace_bytes,
                         void* stream);
+
+/* Front half of a gated MLP: Y = silu(X * W_gate_hat^T) .* (X * W_up_hat^T), two launches: the up
+ * projection into up_scratch (fp16 [M, N], caller-allocated, must not overlap y; holds the up
+ * projection afterwards), then the gate projection, whose store applies SiLU to the fp32
+ * accumulator and multiplies by up_scratch before the one rounding of Y.  Both weights are [N, K]
+ * with their own zeros/scales; for a packed weight cat(W_gate, W_up) in layout L1 pass the two
+ * row slices (w_up = w + N * K / 2 bytes, zs_up = zs + N * (K / g) * 4 bytes).  workspace as for
+ * sq_w4a16_gemm_ws (may be NULL).  In the role of gemm_awq_silu_dot_ut, which the reference's
+ * kernel test imports from a package that is not part of it; the expected value and tolerance
+ * are that test's: silu(x W1^T) * (x W2^T) within atol = rtol = 2e-2 (reference:
+ * quantization/nvidia/script/gemm_awq_test.py:50-56,66-72,105). */
+int sq_w4a16_gemm_silu_dot(const void* x, const void* w_gate, const void* zs_gate, const void* w_up,
+                           const void* zs_up, void* y, void* up_scratch, int M, int N, int K,
+                           int group_size, int layout, void* workspace, size_t workspace_bytes,
+                           void* stream);
 
 /* Up to SQ_SEQUENCE_MAX decode linears (1..4 tokens) with one call:
  *     for l in 0 .. count-1:  y_l = act_l(x_l * W_hat_l^T + bias_l) + residual_l

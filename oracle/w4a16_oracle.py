@@ -24,6 +24,8 @@ Pinning status of every function (what, other than this file, fixes it):
   transpose_merge_zeros_scales   index formula; round trip
   gemm_ref              textbook matmul; float64 cross-check; one-hot rows
   rtn_quantize          closed form on hand-computed vectors
+  silu_dot_ref          scipy's logistic function; closed forms (silu(0) = 0, silu(a) - silu(-a) = a,
+                        large |a| limits); x W^T through gemm_ref
   convert_2bit_to_4bit  exhaustive over the 256 byte values
   convert_4bit_to_2bit_l2 / convert_2bit_to_4bit_l2
                         closed-form masks vs the sixteen terms of each loop evaluated
@@ -256,6 +258,18 @@ def gemm_l1(x, w, zs, g):
 def gemm_l2(x, w, zs, g, in_features, out_features):
     y = gemm_ref(x, dequant_l2(w, zs, g, in_features, out_features))
     return y, y.astype(np.float16)
+
+
+def silu_dot_ref(x, w_hat_gate, w_hat_up):
+    """silu(X W_gate_hat^T) * (X W_up_hat^T) in float64, [M, N].
+
+    The expected value of the fused gated-MLP variant as the reference's kernel test computes it
+    (quantization/nvidia/script/gemm_awq_test.py:50-56: matmul, matmul, silu(first) * second),
+    which that test accepts within atol = rtol = 2e-2 (:105).
+    """
+    a = np.asarray(x, dtype=np.float64) @ np.asarray(w_hat_gate, dtype=np.float64).T
+    b = np.asarray(x, dtype=np.float64) @ np.asarray(w_hat_up, dtype=np.float64).T
+    return a / (1.0 + np.exp(-a)) * b
 
 
 # ---------------------------------------------------------------------------

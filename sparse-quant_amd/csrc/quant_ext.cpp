@@ -261,17 +261,92 @@ at::Tensor gemm_awq_residual_ut(at::Tensor I, at::Tensor W, at::Tensor W_zeros_s
     return gemm_impl(I, W, W_zeros_scales, N, group_size, SQ_ALGO_AUTO, c10::nullopt, R, SQ_ACT_NONE);
 }
 
+int act_code(const std::string& act) {
+    if (act == "relu") return SQ_ACT_RELU;
+    if (act == "silu") return SQ_ACT_SILU;
+    if (act != "none" && !act.empty()) throw std::invalid_argument("unknown activation: " + act);
+    return SQ_ACT_NONE;
+}
+
 // act(I W_hat^T + bias) + residual in one launch; bias [N] / residual [bs, seq, N] optional,
-// act "none" or "relu".
+// act "none", "relu" or "silu".
 at::Tensor gemm_awq_fused_ut(at::Tensor I, at::Tensor W, at::Tensor W_zeros_scales, c10::optional<at::Tensor> bias,
                              c10::optional<at::Tensor> residual, const std::string& act, const int N,
                              const int group_size) {
-    int a = SQ_ACT_NONE;
-    if (act == "relu")
-        a = SQ_ACT_RELU;
-    else if (act != "none" && !act.empty())
-        throw std::invalid_argument("unknown activation: " + act);
-    return gemm_impl(I, W, W_zeros_scales, N, group_size, SQ_ALGO_AUTO, bias, residual, a);
+    return gemm_impl(I, W, W_zeros_scales, N, group_size, SQ_ALGO_AUTO, bias, residual, act_code(act));
+}
+
+// silu(I W1_hat^T) * (I W2_hat^T), [bs, seq, N].  Either the two weights with their zeros_scales, or one packed
+// weight cat(W1, W2) along the output dimension (2N outputs) with its zeros_scales; the others None.  Argument
+// order of the fused variant the reference's kernel test imports, which is also where the expected value comes
+// from (reference: quantization/nvidia/script/gemm_awq_test.py:50-56,66-72).
+at::Tensor gemm_awq_silu_dot_ut(at::Tensor I, c10::optional<at::Tensor> W1, c10::optional<at::Tensor> W2,
+                                c10::optional<at::Tensor> ZS1, c10::optional<at::Tensor> ZS2,
+                                c10::optional<at::Tensor> W13, c10::optional<at::Tensor> ZS13, const int M, const int N,
+                                const int K, const int group_size) {
+    (void)M;
+    (void)K;
+    auto has = [](const c10::optional<at::Tensor>& t) { return t.has_value() && t->defined(); };
+    const bool packed = has(W13) && has(ZS13);
+    if (!packed && !(has(W1) && has(W2) && has(ZS1) && has(ZS2)))
+        throw std::invalid_argument("pass W1, W2 and their zeros_scales, or the packed weight and its zeros_scales");
+    SQ_CHECK_DEVICE(I);
+    SQ_CHECK_CONTIGUOUS(I);
+    SQ_CHECK_DTYPE(I, at::kHalf);
+    SQ_CHECK_DIMS(I, 3);
+    const int64_t rows = I.size(0) * I.size(1);
+    const int64_t Kin = I.size(2);
+    if (group_size <= 0 || Kin % group_size != 0) throw std::invalid_argument("embbed dim must be a multiple of group_size!");
+    TORCH_CHECK(rows < (1LL << 31) && Kin < (1LL << 31), "problem too large");
+    c10::DeviceGuard guard(I.device());
+    // Layout L1 views [N, K/2] / [N, 2K/g] of both halves (an int32-layout weight through the conversion cache).
+    auto l1_of = [&](const at::Tensor& W, const at::Tensor& ZS, int n_out) {
+        SQ_CHECK_DEVICE(W);
+        SQ_CHECK_DEVICE(ZS);
+        SQ_CHECK_CONTIGUOUS(W);
+        SQ_CHECK_CONTIGUOUS(ZS);
+        SQ_CHECK_DTYPE(ZS, at::kHalf);
+        SQ_CHECK_DIMS(W, 2);
+        SQ_CHECK_DIMS(ZS, 2);
+        if (layout_of(W) == SQ_LAYOUT_L1) {
+            if (W.size(0) != n_out) throw std::invalid_argument("output dim mismatch!");
+            if (W.size(1) * 2 != Kin) throw std::invalid_argument("input dim mismatch!");
+            if (ZS.size(0) != n_out || ZS.size(1) != 2 * (Kin / group_size))
+                throw std::invalid_argument("zeros_scales shape mismatch!");
+            return std::make_pair(W, ZS);
+        }
+        if (W.size(0) != Kin) throw std::invalid_argument("input dim mismatch!");
+        if (W.size(1) * 8 != n_out) throw std::invalid_argument("output dim mismatch!");
+        if (group_size != 128) throw std::runtime_error("unsupported group size");
+        if (ZS.size(0) != Kin / group_size || ZS.size(1) != 2 * (int64_t)n_out)
+            throw std::invalid_argument("zeros_scales shape mismatch!");
+        return l1_view_of_l2(W, ZS, n_out, (int)Kin, group_size);
+    };
+    std::pair<at::Tensor, at::Tensor> gate, up;
+    if (packed) {
+        const auto both = l1_of(*W13, *ZS13, 2 * N);
+        gate = {both.first.narrow(0, 0, N), both.second.narrow(0, 0, N)};
+        up = {both.first.narrow(0, N, N), both.second.narrow(0, N, N)};
+    } else {
+        gate = l1_of(*W1, *ZS1, N);
+        up = l1_of(*W2, *ZS2, N);
+    }
+    at::Tensor O = torch::empty({I.size(0), I.size(1), N}, I.options());
+    at::Tensor up_out = torch::empty({rows, (int64_t)N}, I.options());
+    void* stream = current_stream(I);
+    void* ws_ptr = nullptr;
+    size_t ws_bytes = 0;
+    at::Tensor ws;
+    if (rows > 2 && rows <= 1024) {
+        ws = workspace_for(I, stream, sq_w4a16_workspace_bytes((int)rows, N, (int)Kin));
+        ws_ptr = ws.data_ptr();
+        ws_bytes = (size_t)ws.numel();
+    }
+    raise_if_error(sq_w4a16_gemm_silu_dot(I.data_ptr(), gate.first.data_ptr(), gate.second.data_ptr(),
+                                          up.first.data_ptr(), up.second.data_ptr(), O.data_ptr(), up_out.data_ptr(),
+                                          (int)rows, N, (int)Kin, group_size, SQ_LAYOUT_L1, ws_ptr, ws_bytes, stream),
+                   "gemm_awq_silu_dot_ut");
+    return O;
 }
 
 // act(LayerNorm(I) W_hat^T + bias) + residual: the pre-LN pattern of a decoder layer (nn.LayerNorm followed by
@@ -281,13 +356,8 @@ at::Tensor gemm_awq_ln_fused_ut(at::Tensor I, c10::optional<at::Tensor> ln_weigh
                                 double ln_eps, at::Tensor W, at::Tensor W_zeros_scales, c10::optional<at::Tensor> bias,
                                 c10::optional<at::Tensor> residual, const std::string& act, const int N,
                                 const int group_size) {
-    int a = SQ_ACT_NONE;
-    if (act == "relu")
-        a = SQ_ACT_RELU;
-    else if (act != "none" && !act.empty())
-        throw std::invalid_argument("unknown activation: " + act);
     const LnArgs ln{ln_weight, ln_bias, ln_eps};
-    return gemm_impl(I, W, W_zeros_scales, N, group_size, SQ_ALGO_AUTO, bias, residual, a, &ln);
+    return gemm_impl(I, W, W_zeros_scales, N, group_size, SQ_ALGO_AUTO, bias, residual, act_code(act), &ln);
 }
 
 // Same with an explicit kernel id (SQ_ALGO_* | tuning word << 8); for tests and benchmarks.
@@ -443,6 +513,10 @@ PYBIND11_MODULE(quant, m) {
     m.def("gemm_awq_ln_fused_ut", &gemm_awq_ln_fused_ut, py::arg("I"), py::arg("ln_weight") = py::none(),
           py::arg("ln_bias") = py::none(), py::arg("ln_eps") = 1e-5, py::arg("W"), py::arg("W_zeros_scales"),
           py::arg("bias") = py::none(), py::arg("residual") = py::none(), py::arg("act") = "none", py::arg("N"),
+          py::arg("group_size"));
+    m.def("gemm_awq_silu_dot_ut", &gemm_awq_silu_dot_ut, py::arg("I"), py::arg("W1") = py::none(),
+          py::arg("W2") = py::none(), py::arg("ZS1") = py::none(), py::arg("ZS2") = py::none(),
+          py::arg("W13") = py::none(), py::arg("ZS13") = py::none(), py::arg("M"), py::arg("N"), py::arg("K"),
           py::arg("group_size"));
     m.def("convert_2bit_to_4bit", &convert_2bit_to_4bit);
     m.def("convert_4bit_to_2bit", &convert_4bit_to_2bit);

@@ -129,6 +129,7 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
                 const int mb = M - m0 < 32 ? M - m0 : 32;
                 sq::Epilogue e = epi;
                 if (e.residual) e.residual += (long)m0 * N;
+                if (e.mul) e.mul += (long)m0 * N;
                 const hipError_t err = sq::launch_skinny2_tuned(
                     static_cast<const sq::half_t*>(x) + (long)m0 * K, w, zs, static_cast<sq::half_t*>(y) + (long)m0 * N,
                     workspace, mb, N, K, group_size, 0, e, st);
@@ -383,11 +384,27 @@ int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int 
 int sq_w4a16_gemm_fused(const void* x, const void* w, const void* zs, const void* bias, const void* residual, void* y,
                         int M, int N, int K, int group_size, int layout, int act, int algo, void* workspace,
                         size_t workspace_bytes, void* stream) {
-    if (act != SQ_ACT_NONE && act != SQ_ACT_RELU) return SQ_ERR_BAD_ALGO;
+    if (act != SQ_ACT_NONE && act != SQ_ACT_RELU && act != SQ_ACT_SILU) return SQ_ERR_BAD_ALGO;
     if (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)) return SQ_ERR_MISALIGNED;
     if (residual && (reinterpret_cast<uintptr_t>(residual) & 1u)) return SQ_ERR_MISALIGNED;
     const sq::Epilogue epi{static_cast<const sq::half_t*>(bias), static_cast<const sq::half_t*>(residual), act};
     return gemm_dispatch(x, w, zs, y, M, N, K, group_size, layout, algo, epi, workspace, workspace_bytes, stream);
+}
+
+int sq_w4a16_gemm_silu_dot(const void* x, const void* w_gate, const void* zs_gate, const void* w_up, const void* zs_up,
+                           void* y, void* up_scratch, int M, int N, int K, int group_size, int layout, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+    if (M > 0 && (!up_scratch || !w_up || !zs_up)) return SQ_ERR_NULL_POINTER;
+    if (M > 0 && !aligned16(up_scratch)) return SQ_ERR_MISALIGNED;
+    if (M > 0 && up_scratch == y) return SQ_ERR_BAD_SHAPE;
+    // the up projection first, rounded to fp16 once; the gate projection multiplies it into its store
+    const int rc = gemm_dispatch(x, w_up, zs_up, up_scratch, M, N, K, group_size, layout, SQ_ALGO_AUTO,
+                                 sq::Epilogue{nullptr, nullptr, SQ_ACT_NONE}, workspace, workspace_bytes, stream);
+    if (rc != SQ_OK || M == 0) return rc;
+    sq::Epilogue epi{nullptr, nullptr, SQ_ACT_SILU};
+    epi.mul = static_cast<const sq::half_t*>(up_scratch);
+    return gemm_dispatch(x, w_gate, zs_gate, y, M, N, K, group_size, layout, SQ_ALGO_AUTO, epi, workspace,
+                         workspace_bytes, stream);
 }
 
 int sq_w4a16_gemm(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
@@ -524,7 +541,7 @@ int sq_w4a16_gemm_ln_fused(const void* x, const void* ln_gamma, const void* ln_b
                            const void* w, const void* zs, const void* bias, const void* residual, void* y, int M, int N,
                            int K, int group_size, int layout, int act, void* workspace, size_t workspace_bytes,
                            void* stream) {
-    if (act != SQ_ACT_NONE && act != SQ_ACT_RELU) return SQ_ERR_BAD_ALGO;
+    if (act != SQ_ACT_NONE && act != SQ_ACT_RELU && act != SQ_ACT_SILU) return SQ_ERR_BAD_ALGO;
     if (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)) return SQ_ERR_MISALIGNED;
     if (residual && (reinterpret_cast<uintptr_t>(residual) & 1u)) return SQ_ERR_MISALIGNED;
     if ((ln_gamma && !aligned16(ln_gamma)) || (ln_beta && !aligned16(ln_beta))) return SQ_ERR_MISALIGNED;

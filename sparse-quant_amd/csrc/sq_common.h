@@ -130,17 +130,125 @@ struct LnPre {
 };
 
 // What happens to an fp32 accumulator on its way to Y[m, n]: + bias[n], activation,
-// + residual[m, n] (each optional), one rounding to fp16 at the end.
+// * mul[m, n], + residual[m, n] (each optional), one rounding to fp16 at the end.
 struct Epilogue {
     const half_t* bias;      // [N] or null
     const half_t* residual;  // [M, N] or null; must not overlap Y
-    int act;                 // 0 = none, 1 = ReLU
+    int act;                 // 0 = none, 1 = ReLU, 2 = SiLU
+    const half_t* mul = nullptr;  // [M, N] or null; must not overlap Y (the other half of a gated MLP)
 };
-__device__ __forceinline__ half_t epilogue(float v, int m, int n, int N, const Epilogue& e) {
+// The tail without SiLU and multiplicand, for the kernels whose launcher hands those cases to another kernel
+// (the 256-row pipelined GEMM: the longer tail changes its register allocation for the worse).
+__device__ __forceinline__ half_t epilogue_linear(float v, int m, int n, int N, const Epilogue& e) {
     if (e.bias) v += (float)e.bias[n];
     if (e.act == 1) v = fmaxf(v, 0.f);
     if (e.residual) v += (float)e.residual[(long)m * N + n];
     return (half_t)v;
+}
+// The full tail with the multiplicand already in a register (1 where there is none).
+__device__ __forceinline__ half_t epilogue_times(float v, float mulv, int m, int n, int N, const Epilogue& e) {
+    if (e.bias) v += (float)e.bias[n];
+    if (e.act == 1)
+        v = fmaxf(v, 0.f);
+    else if (e.act == 2)
+        v = v * __builtin_amdgcn_rcpf(1.f + __expf(-v));  // v * sigmoid(v); exp overflows to +inf for v << 0, the product is -0
+    v *= mulv;
+    if (e.residual) v += (float)e.residual[(long)m * N + n];
+    return (half_t)v;
+}
+__device__ __forceinline__ half_t epilogue(float v, int m, int n, int N, const Epilogue& e) {
+    return epilogue_times(v, e.mul ? (float)e.mul[(long)m * N + n] : 1.f, m, n, N, e);
+}
+
+// Eight consecutive fp16 values as floats: one 128-bit load where the pointer allows it.
+__device__ __forceinline__ void load8_halves(const half_t* p, bool aligned, float (&out)[8]) {
+    if (aligned) {
+        const half8_t h = *(const half8_t*)p;
+#pragma unroll
+        for (int e = 0; e < 8; e++) out[e] = (float)h[e];
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) out[e] = (float)p[e];
+    }
+}
+
+// The tail of the tiled GEMM kernels: a workgroup of four waves holds a (32 MI) x 256 tile of fp32 sums in the
+// matrix instruction's layout (wave w: columns 64 w .. +63; acc[mi][ni][v] of lane (ln, lc) = row
+// 32 mi + 8 (v / 4) + 4 lc + v % 4, column 32 ni + ln).  Stored straight from that layout every lane would issue
+// one 2-byte access per element, and the memory pipeline takes those one lane at a time (128 of them per lane
+// for a 128-row tile, and as many again for each of bias, multiplicand and residual).  Instead each 32-row
+// slice goes through LDS as fp32 and comes back row-major, eight consecutive columns per thread: bias,
+// activation, multiplicand, residual and the one rounding to fp16 happen there, and every global access of the
+// tail is 128 bits wide with neighbouring lanes on neighbouring addresses.  Same operations in the same order as
+// epilogue(): bit-identical results.  lds: 32 KiB of the workgroup's shared memory that nothing else uses any
+// more (the first barrier below separates it from the main loop's reads).  FULL = false leaves SiLU and the
+// multiplicand out (see epilogue_linear).
+template <int MI, bool FULL>
+__device__ __forceinline__ void tile_store_via_lds(const float16_t (&acc)[MI][2], half_t* __restrict__ Y, int M, int N,
+                                                   int m0, int nb, const Epilogue& epi, float* lds) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int ln = lane & 31;
+    const int lc = lane >> 5;
+    const int c8 = tid & 31;  // this thread's chunk of eight columns on the way out
+    const int r0 = tid >> 5;  // and its first row; the others follow in steps of 8
+    const int n = nb + 8 * c8;
+    const bool col_ok = n < N;  // N is a multiple of 8: a chunk is inside or outside as a whole
+    float bias8[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) bias8[e] = 0.f;
+    if (epi.bias && col_ok) load8_halves(epi.bias + n, (reinterpret_cast<uintptr_t>(epi.bias) & 15u) == 0, bias8);
+    const bool res_aligned = (reinterpret_cast<uintptr_t>(epi.residual) & 15u) == 0;
+    const bool mul_aligned = (reinterpret_cast<uintptr_t>(epi.mul) & 15u) == 0;
+#pragma unroll
+    for (int mi = 0; mi < MI; mi++) {
+        __syncthreads();
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+            for (int v = 0; v < 16; v++)
+                lds[(8 * (v >> 2) + 4 * lc + (v & 3)) * 256 + 64 * wave + 32 * ni + ln] = acc[mi][ni][v];
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int r = r0 + 8 * j;
+            const int m = m0 + 32 * mi + r;
+            if (m < M && col_ok) {
+                const float4_t lo = *(const float4_t*)(lds + r * 256 + 8 * c8);
+                const float4_t hi = *(const float4_t*)(lds + r * 256 + 8 * c8 + 4);
+                float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                const long idx = (long)m * N + n;
+                if (epi.bias) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) v[e] += bias8[e];
+                }
+                if (epi.act == 1) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) v[e] = fmaxf(v[e], 0.f);
+                } else if (FULL && epi.act == 2) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) v[e] = v[e] * __builtin_amdgcn_rcpf(1.f + __expf(-v[e]));
+                }
+                if (FULL && epi.mul) {
+                    float t[8];
+                    load8_halves(epi.mul + idx, mul_aligned, t);
+#pragma unroll
+                    for (int e = 0; e < 8; e++) v[e] *= t[e];
+                }
+                if (epi.residual) {
+                    float t[8];
+                    load8_halves(epi.residual + idx, res_aligned, t);
+#pragma unroll
+                    for (int e = 0; e < 8; e++) v[e] += t[e];
+                }
+                half8_t h;
+#pragma unroll
+                for (int e = 0; e < 8; e++) h[e] = (half_t)v[e];
+                *(half8_t*)(Y + idx) = h;
+            }
+        }
+    }
 }
 
 // 128-bit global accesses at the device-coherent level (cache policy sc1, what agent-scope

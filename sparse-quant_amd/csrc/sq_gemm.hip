@@ -34,10 +34,11 @@ constexpr int GEMM_STAGES = 3;  // register stages; loads run GEMM_STAGES - 1 st
 __device__ __forceinline__ int swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
 // What follows the K loop in both tiled kernels: with K split over gridDim.z workgroups the
-// partial tiles meet in the workspace, then the epilogue and the fp16 stores.
+// partial tiles meet in the workspace, then the epilogue and the fp16 stores (through `lds`, 32 KiB
+// of shared memory that the main loop no longer needs).
 template <int MI>
 __device__ __forceinline__ void gemm_tail(float16_t (&acc)[MI][2], half_t* __restrict__ Y, int M, int N, int m0, int n0,
-                                          const Epilogue& epi, float* part, unsigned* counters) {
+                                          const Epilogue& epi, float* part, unsigned* counters, float* lds) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int ln = lane & 31;
@@ -111,18 +112,7 @@ __device__ __forceinline__ void gemm_tail(float16_t (&acc)[MI][2], half_t* __res
         if (tid == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
-    // Epilogue: fp32 -> fp16, 32 consecutive columns per half-wave.
-#pragma unroll
-    for (int mi = 0; mi < MI; mi++)
-#pragma unroll
-        for (int ni = 0; ni < 2; ni++) {
-            const int n = n0 + 32 * ni + ln;
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int m = m0 + 32 * mi + 8 * (v >> 2) + 4 * lc + (v & 3);
-                if (m < M && n < N) Y[(long)m * N + n] = epilogue(acc[mi][ni][v], m, n, N, epi);
-            }
-        }
+    tile_store_via_lds<MI, true>(acc, Y, M, N, m0, n0 - 64 * (tid >> 6), epi, lds);
 }
 
 // Two waves per SIMD (two workgroups per CU): one wave alone cannot both issue the
@@ -137,7 +127,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     // 16-byte chunks of row R are stored at chunk position c ^ swz(R); 8 consecutive
     // rows then use 8 distinct positions and 16 consecutive rows 16 distinct 16-byte
     // slots of a 256-byte bank period, so the 128-bit operand reads are conflict free.
-    __shared__ __attribute__((aligned(1024))) uint8_t xs[2][BM * 128];
+    // (at least 16 KiB per stage: the tail passes the tile through these 32 KiB)
+    __shared__ __attribute__((aligned(1024))) uint8_t xs[2][BM * 128 < 16384 ? 16384 : BM * 128];
 
     const NibbleMasks nm = nibble_masks();
     const int tid = threadIdx.x;
@@ -284,7 +275,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         step(it + 5, std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
     }
 
-    gemm_tail<MI>(acc, Y, M, N, m0, n0, epi, part, counters);
+    gemm_tail<MI>(acc, Y, M, N, m0, n0, epi, part, counters, reinterpret_cast<float*>(&xs[0][0]));
 }
 
 // Both operands through LDS, for group sizes 32, 64 and 128 and K a multiple of 256.  The kernels above hand
@@ -452,7 +443,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         if constexpr (P == 4) zc ^= 1;
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the last two steps' loads ran ahead of the range
-    gemm_tail<MI>(acc, Y, M, N, m0, n0, epi, part, counters);
+    gemm_tail<MI>(acc, Y, M, N, m0, n0, epi, part, counters, reinterpret_cast<float*>(lds));
 }
 
 constexpr int GEMM_COUNTER_BYTES = 65536;  // start of the workspace: one uint32 per output tile
@@ -578,14 +569,21 @@ hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void*
     int mi = tune & 0x3F;
     int ksplit = (tune >> 8) & 0xFF;
     bool lds = (tune & 0x80) != 0;
-    if (mi >= 8 && mi <= 10) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, mi - 8, epi, st);
-    if (mi != 1 && mi != 2 && mi != 4) {
+    // The pipelined kernels store bias / ReLU / residual only; SiLU or a multiplicand goes through the 128-row
+    // tile kernel (both operands through LDS where that applies).
+    const bool plain_tail = epi.act != 2 && epi.mul == nullptr;
+    if (mi >= 8 && mi <= 10) {
+        if (plain_tail) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, mi - 8, epi, st);
+        mi = 4;
+        ksplit = 1;
+        lds = true;
+    } else if (mi != 1 && mi != 2 && mi != 4) {
         const bool have_ws = ws != nullptr && ws_bytes >= plan_bytes(plan_gemm(M, N, K, g, true), M, N);
         const GemmPlan p = plan_gemm(M, N, K, g, have_ws);
-        if (p.pipe >= 0) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, p.pipe, epi, st);
-        mi = p.mi;
-        ksplit = p.ksplit;
-        lds = p.lds != 0;
+        if (p.pipe >= 0 && plain_tail) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, p.pipe, epi, st);
+        mi = p.pipe >= 0 ? 4 : p.mi;
+        ksplit = p.pipe >= 0 ? 1 : p.ksplit;
+        lds = p.pipe >= 0 ? true : p.lds != 0;
     } else {
         if (ksplit != 2 && ksplit != 4 && ksplit != 8) ksplit = 1;
         const long tiles = (long)((N + 255) / 256) * ((M + 32 * mi - 1) / (32 * mi));

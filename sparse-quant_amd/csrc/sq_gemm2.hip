@@ -176,17 +176,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
         step(it + 5, std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{});
     }
 
-#pragma unroll
-    for (int mi = 0; mi < MI; mi++)
-#pragma unroll
-        for (int ni = 0; ni < 2; ni++) {
-            const int n = n0 + 32 * ni + ln;
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int m = m0 + 32 * mi + 8 * (v >> 2) + 4 * lc + (v & 3);
-                if (m < M && n < N) Y[(long)m * N + n] = epilogue(acc[mi][ni][v], m, n, N, epi);
-            }
-        }
+    // the two activation stages (at least 32 KiB) carry the tile on its way out
+    tile_store_via_lds<MI, false>(acc, Y, M, N, m0, blockIdx.x * G2_BN, epi, reinterpret_cast<float*>(&xs[0][0]));
 }
 
 template <int MI, int OCC>

@@ -29,6 +29,7 @@ SIGNATURES = {
     "sq_w4a16_gemm_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp]),
     "sq_w4a16_gemm_static_ws": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
     "sq_w4a16_gemm_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp]),
+    "sq_w4a16_gemm_silu_dot": (_i, [_vp] * 7 + [_i] * 5 + [_vp, ctypes.c_size_t, _vp]),
     "sq_w4a16_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
     "sq_workspace_reset": (_i, [_vp, ctypes.c_size_t, _vp]),
     "sq_workspace_check": (_i, [_vp, ctypes.c_size_t, _vp]),
@@ -205,7 +206,7 @@ def gemm_static_ws(x, w, zs, n, k, group_size, algo=SQ_ALGO_AUTO, out=None, stre
     return out
 
 
-SQ_ACT_NONE, SQ_ACT_RELU = 0, 1
+SQ_ACT_NONE, SQ_ACT_RELU, SQ_ACT_SILU = 0, 1, 2
 
 
 def gemm_fused(x, w, zs, n, k, group_size, bias=None, residual=None, act=SQ_ACT_NONE, algo=SQ_ALGO_AUTO, out=None,
@@ -220,6 +221,21 @@ def gemm_fused(x, w, zs, n, k, group_size, bias=None, residual=None, act=SQ_ACT_
                                      group_size, SQ_LAYOUT_L1, act, algo, _ptr(ws), 0 if ws is None else ws.numel(),
                                      _stream(stream)), "sq_w4a16_gemm_fused")
     return out
+
+
+def gemm_silu_dot(x, w_gate, zs_gate, w_up, zs_up, n, k, group_size, out=None, stream=None, ws=None, use_workspace=True,
+                  up_out=None):
+    """y = silu(x W_gate_hat^T) * (x W_up_hat^T) through sq_w4a16_gemm_silu_dot; returns (y, up projection)."""
+    m = x.numel() // k
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
+    up = up_out if up_out is not None else torch.empty((m, n), dtype=torch.float16, device=x.device)
+    if ws is None and use_workspace and 2 < m <= 1024:
+        ws = workspace(m, n, k, x.device, stream)
+    _check(lib().sq_w4a16_gemm_silu_dot(_ptr(x), _ptr(w_gate), _ptr(zs_gate), _ptr(w_up), _ptr(zs_up), _ptr(out), _ptr(up),
+                                        m, n, k, group_size, SQ_LAYOUT_L1, _ptr(ws), 0 if ws is None else ws.numel(),
+                                        _stream(stream)), "sq_w4a16_gemm_silu_dot")
+    return out, up
 
 
 def gemm_ln_fused(x, ln_gamma, ln_beta, ln_eps, w, zs, n, k, group_size, bias=None, residual=None, act=SQ_ACT_NONE,

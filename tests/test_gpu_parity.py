@@ -514,8 +514,10 @@ def fused_ref(x, w_hat, bias, residual, act):
     y = orc.gemm_ref(x, w_hat).astype(np.float64)
     if bias is not None:
         y = y + bias.astype(np.float64)[None, :]
-    if act:
+    if act == 1:
         y = np.maximum(y, 0.0)
+    elif act == 2:
+        y = y / (1.0 + np.exp(-y))
     if residual is not None:
         y = y + residual.astype(np.float64)
     return y
@@ -531,7 +533,8 @@ FUSED_CASES = [  # (m, n, k, g, algo name, tune) -- one per kernel family and ti
 
 
 @pytest.mark.parametrize("m,n,k,g,algo_name,tune", FUSED_CASES)
-@pytest.mark.parametrize("use_bias,use_res,act", [(True, False, 0), (False, True, 0), (True, True, 1), (False, False, 1)])
+@pytest.mark.parametrize("use_bias,use_res,act", [(True, False, 0), (False, True, 0), (True, True, 1), (False, False, 1),
+                                                  (True, True, 2)])
 def test_fused_epilogue_every_kernel(capi, m, n, k, g, algo_name, tune, use_bias, use_res, act):
     d = linear(n, k, g, seed=31)
     rng = np.random.default_rng(32)
@@ -546,7 +549,7 @@ def test_fused_epilogue_every_kernel(capi, m, n, k, g, algo_name, tune, use_bias
     y = y.float().cpu().numpy()
     scale = np.max(np.abs(orc.gemm_ref(x, d["w_hat"])))
     assert np.max(np.abs(y - y_ref)) <= TOL * scale
-    if act and not use_res:
+    if act == 1 and not use_res:
         assert y.min() >= 0.0
 
 
@@ -570,6 +573,76 @@ def test_fused_epilogue_is_exactly_the_unfused_sum_in_fp32(capi):
                         algo=capi.SQ_ALGO_GEMV).cpu().numpy()
     want = (d["w_hat"][:, 77].astype(np.float32) + bias.astype(np.float32) + res[0].astype(np.float32)).astype(np.float16)
     assert np.array_equal(y[0].view(np.int16), want.view(np.int16))
+
+
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 16, 24, 32, 40, 100, 300])
+@pytest.mark.parametrize("n,k,g", [(512, 1024, 128), (264, 704, 64)])
+def test_gated_mlp_front_half(capi, m, n, k, g):
+    """silu(x W_gate^T) * (x W_up^T) through sq_w4a16_gemm_silu_dot against the oracle, within this
+    suite's bar relative to the largest output (every decode, streaming and tiled kernel of the
+    automatic dispatch takes a turn over these token counts); the scratch tensor holds the up projection."""
+    gate = linear(n, k, g, seed=51)
+    up = linear(n, k, g, seed=52)
+    x = orc.synth_x(m, k, seed=53)
+    want = orc.silu_dot_ref(x, gate["w_hat"], up["w_hat"])
+    y, up_out = capi.gemm_silu_dot(to_dev(x), gate["w_dev"], gate["zs_dev"], up["w_dev"], up["zs_dev"], n, k, g)
+    torch.cuda.synchronize()
+    got = y.float().cpu().numpy().astype(np.float64)
+    assert np.max(np.abs(got - want)) <= TOL * np.max(np.abs(want))
+    up_ref = orc.gemm_ref(x, up["w_hat"])
+    assert np.max(np.abs(up_out.float().cpu().numpy() - up_ref)) <= TOL * np.max(np.abs(up_ref))
+
+
+def test_gated_mlp_rejections(capi):
+    n, k, g = 256, 1024, 128
+    d = linear(n, k, g, seed=0)
+    x = to_dev(orc.synth_x(2, k))
+    y = torch.empty((2, n), dtype=torch.float16, device=DEV)
+    L = capi.lib()
+    p = lambda t: t.data_ptr()
+    args = (p(x), p(d["w_dev"]), p(d["zs_dev"]), p(d["w_dev"]), p(d["zs_dev"]))
+    assert L.sq_w4a16_gemm_silu_dot(*args, p(y), None, 2, n, k, g, capi.SQ_LAYOUT_L1, None, 0, None) == capi.SQ_ERR_NULL_POINTER
+    assert L.sq_w4a16_gemm_silu_dot(*args, p(y), p(y), 2, n, k, g, capi.SQ_LAYOUT_L1, None, 0, None) == capi.SQ_ERR_BAD_SHAPE
+    assert L.sq_w4a16_gemm_silu_dot(*args, p(y), p(y) + 2, 2, n, k, g, capi.SQ_LAYOUT_L1, None, 0, None) == capi.SQ_ERR_MISALIGNED
+    assert L.sq_w4a16_gemm_silu_dot(*args, p(y), p(x), 2, n, k, 48, capi.SQ_LAYOUT_L1, None, 0, None) == capi.SQ_ERR_BAD_GROUP
+    assert L.sq_w4a16_gemm_silu_dot(*args, p(y), None, 0, n, k, g, capi.SQ_LAYOUT_L1, None, 0, None) == capi.SQ_OK
+
+
+@pytest.mark.parametrize("m", [1, 8, 128])
+def test_quant_extension_gated_mlp(m):
+    """gemm_awq_silu_dot_ut with the call shapes, the data recipe and the tolerance of the reference's kernel
+    test (nn.Linear weights through the packer, x ~ N(0, 0.5), two weights or one packed weight with 2N
+    outputs, allclose at atol = rtol = 2e-2; quantization/nvidia/script/gemm_awq_test.py:50-56,66-72,92-105),
+    in both layouts; the expected value is the oracle's on the dequantised weights."""
+    import quant
+    from sqamd import quant_funcs as qf
+    torch.manual_seed(7)
+    n, k, g = 256, 1024, 128
+    lin1 = torch.nn.Linear(k, n, bias=False, device=DEV, dtype=torch.float16)
+    lin2 = torch.nn.Linear(k, n, bias=False, device=DEV, dtype=torch.float16)
+    qw1, zs1 = qf.quant_muxi(lin1.weight.data, k, n, n_bit=4, group_size=g)
+    qw2, zs2 = qf.quant_muxi(lin2.weight.data, k, n, n_bit=4, group_size=g)
+    w_hat1 = orc.dequant_l1(qw1.cpu().numpy(), zs1.cpu().numpy(), g)
+    w_hat2 = orc.dequant_l1(qw2.cpu().numpy(), zs2.cpu().numpy(), g)
+    xd = torch.empty((1, m, k), dtype=torch.float16, device=DEV).normal_(mean=0.0, std=0.5)
+    want = orc.silu_dot_ref(xd.cpu().numpy().reshape(m, k), w_hat1, w_hat2)
+
+    def check(out):
+        assert tuple(out.shape) == (1, m, n) and out.dtype == torch.float16
+        got = out.float().cpu().numpy().reshape(m, n).astype(np.float64)
+        assert np.all(np.abs(got - want) <= 2e-2 + 2e-2 * np.abs(want))
+        assert np.max(np.abs(got - want)) <= TOL * np.max(np.abs(want))
+
+    check(quant.gemm_awq_silu_dot_ut(xd, qw1, qw2, zs1, zs2, None, None, m, n, k, g))
+    w13 = torch.cat((lin1.weight.data, lin2.weight.data), dim=0).contiguous()
+    qw13, zs13 = qf.quant_muxi(w13, k, 2 * n, n_bit=4, group_size=g)
+    assert torch.equal(qw13, torch.cat((qw1, qw2), dim=0))
+    check(quant.gemm_awq_silu_dot_ut(xd, None, None, None, None, qw13, zs13, m, n, k, g))
+    qw13_l2, zs13_l2, _ = qf.quant_lmdeploy(w13, k, 2 * n, group_size=g, n_bit=4)
+    check(quant.gemm_awq_silu_dot_ut(xd, None, None, None, None, qw13_l2, zs13_l2, m, n, k, g))
+    with pytest.raises(ValueError):
+        quant.gemm_awq_silu_dot_ut(xd, qw1, None, zs1, None, None, None, m, n, k, g)
+    quant.clear_repack_cache()
 
 
 def test_fused_rejects_bad_activation(capi):

@@ -320,6 +320,25 @@ def test_two_bit_kat_and_exhaustive():
         assert out[v, 0] == (a | (bb << 4)) and out[v, 1] == (c | (d << 4))
 
 
+def test_silu_dot_closed_forms():
+    from scipy.special import expit
+    rng = np.random.default_rng(5)
+    x = rng.normal(0, 1, size=(3, 16))
+    wg = rng.normal(0, 1, size=(5, 16))
+    wu = rng.normal(0, 1, size=(5, 16))
+    a, b = x @ wg.T, x @ wu.T
+    got = orc.silu_dot_ref(x, wg, wu)
+    assert np.allclose(got, a * expit(a) * b, rtol=1e-12, atol=1e-12)  # library logistic function
+    # silu(a) - silu(-a) = a, so flipping the gate weight changes the result by exactly a * b
+    assert np.allclose(got - orc.silu_dot_ref(x, -wg, wu), a * b, rtol=1e-12, atol=1e-12)
+    # a zero gate gives zero; a saturated gate passes a * b (positive side) or nothing (negative side)
+    assert np.all(orc.silu_dot_ref(x, np.zeros_like(wg), wu) == 0)
+    g = orc.silu_dot_ref(np.eye(4), np.diag([40.0, -40.0, 0.0, 1.0]), 3.0 * np.eye(4))
+    assert np.allclose(np.diag(g), [120.0, 0.0, 0.0, 3.0 / (1.0 + np.exp(-1.0))], atol=1e-12)
+    # the two projections are not interchangeable
+    assert not np.allclose(got, orc.silu_dot_ref(x, wu, wg))
+
+
 def _int32_sum(terms):
     """Sum as torch's int32 `+=` gives it: modulo 2**32."""
     return sum(terms) & 0xFFFFFFFF
