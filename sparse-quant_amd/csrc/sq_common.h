@@ -137,14 +137,6 @@ struct Epilogue {
     int act;                 // 0 = none, 1 = ReLU, 2 = SiLU
     const half_t* mul = nullptr;  // [M, N] or null; must not overlap Y (the other half of a gated MLP)
 };
-// The tail without SiLU and multiplicand, for the kernels whose launcher hands those cases to another kernel
-// (the 256-row pipelined GEMM: the longer tail changes its register allocation for the worse).
-__device__ __forceinline__ half_t epilogue_linear(float v, int m, int n, int N, const Epilogue& e) {
-    if (e.bias) v += (float)e.bias[n];
-    if (e.act == 1) v = fmaxf(v, 0.f);
-    if (e.residual) v += (float)e.residual[(long)m * N + n];
-    return (half_t)v;
-}
 // The full tail with the multiplicand already in a register (1 where there is none).
 __device__ __forceinline__ half_t epilogue_times(float v, float mulv, int m, int n, int N, const Epilogue& e) {
     if (e.bias) v += (float)e.bias[n];
@@ -181,9 +173,8 @@ __device__ __forceinline__ void load8_halves(const half_t* p, bool aligned, floa
 // activation, multiplicand, residual and the one rounding to fp16 happen there, and every global access of the
 // tail is 128 bits wide with neighbouring lanes on neighbouring addresses.  Same operations in the same order as
 // epilogue(): bit-identical results.  lds: 32 KiB of the workgroup's shared memory that nothing else uses any
-// more (the first barrier below separates it from the main loop's reads).  FULL = false leaves SiLU and the
-// multiplicand out (see epilogue_linear).
-template <int MI, bool FULL>
+// more (the first barrier below separates it from the main loop's reads).
+template <int MI>
 __device__ __forceinline__ void tile_store_via_lds(const float16_t (&acc)[MI][2], half_t* __restrict__ Y, int M, int N,
                                                    int m0, int nb, const Epilogue& epi, float* lds) {
     const int tid = threadIdx.x;
@@ -226,11 +217,11 @@ __device__ __forceinline__ void tile_store_via_lds(const float16_t (&acc)[MI][2]
                 if (epi.act == 1) {
 #pragma unroll
                     for (int e = 0; e < 8; e++) v[e] = fmaxf(v[e], 0.f);
-                } else if (FULL && epi.act == 2) {
+                } else if (epi.act == 2) {
 #pragma unroll
                     for (int e = 0; e < 8; e++) v[e] = v[e] * __builtin_amdgcn_rcpf(1.f + __expf(-v[e]));
                 }
-                if (FULL && epi.mul) {
+                if (epi.mul) {
                     float t[8];
                     load8_halves(epi.mul + idx, mul_aligned, t);
 #pragma unroll

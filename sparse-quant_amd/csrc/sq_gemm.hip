@@ -112,7 +112,7 @@ __device__ __forceinline__ void gemm_tail(float16_t (&acc)[MI][2], half_t* __res
         if (tid == 0) __hip_atomic_store(&counters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
-    tile_store_via_lds<MI, true>(acc, Y, M, N, m0, n0 - 64 * (tid >> 6), epi, lds);
+    tile_store_via_lds<MI>(acc, Y, M, N, m0, n0 - 64 * (tid >> 6), epi, lds);
 }
 
 // Two waves per SIMD (two workgroups per CU): one wave alone cannot both issue the
@@ -569,21 +569,14 @@ hipError_t launch_gemm_tuned(const void* x, const void* w, const void* zs, void*
     int mi = tune & 0x3F;
     int ksplit = (tune >> 8) & 0xFF;
     bool lds = (tune & 0x80) != 0;
-    // The pipelined kernels store bias / ReLU / residual only; SiLU or a multiplicand goes through the 128-row
-    // tile kernel (both operands through LDS where that applies).
-    const bool plain_tail = epi.act != 2 && epi.mul == nullptr;
-    if (mi >= 8 && mi <= 10) {
-        if (plain_tail) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, mi - 8, epi, st);
-        mi = 4;
-        ksplit = 1;
-        lds = true;
-    } else if (mi != 1 && mi != 2 && mi != 4) {
+    if (mi >= 8 && mi <= 10) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, mi - 8, epi, st);
+    if (mi != 1 && mi != 2 && mi != 4) {
         const bool have_ws = ws != nullptr && ws_bytes >= plan_bytes(plan_gemm(M, N, K, g, true), M, N);
         const GemmPlan p = plan_gemm(M, N, K, g, have_ws);
-        if (p.pipe >= 0 && plain_tail) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, p.pipe, epi, st);
-        mi = p.pipe >= 0 ? 4 : p.mi;
-        ksplit = p.pipe >= 0 ? 1 : p.ksplit;
-        lds = p.pipe >= 0 ? true : p.lds != 0;
+        if (p.pipe >= 0) return launch_gemm_pipe(x, w, zs, y, M, N, K, g, p.pipe, epi, st);
+        mi = p.mi;
+        ksplit = p.ksplit;
+        lds = p.lds != 0;
     } else {
         if (ksplit != 2 && ksplit != 4 && ksplit != 8) ksplit = 1;
         const long tiles = (long)((N + 255) / 256) * ((M + 32 * mi - 1) / (32 * mi));

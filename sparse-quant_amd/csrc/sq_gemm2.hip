@@ -177,7 +177,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
     }
 
     // the two activation stages (at least 32 KiB) carry the tile on its way out
-    tile_store_via_lds<MI, false>(acc, Y, M, N, m0, blockIdx.x * G2_BN, epi, reinterpret_cast<float*>(&xs[0][0]));
+    tile_store_via_lds<MI>(acc, Y, M, N, m0, blockIdx.x * G2_BN, epi, reinterpret_cast<float*>(&xs[0][0]));
 }
 
 template <int MI, int OCC>
