@@ -291,7 +291,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 //   * activations: the swizzled chunk order of the register-staged kernel, written by the load
 //     instead of a store;
 //   * zeros/scales: the two pairs of 2 g columns (four steps at group size 128, two at 64, one
-//     at 32), one dword per lane and pair.
+//     at 32), one dword per lane, two neighbouring lanes on the two pairs of a row.
 // Three stages (two for zeros/scales, three at group size 32), loads two steps ahead; one barrier per step, behind a
 // counted wait for the loads of the next step (the loads just issued stay in flight).  Same
 // operand mapping and arithmetic as gemm_kernel: bit-identical results.
@@ -343,12 +343,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
         const int r = 32 * i + (lane >> 1);
         wlane[i] = (uint32_t)((long)imin(n0 + r, N - 1) * (K >> 1) + 16 * ((lane & 1) ^ ((r >> 3) & 1)));
     }
-    const uint32_t zlane = (uint32_t)((long)imin(n0 + lane, N - 1) * groups * 4);  // lane = row of the wave's 64
+    // zeros/scales: instruction i moves the two pairs of rows 32 i .. 32 i + 31, two neighbouring lanes per row
+    // (8 contiguous bytes), so that it touches 32 places in memory rather than 64
+    uint32_t zlane[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+        zlane[i] = (uint32_t)((long)imin(n0 + 32 * i + (lane >> 1), N - 1) * groups * 4 + (lane & 1) * 4);
     int woff[2], zoff[2];
 #pragma unroll
     for (int ni = 0; ni < 2; ni++) {
         woff[ni] = W_OFF + wave * 2048 + ((32 * ni + ln) * 2 + (lc ^ ((ln >> 3) & 1))) * 16;
-        zoff[ni] = Z_OFF + wave * 512 + (32 * ni + ln) * 4 + (GS == 5 ? lc * 256 : 0);  // g = 32: the pair of the lane's half
+        zoff[ni] = Z_OFF + wave * 512 + ni * 256 + ln * 8 + (GS == 5 ? lc * 4 : 0);  // g = 32: the pair of the lane's half
     }
     int xoff[4];
 #pragma unroll
@@ -376,8 +381,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
     // The two zeros/scales pairs of the P steps that start at step `it`, into stage zc.
     auto issue_zs = [&](int it, int zc) {
         const half2_t* zb = ZS + imin((it * GEMM_BK) >> GS, groups - 2);
-        load_to_lds_x1(zb, zlane, lds0 + Z_OFF + zc * ZB + wave * 512);
-        load_to_lds_x1(zb + 1, zlane, lds0 + Z_OFF + zc * ZB + wave * 512 + 256);
+        load_to_lds_x1(zb, zlane[0], lds0 + Z_OFF + zc * ZB + wave * 512);
+        load_to_lds_x1(zb, zlane[1], lds0 + Z_OFF + zc * ZB + wave * 512 + 256);
     };
 
     // One K step: J = step within its group of four, c = its stage, cf = the stage read in the step
@@ -395,7 +400,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void g
 #pragma unroll
         for (int ni = 0; ni < 2; ni++) {
             q[ni] = *(const u32x4_t*)(lds + c * WB + woff[ni]);
-            const half2_t zsv = *(const half2_t*)(lds + zcur * ZB + (P == 4 ? (j >> 1) : (P == 2 ? (j & 1) : 0)) * 256 + zoff[ni]);
+            const half2_t zsv = *(const half2_t*)(lds + zcur * ZB + (P == 4 ? (j >> 1) : (P == 2 ? (j & 1) : 0)) * 4 + zoff[ni]);
             const half_t sv = kin ? zsv.y : (half_t)0.f;
             z64[ni] = (half2_t){zsv.x, zsv.x};
             sc[ni] = (half2_t){sv, sv};
