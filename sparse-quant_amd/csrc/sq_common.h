@@ -152,6 +152,40 @@ __device__ __forceinline__ half_t epilogue(float v, int m, int n, int N, const E
     return epilogue_times(v, e.mul ? (float)e.mul[(long)m * N + n] : 1.f, m, n, N, e);
 }
 
+// Four consecutive outputs of one row (n a multiple of 4; N is a multiple of 8, so they are inside or outside
+// together) whose bias and residual are requested ahead of the data they meet: the last workgroup of a K split
+// asks for them before it fetches the partial tiles, so that the two round trips overlap.
+struct Tail4 {
+    u32x2_t bias, res;
+};
+__device__ __forceinline__ bool tail4_applies(const Epilogue& e) {
+    return e.mul == nullptr && (reinterpret_cast<uintptr_t>(e.bias) & 7u) == 0 &&
+           (reinterpret_cast<uintptr_t>(e.residual) & 7u) == 0;
+}
+__device__ __forceinline__ Tail4 tail4_request(const Epilogue& e, int m, int n, int N, bool inside) {
+    Tail4 t = {{0u, 0u}, {0u, 0u}};
+    if (e.bias && inside) t.bias = *(const u32x2_t*)(e.bias + n);
+    if (e.residual && inside) t.res = *(const u32x2_t*)(e.residual + (long)m * N + n);
+    return t;
+}
+__device__ __forceinline__ void tail4_store(float4_t v, const Tail4& t, half_t* __restrict__ Y, int m, int n, int N,
+                                            const Epilogue& e) {
+    const half4_t b = bit_cast<half4_t>(t.bias), r = bit_cast<half4_t>(t.res);
+    half4_t o;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float x = v[i];
+        if (e.bias) x += (float)b[i];
+        if (e.act == 1)
+            x = fmaxf(x, 0.f);
+        else if (e.act == 2)
+            x = x * __builtin_amdgcn_rcpf(1.f + __expf(-x));
+        if (e.residual) x += (float)r[i];
+        o[i] = (half_t)x;
+    }
+    *(half4_t*)(Y + (long)m * N + n) = o;
+}
+
 // Eight consecutive fp16 values as floats: one 128-bit load where the pointer allows it.
 __device__ __forceinline__ void load8_halves(const half_t* p, bool aligned, float (&out)[8]) {
     if (aligned) {

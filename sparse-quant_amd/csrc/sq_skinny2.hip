@@ -279,7 +279,16 @@ __device__ __forceinline__ void skinny2_body(const uint8_t* __restrict__ W, cons
     }
     __syncthreads();
     if (!last_flag) return;
+    const bool fast_tail = tail4_applies(epi);
     for (int t4 = tid * 4; t4 < TILE; t4 += 4 * 64 * NWV) {
+        // the four elements t4 .. t4 + 3 are one token and four consecutive rows of the weight; their bias and
+        // residual are requested ahead of the partial tiles
+        const int l4 = t4 & 63, v4 = (t4 >> 6) & 3, mt4 = (t4 >> 8) % MT, rt4 = (t4 >> 8) / MT;
+        const int m4 = 16 * mt4 + 4 * (l4 >> 4) + v4;
+        const int n4 = rb * ROWS + 16 * rt4 + (l4 & 15);
+        const bool inside = m4 < M && n4 < N;
+        Tail4 pre = {{0u, 0u}, {0u, 0u}};
+        if (fast_tail) pre = tail4_request(epi, m4, n4, N, inside);
         // eight loads regardless of ksplit (absent partials re-read partial 0 and are dropped)
         const float* src[8];
 #pragma unroll
@@ -290,14 +299,13 @@ __device__ __forceinline__ void skinny2_body(const uint8_t* __restrict__ W, cons
 #pragma unroll
         for (int q = 1; q < 8; q++)
             if (q < ksplit) sum += pv[q];  // fixed order
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int t = t4 + e;
-            const int l = t & 63, v = (t >> 6) & 3, mt = (t >> 8) % MT, rt = (t >> 8) / MT;
-            const int m = 16 * mt + 4 * (l >> 4) + v;
-            const int n = rb * ROWS + 16 * rt + (l & 15);
-            if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum[e], m, n, N, epi);
+        if (fast_tail) {
+            if (inside) tail4_store(sum, pre, Y, m4, n4, N, epi);
+            continue;
         }
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            if (inside) Y[(long)m4 * N + n4 + e] = epilogue(sum[e], m4, n4 + e, N, epi);
     }
     // leave the workspace ready for the next call
     if (tid == 0) __hip_atomic_store(&counters[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
