@@ -645,6 +645,33 @@ def test_quant_extension_gated_mlp(m):
     quant.clear_repack_cache()
 
 
+@pytest.mark.parametrize("m,n,k,g", [(300, 520, 1056, 32), (70, 264, 1024, 128), (24, 256, 8192, 128), (8, 256, 16384, 128),
+                                     (2048, 512, 1024, 128)])
+def test_fused_epilogue_operands_at_odd_addresses(capi, m, n, k, g):
+    """bias and residual only need 2-byte alignment: the tiled kernels' tile store and the split-K decode
+    kernels' four-column tail fall back from their wide loads, same results as with aligned operands."""
+    d = linear(n, k, g, seed=71)
+    rng = np.random.default_rng(72)
+    x = to_dev(orc.synth_x(m, k, seed=73))
+    bias = rng.normal(0, 2.0, size=n).astype(np.float16)
+    res = rng.normal(0, 2.0, size=(m, n)).astype(np.float16)
+    bias_buf = torch.zeros(n + 8, dtype=torch.float16, device=DEV)
+    res_buf = torch.zeros(m * n + 8, dtype=torch.float16, device=DEV)
+    outs = []
+    for off in (0, 1, 4):  # 16-byte, 2-byte and 8-byte aligned
+        b = bias_buf[off:off + n]
+        r = res_buf[off:off + m * n].view(m, n)
+        b.copy_(to_dev(bias))
+        r.copy_(to_dev(res))
+        assert b.data_ptr() % 16 == 2 * off
+        y = capi.gemm_fused(x, d["w_dev"], d["zs_dev"], n, k, g, bias=b, residual=r, act=capi.SQ_ACT_RELU)
+        torch.cuda.synchronize()
+        outs.append(y.clone())
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    want = fused_ref(x.cpu().numpy(), d["w_hat"], bias, res, 1)
+    assert np.max(np.abs(outs[0].float().cpu().numpy() - want)) <= TOL * np.max(np.abs(orc.gemm_ref(x.cpu().numpy(), d["w_hat"])))
+
+
 def test_fused_rejects_bad_activation(capi):
     d = linear(256, 1024, 128, seed=0)
     x = to_dev(orc.synth_x(2, 1024))
