@@ -332,7 +332,9 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     sk3_barrier();
 
     // Element t of the tile: lane l = t % 64, v, rt -> token m = 4 (l / 16) + v, row n = ROWS rb + 16 rt + l % 16.
-    if (ksplit == 1) {
+    if (ksplit == 1 && RT == 1) {
+        // a 16-row workgroup has 256 elements: one per thread is faster than four for a quarter of the threads
+        // (4096 x 4096 at 8 tokens: 5.0 against 5.4 us)
         for (int t = tid; t < TILE; t += SK3_NT) {
             float sum = 0.f;
 #pragma unroll
@@ -341,6 +343,30 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
             const int m = 4 * (l >> 4) + v;
             const int n = rb * ROWS + 16 * rt + (l & 15);
             if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum, m, n, N, epi);
+        }
+        return;
+    }
+    if (ksplit == 1) {
+        // four consecutive elements per thread: one token, four consecutive rows of the weight, so that bias,
+        // residual and result travel as 64-bit accesses
+        const bool fast_tail = tail4_applies(epi);
+        for (int t4 = tid * 4; t4 < TILE; t4 += 4 * SK3_NT) {
+            const int l4 = t4 & 63, v4 = (t4 >> 6) & 3, rt4 = t4 >> 8;
+            const int m4 = 4 * (l4 >> 4) + v4;
+            const int n4 = rb * ROWS + 16 * rt4 + (l4 & 15);
+            const bool inside = m4 < M && n4 < N;
+            Tail4 pre = {{0u, 0u}, {0u, 0u}};
+            if (fast_tail) pre = tail4_request(epi, m4, n4, N, inside);
+            float4_t sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int p = 0; p < SK3_NWV; p++) sum += *(const float4_t*)(&red[p * TILE + t4]);
+            if (fast_tail) {
+                if (inside) tail4_store(sum, pre, Y, m4, n4, N, epi);
+                continue;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (inside) Y[(long)m4 * N + n4 + e] = epilogue(sum[e], m4, n4 + e, N, epi);
         }
         return;
     }
@@ -588,14 +614,26 @@ __device__ __forceinline__ void skinny3_wide_body(const uint8_t* __restrict__ W,
 
     // Element t of the tile: lane l = t % 64, v, mt, rt -> token m = 16 mt + 4 (l / 16) + v, row n = 64 rb + 16 rt + l % 16.
     if (ksplit == 1) {
-        for (int t = tid; t < TILE; t += SK3_NT) {
-            float sum = 0.f;
+        // four consecutive elements per thread: one token, four consecutive rows of the weight, so that bias,
+        // residual and result travel as 64-bit accesses
+        const bool fast_tail = tail4_applies(epi);
+        for (int t4 = tid * 4; t4 < TILE; t4 += 4 * SK3_NT) {
+            const int l4 = t4 & 63, v4 = (t4 >> 6) & 3, mt4 = (t4 >> 8) % MT, rt4 = (t4 >> 8) / MT;
+            const int m4 = 16 * mt4 + 4 * (l4 >> 4) + v4;
+            const int n4 = rb * ROWS + 16 * rt4 + (l4 & 15);
+            const bool inside = m4 < M && n4 < N;
+            Tail4 pre = {{0u, 0u}, {0u, 0u}};
+            if (fast_tail) pre = tail4_request(epi, m4, n4, N, inside);
+            float4_t sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int p = 0; p < SK3_NWV; p++) sum += *red(p, t);
-            const int l = t & 63, v = (t >> 6) & 3, mt = (t >> 8) % MT, rt = (t >> 8) / MT;
-            const int m = 16 * mt + 4 * (l >> 4) + v;
-            const int n = rb * ROWS + 16 * rt + (l & 15);
-            if (m < M && n < N) Y[(long)m * N + n] = epilogue(sum, m, n, N, epi);
+            for (int p = 0; p < SK3_NWV; p++) sum += *(const float4_t*)red(p, t4);
+            if (fast_tail) {
+                if (inside) tail4_store(sum, pre, Y, m4, n4, N, epi);
+                continue;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (inside) Y[(long)m4 * N + n4 + e] = epilogue(sum[e], m4, n4 + e, N, epi);
         }
         return;
     }
