@@ -5,6 +5,7 @@ token rows (all N columns of each), which keeps the fp32 reference matmul to sec
   * prefill: M in {2048, 4096} on the five prefill shapes (4096x4096, 4096->16384, 16384->4096,
     4096->11008, 11008->4096), group 128, through the C ABI and through quant.gemm_awq_ut, the
     int32 tensor-core layout included (weights packed by the oracle, not by the package);
+  * the gated MLP front half at the Llama-7B size (two 11008 x 4096 weights) at 1, 8 and 2048 tokens;
   * LUT attention at batch 8, 16 heads, head dim 64, 4096 tokens, 25 % density, non-causal, on
     sampled (batch, head) pairs;
   * one full-width OPT-6.7B decoder layer (hidden 4096, FFN 16384, 32 heads, batch 8, 640-row cache)
@@ -76,6 +77,35 @@ def test_prefill_full_size_against_oracle(capi, n, k):
         # the rows that were not sampled: finite, and the two call paths agree on the whole output
         assert torch.isfinite(y_abi).all()
         assert torch.equal(y_abi, y_ext.view(m, n))
+
+
+@pytest.mark.parametrize("m", [1, 8, 2048])
+def test_gated_mlp_llama_size_against_oracle(capi, m):
+    """silu(x W_gate^T) * (x W_up^T) at the Llama-7B MLP size (two 11008 x 4096 weights, group 128): the fused
+    entry point and the extension's packed call shape against the oracle on sampled token rows, with bias-free
+    weights packed by the oracle; the scratch tensor holds the plain up projection."""
+    import quant
+    n, k, g = 11008, 4096, 128
+    gate = orc.synth_linear(n, k, g, seed=5)
+    up = orc.synth_linear(n, k, g, seed=6)
+    wg_hat = orc.dequant_l1(gate["w_l1"], gate["zs_l1"], g)
+    wu_hat = orc.dequant_l1(up["w_l1"], up["zs_l1"], g)
+    x = orc.synth_x(m, k, seed=m)
+    rows = sample_rows(m, 32, seed=m) if m > 64 else np.arange(m)
+    want = orc.silu_dot_ref(x[rows], wg_hat, wu_hat)
+    xd = to_dev(x)
+    wg, zg, wu, zu = (to_dev(a) for a in (gate["w_l1"], gate["zs_l1"], up["w_l1"], up["zs_l1"]))
+    print("gated mlp parity m=%d" % m, flush=True)
+    y, up_out = capi.gemm_silu_dot(xd, wg, zg, wu, zu, n, k, g)
+    w13 = torch.cat((wg, wu), dim=0).contiguous()
+    zs13 = torch.cat((zg, zu), dim=0).contiguous()
+    y_ext = quant.gemm_awq_silu_dot_ut(xd.view(1, m, k), None, None, None, None, w13, zs13, m, n, k, g)
+    torch.cuda.synchronize()
+    idx = torch.from_numpy(rows).to(DEV)
+    assert rel_err(y[idx].float().cpu().numpy(), want) <= TOL
+    assert rel_err(up_out[idx].float().cpu().numpy(), orc.gemm_ref(x[rows], wu_hat)) <= TOL
+    assert torch.isfinite(y).all()
+    assert torch.equal(y, y_ext.view(m, n))
 
 
 @pytest.mark.parametrize("n,k", [(4096, 4096), (4096, 11008)])
