@@ -36,18 +36,6 @@ int sq_read_probe(const void* w, const void* zs, void* out, int N, int K, int gr
  * prefill figures). */
 int sq_mfma_probe(const void* data, void* out, int workgroups, int iters, void* stream);
 
-/* sq_w4a16_gemv_sequence (include/sq_w4a16.h) in its time-stamping instantiation: the same
- * persistent kernel on `count` (1..8) linears without epilogue, arguments as parallel arrays of
- * length count, M in 1..4, workspace as for the product call.  trace receives 64 uint64 per
- * workgroup (one workgroup per CU), readings of the constant 100 MHz counter: 0 start, 1 first
- * activations staged, then for linear l at 2 + 4l: streaming wave 0 done with the linear's weights,
- * control waves done storing Y, grid barrier passed, next activations staged; 60 streaming wave 0
- * leaves, 61 control waves leave.  Shows where a sequence spends its time (barriers against
- * streaming). */
-int sq_sequence_trace(const void* const* x, const void* const* w, const void* const* zs, void* const* y,
-                      const int* N, const int* K, const int* depends, int count, int M, int group_size,
-                      void* workspace, void* trace, void* stream);
-
 /* a single wave spins for `spins`
  * (1 .. 2^26) dependent multiply-adds and writes three uint64 to out: shader-clock
  * ticks elapsed, ticks of the constant 100 MHz counter elapsed, and a dummy.  Run on

@@ -37,6 +37,7 @@ extern "C" {
 #define SQ_ERR_LAUNCH 7          /* the HIP runtime rejected the launch */
 #define SQ_ERR_WORKSPACE 8       /* workspace missing or too small */
 #define SQ_ERR_STATIC_WS 9       /* sq_w4a16_gemm_static_ws: the shape needs more than SQ_STATIC_WS_BYTES */
+#define SQ_ERR_SEQ_TIMEOUT 10    /* sq_w4a16_gemv_sequence_status: a one-launch sequence gave up a wait */
 
 #define SQ_LAYOUT_L1 1
 #define SQ_LAYOUT_L2 2
@@ -185,23 +186,37 @@ int sq_w4a16_gemm_silu_dot(const void* x, const void* w_gate, const void* zs_gat
  *            earlier linear of the same call.  Linears without it may run ahead of earlier ones.
  *            A buffer written by linear i may be read or overwritten by linear j > i only if j, or
  *            a linear between them, has depends set; y_l must not alias x_l or residual_l.
- *   mode     SQ_SEQ_AUTO: as above (the kernel boundary is the cheapest dependency on this part);
+ *   mode     SQ_SEQ_AUTO: as above;
  *            SQ_SEQ_ONE_LAUNCH: everything in one persistent launch (one workgroup per CU stays
- *            resident, the weight stream never stops between linears, dependencies are honoured by a
- *            grid barrier inside the kernel); faster than one launch per linear only when nothing
- *            depends on anything, kept for that case and for measurement.
+ *            resident and the weight stream runs on across the linears).  There is no grid
+ *            barrier: an output that a later linear of the call reads (x_j or residual_j is exactly
+ *            the buffer y_i, same address and extent) is also written to the workspace as 8-byte
+ *            words {two fp16, launch tag}, and the reader repeats its load until the tags are the
+ *            launch's, so a dependency costs one store and one load; meanwhile the waiting
+ *            workgroup keeps fetching the next weights into LDS.  Needs 1..4 tokens, one group size
+ *            for all linears, bias and residual 4-byte aligned, activations of a linear within LDS
+ *            (M * K * 2 bytes up to about 64 KiB), a data flow it can see (depends set only where a
+ *            pointer matches an earlier y; no output that aliases a buffer an unordered linear
+ *            still reads) and every workgroup resident at once (one per CU: the GPU otherwise idle;
+ *            other work delays it, and a workgroup that never becomes resident makes the others'
+ *            waits run out).  Whatever does not fit is launched as under SQ_SEQ_AUTO.
  *   workspace  NULL, or sq_w4a16_gemv_sequence_workspace_bytes(linears, count, M) bytes, 16-byte
- *            aligned, its first 64 KiB zero before the first call (every call leaves them zero);
- *            calls that share it must be ordered.  With 1 or 2 tokens it is used by
- *            SQ_SEQ_ONE_LAUNCH only (256 bytes); with 3..32 tokens it is the split-K workspace of
- *            sq_w4a16_gemm_ws, sized for the linears that may share a launch.
- *            Word 9 of it is a sticky error flag: it becomes 1 if a grid barrier ever ran out of
- *            polls (results of that call are then undefined).
+ *            aligned, ALL of it zero before the first call; calls that share it must be ordered and
+ *            must describe the same list.  Its first part is the split-K workspace of
+ *            sq_w4a16_gemm_ws (64 KiB of counters, every call leaves them zero, and with 3..32
+ *            tokens the partial tiles of the linears that may share a launch); behind it lies the
+ *            region of SQ_SEQ_ONE_LAUNCH (launch number, sticky error word, exit counter, exchange
+ *            words), which only that mode touches.
+ * sq_w4a16_gemv_sequence_status (the one call here that SYNCHRONISES) reads that region back:
+ * SQ_OK, SQ_ERR_SEQ_TIMEOUT if a wait for another workgroup's output ever ran out of polls since
+ * the word was last cleared (the results of that call are undefined; `clear` != 0 resets the word
+ * with a fill kernel on `stream`), SQ_ERR_WORKSPACE if a launch did not finish.
+ * sq_w4a16_gemv_sequence_tune sets, process-wide, the number of polls a wait may take (default
+ * 65536, each a round trip to memory) and the loads a streaming wave keeps in flight (0 = default,
+ * at most 16); tests use a poll limit of 0 to drive the give-up path from the host.
  * Shapes as for sq_w4a16_gemm (all linears share M).  A lone linear, M > 32, and whatever does not
  * fit the rules above is launched linear by linear on the stream (the automatic dispatch of
- * sq_w4a16_gemm_ws): same results.  SQ_SEQ_ONE_LAUNCH falls back to the same when there is no workspace, M > 4, or the
- * activations of a linear do not fit the LDS (M * K * 2 bytes beyond about 128 KiB); its persistent
- * kernel needs every workgroup resident at once (one per CU); other work on the GPU only delays it. */
+ * sq_w4a16_gemm_ws): same results. */
 #define SQ_SEQ_AUTO 0
 #define SQ_SEQ_ONE_LAUNCH 1
 #define SQ_SEQUENCE_MAX 8
@@ -219,6 +234,9 @@ typedef struct sq_linear_desc {
 int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int layout, int mode,
                            void* workspace, size_t workspace_bytes, void* stream);
 size_t sq_w4a16_gemv_sequence_workspace_bytes(const sq_linear_desc* linears, int count, int M);
+int sq_w4a16_gemv_sequence_status(const sq_linear_desc* linears, int count, int M, void* workspace,
+                                  size_t workspace_bytes, int clear, void* stream);
+int sq_w4a16_gemv_sequence_tune(unsigned spin_limit, int loads_in_flight);
 
 /* out[N,K] (fp16) = W_hat in natural k order, bit-identical to fp16
  * (q_fp16 - z_fp16) * s_fp16.  Replaces dequant

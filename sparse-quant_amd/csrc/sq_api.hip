@@ -202,6 +202,7 @@ const char* sq_strerror(int code) {
         case SQ_ERR_LAUNCH: return "HIP kernel launch failed";
         case SQ_ERR_WORKSPACE: return "workspace missing or too small";
         case SQ_ERR_STATIC_WS: return "problem needs a larger workspace than the library's static buffer (SQ_STATIC_WS_BYTES)";
+        case SQ_ERR_SEQ_TIMEOUT: return "a one-launch sequence gave up waiting for another workgroup's output (results of that call are undefined)";
         default: return "unknown error code";
     }
 }
@@ -267,21 +268,69 @@ int sq_workspace_check(const void* workspace, size_t bytes, void* stream) {
     return SQ_OK;
 }
 
-size_t sq_w4a16_gemv_sequence_workspace_bytes(const sq_linear_desc* linears, int count, int M) {
-    size_t need = sq::gemv_seq_workspace_bytes();
-    if (!linears || count <= 0 || count > SQ_SEQUENCE_MAX || M <= 2) return need;
+static void to_problems(const sq_linear_desc* linears, int count, sq::SeqProblem* probs) {
+    for (int l = 0; l < count; l++) {
+        const sq_linear_desc& d = linears[l];
+        probs[l] = sq::SeqProblem{d.x, d.w, d.zs, d.bias, d.residual, d.y, d.N, d.K, d.group_size, d.act, d.depends};
+    }
+}
+
+// A sequence's workspace: first what the split-K kernels of the launch-per-linear path want (64 KiB of counters
+// and the partial tiles; nothing beyond the counters up to 2 tokens), then, 256-byte aligned, the region of the
+// one-launch kernel (control block and exchange words), which no other kernel writes.
+static size_t sequence_splitk_bytes(const sq_linear_desc* linears, int count, int M) {
+    const size_t base = 65536;
+    if (!linears || count <= 0 || count > SQ_SEQUENCE_MAX || M <= 2) return base;
     // more than 2 tokens: what sq_w4a16_gemm_ws wants for the largest run of linears that may share a launch
     // (their rows concatenated, each rounded up to a 64-row block) and for every single linear
     long rows = 0;
     int kmax = 0;
     for (int l = 0; l < count; l++) {
-        if (linears[l].N <= 0 || linears[l].K <= 0) return need;
+        if (linears[l].N <= 0 || linears[l].K <= 0) return base;
         rows += ((long)linears[l].N + 63) / 64 * 64;
         if (linears[l].K > kmax) kmax = linears[l].K;
     }
-    if (rows > (1L << 30)) return need;
-    const size_t a = sq_w4a16_workspace_bytes(M, (int)rows, kmax);
-    return a > need ? a : need;
+    if (rows > (1L << 30)) return base;
+    const size_t a = (sq_w4a16_workspace_bytes(M, (int)rows, kmax) + 255) & ~(size_t)255;
+    return a > base ? a : base;
+}
+
+size_t sq_w4a16_gemv_sequence_workspace_bytes(const sq_linear_desc* linears, int count, int M) {
+    sq::SeqProblem probs[SQ_SEQUENCE_MAX];
+    const bool listed = linears && count > 0 && count <= SQ_SEQUENCE_MAX;
+    if (listed) to_problems(linears, count, probs);
+    return sequence_splitk_bytes(linears, count, M) + sq::gemv_seq_workspace_bytes(listed ? probs : nullptr, count, M);
+}
+
+int sq_w4a16_gemv_sequence_status(const sq_linear_desc* linears, int count, int M, void* workspace,
+                                  size_t workspace_bytes, int clear, void* stream) {
+    if (!linears || !workspace) return SQ_ERR_NULL_POINTER;
+    if (count <= 0 || count > SQ_SEQUENCE_MAX) return SQ_ERR_BAD_SHAPE;
+    const size_t off = sequence_splitk_bytes(linears, count, M);
+    if (!aligned16(workspace) || workspace_bytes < off + 256) return SQ_ERR_WORKSPACE;
+    unsigned* ctrl = reinterpret_cast<unsigned*>(static_cast<uint8_t*>(workspace) + off);
+    unsigned host[4] = {0, 0, 0, 0};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (hipMemcpyAsync(host, ctrl, sizeof(host), hipMemcpyDeviceToHost, st) != hipSuccess) return SQ_ERR_LAUNCH;
+    if (hipStreamSynchronize(st) != hipSuccess) return SQ_ERR_LAUNCH;
+    if (clear && host[1] != 0u) {
+        hipLaunchKernelGGL(zero_words_kernel, dim3(1), dim3(64), 0, st, ctrl + 1, 1);
+        if (hipGetLastError() != hipSuccess) return SQ_ERR_LAUNCH;
+    }
+    if (host[2] != 0u) return SQ_ERR_WORKSPACE;  // an exit counter that is not back at zero: a launch did not finish
+    return host[1] != 0u ? SQ_ERR_SEQ_TIMEOUT : SQ_OK;
+}
+
+// Tuning of the persistent sequence kernel (sq_w4a16_gemv_sequence_tune): polls allowed for another workgroup's
+// output, and loads a streaming wave keeps in flight (0: the kernel's default).
+static unsigned g_seq_spin_limit = 1u << 16;
+static int g_seq_lim = 0;
+
+int sq_w4a16_gemv_sequence_tune(unsigned spin_limit, int loads_in_flight) {
+    if (loads_in_flight < 0 || loads_in_flight > 16) return SQ_ERR_BAD_SHAPE;
+    g_seq_spin_limit = spin_limit;
+    g_seq_lim = loads_in_flight;
+    return SQ_OK;
 }
 
 int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int layout, int mode, void* workspace,
@@ -309,11 +358,13 @@ int sq_w4a16_gemv_sequence(const sq_linear_desc* linears, int count, int M, int 
     }
     if (M == 0) return SQ_OK;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const bool ws_ok = workspace && aligned16(workspace) && workspace_bytes >= sq::gemv_seq_workspace_bytes();
     if (workspace && !aligned16(workspace)) workspace = nullptr;
-    if (mode == SQ_SEQ_ONE_LAUNCH && ws_ok && M <= 4) {
-        // everything in one persistent launch, dependencies honoured by a grid barrier inside the kernel
-        const int rc = sq::launch_gemv_seq(probs, count, M, workspace, 1u << 20, st);
+    if (mode == SQ_SEQ_ONE_LAUNCH && workspace && M <= 4) {
+        // everything in one persistent launch; outputs that later linears read travel as tagged words
+        const size_t off = sequence_splitk_bytes(linears, count, M);
+        const int rc = workspace_bytes > off ? sq::launch_gemv_seq(probs, count, M, static_cast<uint8_t*>(workspace) + off,
+                                                                   workspace_bytes - off, g_seq_spin_limit, g_seq_lim, st)
+                                             : 1;
         if (rc == 0) return SQ_OK;
         if (rc == 2) return SQ_ERR_LAUNCH;
     }

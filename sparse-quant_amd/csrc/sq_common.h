@@ -306,21 +306,20 @@ __device__ __forceinline__ void load8_coherent_x4(const float* const (&p)[8], fl
 // later LDS read wait for ALL outstanding vector memory loads unless it can prove the two apart,
 // which it cannot for stages picked at run time.  The kernel orders them itself (a counted
 // s_waitcnt and a barrier per step); the "memory" clobbers keep LDS reads from moving across.
+// The LDS address travels in m0, bound as an input so that the compiler knows the register is written.
 __device__ __forceinline__ void load_to_lds_x4(const void* g, uint32_t lds_byte) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "s"(lds_byte) : "memory");
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(g), "{m0}"(lds_byte) : "memory");
 }
 __device__ __forceinline__ void load_to_lds_x1(const void* g, uint32_t lds_byte) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "s"(lds_byte) : "memory");
+    asm volatile("s_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(g), "{m0}"(lds_byte) : "memory");
 }
 // The same with the address split into a wave-uniform base and a 32-bit byte offset per lane: a loop that
 // walks along K then advances one scalar instead of one 64-bit sum per lane and load.
 __device__ __forceinline__ void load_to_lds_x4(const void* base, uint32_t lane_byte, uint32_t lds_byte) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_byte), "s"(base), "s"(lds_byte)
-                 : "memory");
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_byte), "s"(base), "{m0}"(lds_byte) : "memory");
 }
 __device__ __forceinline__ void load_to_lds_x1(const void* base, uint32_t lane_byte, uint32_t lds_byte) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(lane_byte), "s"(base), "s"(lds_byte)
-                 : "memory");
+    asm volatile("s_nop 0\n\tglobal_load_lds_dword %0, %1" ::"v"(lane_byte), "s"(base), "{m0}"(lds_byte) : "memory");
 }
 
 // Sixteen coherent 128-bit loads in flight: p[i] points at the SECOND of two locations 4096 bytes

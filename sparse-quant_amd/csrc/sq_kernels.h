@@ -49,13 +49,17 @@ hipError_t launch_gemv2_group(const SeqProblem* probs, int count, int M, hipStre
 // sq_w4a16_gemm_ws, at least skinny2_group_workspace_bytes().
 size_t skinny2_group_workspace_bytes(const SeqProblem* probs, int count, int M);
 hipError_t launch_skinny2_group(const SeqProblem* probs, int count, int M, void* ws, size_t ws_bytes, hipStream_t st);
-size_t gemv_seq_workspace_bytes();
-// 0: launched; 1: the sequence does not fit this kernel (the caller launches the linears one by
-// one); 2: the HIP runtime rejected the launch.  workspace: gemv_seq_workspace_bytes() bytes, zero
-// between launches.  spin_limit bounds the polls of a grid barrier.
-// trace (diagnostic, normally null): 64 uint64 per workgroup, time stamps of the 100 MHz counter.
-int launch_gemv_seq(const SeqProblem* probs, int count, int M, void* workspace, unsigned spin_limit, hipStream_t st,
-                    unsigned long long* trace = nullptr);
+// sq_gemv_seq.hip: up to SEQ_MAX_LINEARS decode linears (M <= 4) in one persistent launch; outputs that later
+// linears of the list read travel between workgroups as tagged words in the workspace.
+// gemv_seq_workspace_bytes: a control block of 256 bytes ([0] launch number, [1] sticky error word, [2] exit
+// counter) + the exchange words; a region of its own, 256-byte aligned, that no other kernel writes.
+size_t gemv_seq_workspace_bytes(const SeqProblem* probs, int count, int M);
+// 0: launched; 1: the sequence does not fit this kernel (the caller launches the linears one by one);
+// 2: the HIP runtime rejected the launch.  The workspace's control block and exchange words are zero before the
+// first launch.  spin_limit bounds the polls for another workgroup's output; lim = loads a streaming wave keeps
+// in flight (0: default).
+int launch_gemv_seq(const SeqProblem* probs, int count, int M, void* workspace, size_t workspace_bytes,
+                    unsigned spin_limit, int lim, hipStream_t st);
 
 // sq_skinny.hip: M <= 64.  tune = waves | mode << 8 (mode 1 = exact, 2 = fixup).
 hipError_t launch_skinny_tuned(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int g,

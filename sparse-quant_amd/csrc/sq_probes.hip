@@ -162,24 +162,6 @@ int sq_mfma_probe(const void* data, void* out, int workgroups, int iters, void* 
     return launch_code(sq::launch_mfma_probe(data, out, workgroups, iters, static_cast<hipStream_t>(stream)));
 }
 
-int sq_sequence_trace(const void* const* x, const void* const* w, const void* const* zs, void* const* y, const int* N,
-                      const int* K, const int* depends, int count, int M, int group_size, void* workspace, void* trace,
-                      void* stream) {
-    if (!x || !w || !zs || !y || !N || !K || !depends || !workspace || !trace) return SQP_ERR_NULL_POINTER;
-    if (count < 1 || count > sq::SEQ_MAX_LINEARS || M < 1 || M > 4) return SQP_ERR_BAD_SHAPE;
-    if (group_size != 32 && group_size != 64 && group_size != 128) return SQP_ERR_BAD_SHAPE;
-    sq::SeqProblem p[sq::SEQ_MAX_LINEARS];
-    for (int l = 0; l < count; l++) {
-        if (!x[l] || !w[l] || !zs[l] || !y[l]) return SQP_ERR_NULL_POINTER;
-        if (N[l] <= 0 || K[l] <= 0 || N[l] % 8 != 0 || K[l] % 32 != 0 || K[l] % group_size != 0) return SQP_ERR_BAD_SHAPE;
-        if (!aligned16(x[l]) || !aligned16(w[l]) || !aligned16(zs[l]) || !aligned16(y[l])) return SQP_ERR_MISALIGNED;
-        p[l] = sq::SeqProblem{x[l], w[l], zs[l], nullptr, nullptr, y[l], N[l], K[l], group_size, 0, depends[l]};
-    }
-    const int rc = sq::launch_gemv_seq(p, count, M, workspace, 1u << 20, static_cast<hipStream_t>(stream),
-                                       static_cast<unsigned long long*>(trace));
-    return rc == 0 ? SQP_OK : (rc == 1 ? SQP_ERR_BAD_SHAPE : SQP_ERR_LAUNCH);
-}
-
 int sq_clock_probe(void* out, int spins, void* stream) {
     if (!out) return SQP_ERR_NULL_POINTER;
     if (spins <= 0 || spins > (1 << 26)) return SQP_ERR_BAD_SHAPE;

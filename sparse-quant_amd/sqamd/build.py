@@ -75,9 +75,7 @@ def build_lib(verbose=True):
     with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
         list(pool.map(compile_one, zip(sources, objs)))
     n = len(HIP_SOURCES)
-    # the diagnostic library carries its own copy of the sequence kernel (for its time-stamping instantiation)
-    seq_obj = [o for o in objs[:n] if o.endswith("sq_gemv_seq.o")]
-    for path, part in ((LIB_PATH, objs[:n]), (PROBES_PATH, objs[n:] + seq_obj)):
+    for path, part in ((LIB_PATH, objs[:n]), (PROBES_PATH, objs[n:])):
         _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", path] + part +
              ["-Wl,-rpath," + os.path.join(ROCM, "lib")])
         if verbose:

@@ -57,7 +57,6 @@ PROBE_SIGNATURES = {
     "sq_clock_probe": (_i, [_vp, _i, _vp]),
     "sq_mfma_probe": (_i, [_vp, _vp, _i, _i, _vp]),
     "sq_read_probe": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
-    "sq_sequence_trace": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp]),
 }
 
 
@@ -71,6 +70,9 @@ class LinearDesc(ctypes.Structure):
 SIGNATURES["sq_w4a16_gemv_sequence"] = (_i, [ctypes.POINTER(LinearDesc), _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp])
 SQ_SEQ_AUTO, SQ_SEQ_ONE_LAUNCH = 0, 1
 SIGNATURES["sq_w4a16_gemv_sequence_workspace_bytes"] = (ctypes.c_size_t, [ctypes.POINTER(LinearDesc), _i, _i])
+SIGNATURES["sq_w4a16_gemv_sequence_tune"] = (_i, [ctypes.c_uint, _i])
+SIGNATURES["sq_w4a16_gemv_sequence_status"] = (_i, [ctypes.POINTER(LinearDesc), _i, _i, _vp, ctypes.c_size_t, _i, _vp])
+SQ_ERR_SEQ_TIMEOUT = 10
 SQ_SEQUENCE_MAX = 8
 
 _lib = None
@@ -283,9 +285,21 @@ class LinearSequence:
         _check(self._fn(self.descs, self.count, self.m, SQ_LAYOUT_L1, self.mode, _ptr(self.ws),
                         0 if self.ws is None else self.ws.numel(), _stream(stream)), "sq_w4a16_gemv_sequence")
 
-    def error_flag(self):
-        """The sticky error word of the workspace (synchronises): non-zero if a grid barrier ran out of polls."""
-        return 0 if self.ws is None else int(self.ws.view(torch.int32)[9].item())
+    def error_flag(self, clear=False, stream=None):
+        """1 if a wait of the one-launch kernel for another workgroup's output ever ran out of polls since the
+        word was last cleared, else 0 (synchronises; sq_w4a16_gemv_sequence_status)."""
+        if self.ws is None:
+            return 0
+        rc = lib().sq_w4a16_gemv_sequence_status(self.descs, self.count, self.m, _ptr(self.ws), self.ws.numel(),
+                                                 int(bool(clear)), _stream(stream))
+        if rc not in (SQ_OK, SQ_ERR_SEQ_TIMEOUT):
+            raise SqError(rc, "sq_w4a16_gemv_sequence_status")
+        return int(rc == SQ_ERR_SEQ_TIMEOUT)
+
+
+def sequence_tune(spin_limit=1 << 16, loads_in_flight=0):
+    """Process-wide tuning of the one-launch sequence kernel: polls allowed per wait, loads a wave keeps in flight."""
+    _check(lib().sq_w4a16_gemv_sequence_tune(int(spin_limit), int(loads_in_flight)), "sq_w4a16_gemv_sequence_tune")
 
 
 def dequant(w, zs, n, k, group_size, layout=SQ_LAYOUT_L1, stream=None):
@@ -419,21 +433,6 @@ def layernorm(x, gamma, beta, eps=1e-5, out=None, stream=None):
     _check(lib().sq_layernorm(_ptr(x), _ptr(gamma), _ptr(beta), _ptr(out), x.numel() // cols, cols, float(eps),
                               _stream(stream)), "sq_layernorm")
     return out
-
-
-def sequence_trace(linears, m, group_size, stream=None):
-    """Run the linears (dicts with x, w, zs, y, n, k, depends) through the time-stamping instantiation of the
-    sequence kernel; returns an int64 tensor [workgroups, 64] of 100 MHz counter readings (see sq_probes.h)."""
-    cnt = len(linears)
-    dev = linears[0]["x"].device
-    arr = lambda key: (ctypes.c_void_p * cnt)(*[l[key].data_ptr() for l in linears])
-    ints = lambda key: (ctypes.c_int * cnt)(*[int(l.get(key, 0)) for l in linears])
-    ws = torch.zeros(256, dtype=torch.uint8, device=dev)
-    cus = torch.cuda.get_device_properties(dev).multi_processor_count
-    trace = torch.zeros((cus, 64), dtype=torch.int64, device=dev)
-    _check(probes().sq_sequence_trace(arr("x"), arr("w"), arr("zs"), arr("y"), ints("n"), ints("k"), ints("depends"), cnt,
-                                      int(m), int(group_size), _ptr(ws), _ptr(trace), _stream(stream)), "sq_sequence_trace")
-    return trace
 
 
 def mfma_probe(data, workgroups, iters, stream=None):

@@ -78,7 +78,7 @@ def test_independent_linears_of_mixed_shapes(capi, m):
 
 
 @pytest.mark.parametrize("mode", ["auto", "one_launch"])
-@pytest.mark.parametrize("m", [1, 4])
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
 def test_dependent_chain_with_epilogues(capi, m, mode):
     """y0 = relu(x W0 + b0); y1 = y0 W1 + b1 + x; y2 = y1 W2; y3 = relu(y1 W3) + y2: every linear consumes what an
     earlier one of the same launch wrote (input and residual), against the same chain through the oracle with
@@ -184,6 +184,117 @@ def test_opt67_layer_linears_in_one_launch(capi, m, mode):
     assert seq.error_flag() == 0 and capi.workspace_is_clean(seq.ws)  # counters; partial tiles may stay
 
 
+def _chained_opt_layer(capi, m, seed=11, x_scale=1.0 / 64):
+    """The six linears of an OPT-6.7B decoder layer wired as a chain of real buffers: q, k, v read x; out_proj reads
+    q's output, fc1 (ReLU, bias) reads out_proj's, fc2 reads fc1's and adds out_proj's output as residual."""
+    g = 128
+    shapes = [(4096, 4096), (4096, 4096), (4096, 4096), (4096, 4096), (16384, 4096), (4096, 16384)]
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(seed)
+    x = (torch.randn((m, 4096), device=DEV, generator=gen) * x_scale).half()
+    ys = [torch.full((m, n), float("nan"), dtype=torch.float16, device=DEV) for n, _ in shapes]
+    xin = [x, x, x, ys[0], ys[3], ys[4]]
+    lin = []
+    for idx, (n, k) in enumerate(shapes):
+        w = torch.randint(0, 256, (n, k // 2), dtype=torch.uint8, device=DEV, generator=gen)
+        z = torch.randint(0, 16, (n, k // g), device=DEV, generator=gen).half() + 64
+        s = (torch.randn((n, k // g), device=DEV, generator=gen).abs() * 0.02 + 1e-3).half()
+        zs = torch.stack([z, s], dim=-1).reshape(n, 2 * (k // g)).contiguous()
+        lin.append(dict(x=xin[idx], w=w, zs=zs, y=ys[idx], n=n, k=k, group_size=g, depends=idx >= 3))
+    lin[4]["bias"] = (torch.randn(16384, device=DEV, generator=gen) * 0.1).half()
+    lin[4]["act"] = capi.SQ_ACT_RELU
+    lin[5]["residual"] = ys[3]
+    return lin, ys, x
+
+
+def _check_chain_against_oracle(lin, rng, tol=5e-3):
+    """Every linear against the oracle on sampled output rows, fed with the input the device actually read."""
+    for l in lin:
+        n, k, g = l["n"], l["k"], l["group_size"]
+        rows = np.sort(rng.choice(n, size=64, replace=False))
+        rows[0], rows[-1] = 0, n - 1
+        ridx = torch.from_numpy(rows).to(DEV)
+        w_hat = orc.dequant_l1(l["w"][ridx].cpu().numpy(), l["zs"][ridx].cpu().numpy(), g)
+        ref = orc.gemm_ref(l["x"].cpu().numpy(), w_hat).astype(np.float64)
+        if l.get("bias") is not None:
+            ref = ref + l["bias"][ridx].float().cpu().numpy()[None, :]
+        if l.get("act"):
+            ref = np.maximum(ref, 0.0)
+        if l.get("residual") is not None:
+            ref = ref + l["residual"][:, ridx].float().cpu().numpy()
+        assert torch.isfinite(l["y"]).all()
+        assert rel_err(l["y"][:, ridx].float().cpu().numpy(), ref) <= tol, (n, k)
+
+
+@pytest.mark.parametrize("m", [1, 2, 3, 4])
+def test_opt67_layer_chained_in_one_launch(capi, m):
+    """The decoder layer's linears with their real data flow in ONE persistent launch: the outputs that later
+    linears read travel between workgroups as tagged words.  Oracle per linear on the inputs the device read;
+    eager launches and HIP-graph replays give the same bits; the launch counter advances, nothing times out."""
+    lin, ys, _ = _chained_opt_layer(capi, m)
+    seq = capi.LinearSequence(lin, m, DEV, mode=capi.SQ_SEQ_ONE_LAUNCH)
+    seq.run()
+    torch.cuda.synchronize()
+    _check_chain_against_oracle(lin, np.random.default_rng(m))
+    first = [y.clone() for y in ys]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        seq.run(stream=side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            seq.run(stream=side)
+    for rep in range(4):
+        for y in ys:
+            y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for y, f in zip(ys, first):
+            assert torch.equal(y, f)
+    assert seq.error_flag() == 0 and capi.workspace_is_clean(seq.ws)
+    # the same chain through a launch per dependent linear
+    lin2, ys2, _ = _chained_opt_layer(capi, m)
+    capi.LinearSequence(lin2, m, DEV, mode=capi.SQ_SEQ_AUTO).run()
+    torch.cuda.synchronize()
+    for a, b in zip(ys, ys2):
+        assert (a.float() - b.float()).abs().max().item() <= 1e-2 * max(b.float().abs().max().item(), 1e-3)
+
+
+def test_one_launch_gives_up_cleanly(capi):
+    """With no polls allowed, a wait for another workgroup's output gives up at once: the launch still ends, the
+    sticky error word is reported, the split-K counters in front of it stay zero and a split-K launch on the same
+    workspace is right; after the word is cleared and polls are allowed again the same sequence is right."""
+    m = 2  # (with 3 or 4 tokens the activations of fc2 leave no room for the weight ring: launch per linear)
+    lin, ys, x = _chained_opt_layer(capi, m)
+    seq = capi.LinearSequence(lin, m, DEV, mode=capi.SQ_SEQ_ONE_LAUNCH)
+    try:
+        capi.sequence_tune(spin_limit=0)
+        seq.run()
+        torch.cuda.synchronize()
+    finally:
+        capi.sequence_tune()
+    assert seq.error_flag() == 1
+    assert capi.workspace_is_clean(seq.ws)
+    # a split-K decode launch (8 tokens, K = 16384) on the same workspace
+    l5 = lin[5]
+    x8 = (torch.randn((8, 16384), device=DEV) * 0.1).half()
+    y8 = capi.gemm_ws(x8, l5["w"], l5["zs"], 4096, 16384, 128, ws=seq.ws)
+    torch.cuda.synchronize()
+    rows = torch.arange(0, 4096, 67, device=DEV)
+    ref = orc.gemm_ref(x8.cpu().numpy(), orc.dequant_l1(l5["w"][rows].cpu().numpy(), l5["zs"][rows].cpu().numpy(), 128))
+    assert rel_err(y8[:, rows].float().cpu().numpy(), ref.astype(np.float64)) <= 5e-3
+    assert capi.workspace_is_clean(seq.ws)
+    assert seq.error_flag(clear=True) == 1 and seq.error_flag() == 0
+    for y in ys:
+        y.fill_(float("nan"))
+    seq.run()
+    torch.cuda.synchronize()
+    _check_chain_against_oracle(lin, np.random.default_rng(0))
+    assert seq.error_flag() == 0
+
+
 @pytest.mark.parametrize("m", [5, 8, 16, 32])
 def test_grouped_launch_for_decode_batches(capi, m):
     """5..32 tokens: q, k and v (three weights, one input) share one launch of the split-K decode kernel, a
@@ -262,7 +373,8 @@ def test_sequence_rejections(capi):
         d.N, d.K, d.group_size = 64, 128, 64
     ws = ctypes.c_void_p(p)
     call = lambda count, m, layout=1, mode=0: L.sq_w4a16_gemv_sequence(descs, count, m, layout, mode, ws, 256, None)
-    assert L.sq_w4a16_gemv_sequence_workspace_bytes(descs, 2, 1) == 256
+    # 64 KiB for the split-K kernels' counters, then the one-launch kernel's control block (nothing to exchange here)
+    assert L.sq_w4a16_gemv_sequence_workspace_bytes(descs, 2, 1) == 65536 + 256
     assert call(2, 1, mode=5) == capi.SQ_ERR_BAD_ALGO
     assert call(9, 1) == capi.SQ_ERR_BAD_SHAPE
     assert call(0, 1) == capi.SQ_OK
