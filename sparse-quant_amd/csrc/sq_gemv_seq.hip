@@ -98,21 +98,19 @@ struct SeqArgs {
     int zbytes;           // bytes of one zeros/scales slot = 256 nz
     int nz;               // zeros/scales loads per unit = 2048 / group size / 16 (all linears share the group size)
     int lim;              // units a streaming wave keeps in flight (1 or 2; 3 only counts as 2 when it waits)
-#ifdef SQ_SEQ_TRACE
-    unsigned long long* trace;  // 64 stamps of the 100 MHz counter per workgroup
-#endif
 };
 
-#ifdef SQ_SEQ_TRACE
-__device__ __forceinline__ void stamp(const SeqArgs& a, int slot, bool who) {
-    if (a.trace && who) a.trace[(long)blockIdx.x * 64 + slot] = wall_clock64();
-}
-#else
-__device__ __forceinline__ void stamp(const SeqArgs&, int, bool) {}
-#endif
 
 __device__ __forceinline__ void load_to_lds_nt_x4(const void* g, uint32_t lds_byte) {
     asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(g), "{m0}"(lds_byte) : "memory");
+}
+
+// A value read from the argument buffer, pinned in scalar registers: without this the compiler, knowing the buffer
+// never changes, re-reads a field wherever it is used (a scalar load and a wait of a few hundred cycles each time).
+template <typename T>
+__device__ __forceinline__ T pinned(T v) {
+    asm volatile("" : "+s"(v));
+    return v;
 }
 
 __device__ __forceinline__ int lds_counter(const int* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
@@ -123,30 +121,22 @@ __device__ __forceinline__ int lds_counter(const int* p) { return __hip_atomic_l
 struct UnitCursor {
     int l, u, rg, c;
 };
-__device__ __forceinline__ void cursor_place(const SeqArgs& a, UnitCursor& cur, int wave) {
-    while (cur.l < a.count && cur.u >= a.p[cur.l].units) {
+// First linear at or behind cur.l in which this wave has a unit (cur.u = wave on entry to a new linear).
+__device__ __forceinline__ void cursor_place(const SeqArgs& a, int count, UnitCursor& cur, int wave) {
+    while (cur.l < count && cur.u >= pinned(a.p[cur.l].units)) {
         cur.l++;
         cur.u = wave;
     }
-    if (cur.l < a.count) {
-        cur.rg = cur.u / a.p[cur.l].nch;
-        cur.c = cur.u - cur.rg * a.p[cur.l].nch;
-    }
 }
-// One unit on: returns true when the cursor moved to another linear (or past the last).
-__device__ __forceinline__ bool cursor_advance(const SeqArgs& a, UnitCursor& cur, const SeqLinear& L, int wave) {
+// One unit on inside a linear of `units` units and `nch` pieces of K; false when the linear is exhausted.
+__device__ __forceinline__ bool cursor_step(UnitCursor& cur, int units, int nch) {
     cur.u += SEQ_SW;
-    if (cur.u < L.units) {
-        cur.c += SEQ_SW;
-        while (cur.c >= L.nch) {
-            cur.c -= L.nch;
-            cur.rg++;
-        }
-        return false;
+    if (cur.u >= units) return false;
+    cur.c += SEQ_SW;
+    while (cur.c >= nch) {
+        cur.c -= nch;
+        cur.rg++;
     }
-    cur.l++;
-    cur.u = wave;
-    cursor_place(a, cur, wave);
     return true;
 }
 
@@ -172,42 +162,59 @@ __device__ __forceinline__ void streaming_wave(const SeqArgs& a, uint8_t* lds, i
     const int i = lane & 3;
     const int b = lane >> 2;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)lds;
-    const int uslots = a.uslots;
-    const uint32_t wring = a.ring_off + wave * a.ring_stride;  // unit slots of 4 KiB, then their zeros/scales slots
+    const int uslots = pinned(a.uslots);
+    const int zbytes = pinned(a.zbytes);
+    const uint32_t wring = pinned(a.ring_off + wave * a.ring_stride);  // unit slots of 4 KiB, then their zeros/scales slots
     const uint32_t zring = wring + uslots * 4096;
     const uint8_t* xbuf = lds;
     const float* xsum = (const float*)(lds + a.xsum_off);
     int* sync = (int*)(lds + a.sync_off);
-    const int nz = a.nz;
-    const int lim = a.lim;
+    const int nz = pinned(a.nz);
+    const int lim = pinned(a.lim);
+    const int red_base = pinned(a.red_off);
 
     // The counters in LDS start at zero; the one workgroup barrier of the kernel separates that from their first
     // use, and lets the control waves' first activation loads into the memory pipeline ahead of the weights.
     if (wave == 0 && lane < 1 + SEQ_MAX_LINEARS) sync[lane] = 0;
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
+    const int count = pinned(a.count);
     UnitCursor ic = {0, wave, 0, 0}, cc = {0, wave, 0, 0};  // issue side, consume side
-    cursor_place(a, ic, wave);
-    cursor_place(a, cc, wave);
+    cursor_place(a, count, ic, wave);
+    cc = ic;
     // the linears at the two cursors, kept in scalar registers (the argument buffer is read on a change only)
-    SeqLinear Li = a.p[ic.l < a.count ? ic.l : 0], Lc = a.p[cc.l < a.count ? cc.l : 0];
+    struct Pinned {
+        const uint8_t* w;
+        const uint32_t* zs;
+        int N, K, gshift, rows, nch, units, kpad, stage, red_off;
+    };
+    auto fetch = [&a](int l) {
+        const SeqLinear& q = a.p[l];
+        return Pinned{pinned(q.w), pinned((const uint32_t*)q.zs), pinned(q.N), pinned(q.K), pinned(q.gshift), pinned(q.rows),
+                      pinned(q.nch), pinned(q.units), pinned(q.kpad), pinned(q.stage), pinned(q.red_off)};
+    };
+    Pinned Li = fetch(ic.l < count ? ic.l : 0);
+    ic.rg = ic.u / Li.nch;
+    ic.c = ic.u - ic.rg * Li.nch;
+    cc = ic;
+    Pinned Lc = Li;
     int u_issued = 0, u_consumed = 0;  // units requested / multiplied so far
     int u_returned = 0;                // units known to have arrived
     int slot_i = 0, slot_c = 0;        // ring slots at the two cursors
     int staged = 0;                    // last value read of the staging counter
 
-    while (cc.l < a.count) {
+    while (cc.l < count) {
         // ---- request: as long as there is a free slot and the wave is within its in-flight allowance
-        while (ic.l < a.count && u_issued - u_consumed < uslots && u_issued - u_returned < lim) {
-            const SeqLinear& L = Li;
+        while (ic.l < count && u_issued - u_consumed < uslots && u_issued - u_returned < lim) {
+            const Pinned& L = Li;
             const int row0 = wg * L.rows + 4 * ic.rg;
             {
                 // zeros/scales of the unit: lane 16 r + q fetches group q + 16 t of row r
                 const int gpu_ = SEQ_KSUB >> L.gshift;  // groups per unit and row
                 const int groups = L.K >> L.gshift;
                 const int zr = imin(row0 + (lane >> 4), L.N - 1);
-                const uint32_t* zrow = (const uint32_t*)L.zs + (long)zr * groups;
-                const uint32_t zslot = lds0 + zring + slot_i * a.zbytes;
+                const uint32_t* zrow = L.zs + (long)zr * groups;
+                const uint32_t zslot = lds0 + zring + slot_i * zbytes;
                 for (int t = 0; t < nz; t++) {
                     const int gi = ic.c * gpu_ + 16 * t + (lane & 15);
                     load_to_lds_x1(zrow + (gi < groups ? gi : 0), zslot + t * 256);
@@ -224,10 +231,19 @@ __device__ __forceinline__ void streaming_wave(const SeqArgs& a, uint8_t* lds, i
             }
             u_issued++;
             slot_i = slot_i + 1 == uslots ? 0 : slot_i + 1;
-            if (cursor_advance(a, ic, L, wave) && ic.l < a.count) Li = a.p[ic.l];
+            if (!cursor_step(ic, L.units, L.nch)) {
+                ic.l++;
+                ic.u = wave;
+                cursor_place(a, count, ic, wave);
+                if (ic.l < count) {
+                    Li = fetch(ic.l);
+                    ic.rg = ic.u / Li.nch;
+                    ic.c = ic.u - ic.rg * Li.nch;
+                }
+            }
         }
         // ---- are the activations of the linear at the consume cursor in LDS?
-        const SeqLinear& L = Lc;
+        const Pinned& L = Lc;
         if (staged < SEQ_CW * L.stage) staged = __builtin_amdgcn_readfirstlane(lds_counter(&sync[0]));
         if (staged >= SEQ_CW * L.stage) {
             // wait for the unit's loads (zeros/scales first, then the four steps)
@@ -235,10 +251,9 @@ __device__ __forceinline__ void streaming_wave(const SeqArgs& a, uint8_t* lds, i
                 wait_units(u_issued - u_consumed - 1, nz);
                 u_returned = u_consumed + 1;
             }
-            if (cc.u == wave) stamp(a, 4 + 4 * cc.l + 3, threadIdx.x == 0);
             const int pitch = L.kpad * 2 + 16;
             const uint8_t* wslot = lds + wring + slot_c * 4096 + lane * 16;
-            const uint8_t* zslot = lds + zring + slot_c * a.zbytes + 64 * i;
+            const uint8_t* zslot = lds + zring + slot_c * zbytes + 64 * i;
             const int kb0 = cc.c * SEQ_KSUB + 32 * b;
             const uint8_t* xp0 = xbuf + (i & (MROWS - 1)) * pitch + kb0 * 2;
             const float* xs0 = xsum + (kb0 >> 5) * MROWS * 2;
@@ -272,7 +287,7 @@ __device__ __forceinline__ void streaming_wave(const SeqArgs& a, uint8_t* lds, i
                 for (int m = 0; m < MROWS; m++) acc[m] += sf * ((tmp[m] - xs[2 * m + 1]) - zf * xs[2 * m]);
             }
             // fold the 16 blocks of the wave; lanes 0..3 hold rows 4*rg + 0..3
-            float* red = (float*)(lds + a.red_off) + L.red_off;
+            float* red = (float*)(lds + red_base) + L.red_off;
 #pragma unroll
             for (int m = 0; m < MROWS; m++) {
                 float v = row_sum_stride4(acc[m]);
@@ -282,14 +297,20 @@ __device__ __forceinline__ void streaming_wave(const SeqArgs& a, uint8_t* lds, i
             }
             u_consumed++;
             slot_c = slot_c + 1 == uslots ? 0 : slot_c + 1;
-            const int l_done = cc.l;
-            if (cursor_advance(a, cc, L, wave)) {
+            if (!cursor_step(cc, L.units, L.nch)) {
                 // this wave's last unit of the linear: its partial sums are in LDS before the count moves
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                if (lane == 0) __hip_atomic_fetch_add(&sync[1 + l_done], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-                if (cc.l < a.count) Lc = a.p[cc.l];
+                if (lane == 0) __hip_atomic_fetch_add(&sync[1 + cc.l], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                cc.l++;
+                cc.u = wave;
+                cursor_place(a, count, cc, wave);
+                if (cc.l < count) {
+                    Lc = fetch(cc.l);
+                    cc.rg = cc.u / Lc.nch;
+                    cc.c = cc.u - cc.rg * Lc.nch;
+                }
             }
-        } else if (u_issued > u_returned && ic.l < a.count && u_issued - u_consumed < uslots) {
+        } else if (u_issued > u_returned && ic.l < count && u_issued - u_consumed < uslots) {
             // not yet: make room in the in-flight allowance by waiting for the oldest outstanding unit
             wait_units(u_issued - u_returned - 1, nz);
             u_returned++;
@@ -446,10 +467,7 @@ __device__ __forceinline__ void control_wave(const SeqArgs& a, uint8_t* lds, int
     // the launch's tag: one more than the number the previous launch on this workspace left behind
     const unsigned tag = __hip_atomic_load(&a.ctrl[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
     bool failed = false;
-
-    stamp(a, 0, ct == 0);
     stage_plain<MROWS>(a.p[0], M, xbuf, xsum, ct, true);  // contains the workgroup barrier of the kernel's start
-    stamp(a, 1, ct == 0);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     if ((ct & 63) == 0) __hip_atomic_fetch_add(&sync[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 
@@ -471,7 +489,6 @@ __device__ __forceinline__ void control_wave(const SeqArgs& a, uint8_t* lds, int
                           : (u64) * (const uint32_t*)(L.residual + (long)m0 * L.N + n00) | ((u64)tag << 32);
         // every streaming wave with units of this linear has left its partial sums
         while (lds_counter(&sync[1 + cl]) < L.need) __builtin_amdgcn_s_sleep(1);
-        stamp(a, 4 + 4 * cl, ct == 0);
         const float* red = (const float*)(lds + a.red_off) + L.red_off;
         for (int t = ct; t < items; t += SEQ_CT) {
             const int m = t / half_rows;
@@ -523,7 +540,6 @@ __device__ __forceinline__ void control_wave(const SeqArgs& a, uint8_t* lds, int
                 *(uint32_t*)(L.y + (long)m * L.N + n0) = bits;
             }
         }
-        stamp(a, 4 + 4 * cl + 1, ct == 0);
         if (cl + 1 < count && a.p[cl + 1].restage) {
             const SeqLinear& Ln = a.p[cl + 1];
             if (Ln.xsrc) {
@@ -533,10 +549,8 @@ __device__ __forceinline__ void control_wave(const SeqArgs& a, uint8_t* lds, int
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             if ((ct & 63) == 0) __hip_atomic_fetch_add(&sync[0], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            stamp(a, 4 + 4 * cl + 2, ct == 0);
         }
     }
-    stamp(a, 62, ct == 0);
     if (__builtin_amdgcn_ballot_w64(failed) != 0 && (ct & 63) == 0)
         __hip_atomic_store(&a.ctrl[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // Exit: the last control wave of the launch to get here advances the launch number (every poll of this
@@ -635,15 +649,9 @@ bool plan_flow(const SeqProblem* probs, int count, int M, int* src_x, int* src_r
     return true;
 }
 
-#ifdef SQ_SEQ_TRACE
-unsigned long long* g_seq_trace = nullptr;
-#endif
 
 }  // namespace
 
-#ifdef SQ_SEQ_TRACE
-extern "C" void sq_seq_set_trace(void* p) { g_seq_trace = (unsigned long long*)p; }
-#endif
 
 size_t gemv_seq_workspace_bytes(const SeqProblem* probs, int count, int M) {
     size_t need = SEQ_XCHG_OFF;
@@ -674,9 +682,6 @@ int launch_gemv_seq(const SeqProblem* probs, int count, int M, void* workspace, 
     a.M = M;
     a.ctrl = (unsigned*)workspace;
     a.spin_limit = spin_limit;
-#ifdef SQ_SEQ_TRACE
-    a.trace = g_seq_trace;
-#endif
     int kpad_max = 0, red_floats = 0, stage = 0;
     size_t xchg = SEQ_XCHG_OFF;
     u64* dst[SEQ_MAX_LINEARS] = {};
