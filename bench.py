@@ -4,10 +4,12 @@
 Workload (the headline decode configuration): the six W4A16 linears of one
 OPT-6.7B decoder layer -- q/k/v/out 4096x4096, fc1 4096->16384, fc2 16384->4096 --
 int4 weights in layout L1, group size 128, fp16 activations, M = 1 token.  One
-"step" is one pass over the six linears of one layer, launched back to back on one
-HIP stream through the C ABI (sq_w4a16_gemm).  Successive steps walk a pool of
-distinct layers (> 256 MB in total), so every launch streams its weights from HBM
-rather than from the Infinity Cache.
+"step" is one pass over the six linears of one layer on one HIP stream through the
+C ABI: sq_w4a16_gemv_sequence with the layer's data flow (q, k and v share a launch;
+out_proj, fc1 and fc2 get one each: four launches), or with --per-linear one
+sq_w4a16_gemm per linear (six launches).  Successive steps walk a pool of distinct
+layers (> 256 MB in total), so every launch streams its weights from HBM rather than
+from the Infinity Cache.
 
 The metric is achieved GB/s: algorithmic bytes of a step
     sum over linears of  N*K/2 + (K/g)*N*4 + M*K*2 + M*N*2   (= 107 102 208 B at M = 1)
