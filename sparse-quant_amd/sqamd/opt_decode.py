@@ -6,10 +6,13 @@ vocab 50272, learned positions with OPT's +2 offset, fp16 lm_head; q/k/v/out/fc1
 are `WALinear` modules (layout L1, group 128) with random packed weights -- the same
 six linears per layer, in the same order and with the same [1, tokens, K] call shape
 the reference feeds to gemm_awq_ut (test/nvidia/module/opt/modeling_opt_ours.py:
-158-164, 505-506, 598-611).  Attention is dense (the reference's decode path is dense
+158-164, 505-506, 598-611).  Decode attention is dense (the reference's decode path is dense
 too): the decode step appends to the preallocated fp16 KV cache and attends in one kernel
 (sq_decode_attention) that reads the position from the device, so the step is a fixed
-kernel sequence that can be captured in a HIP graph.
+kernel sequence that can be captured in a HIP graph.  Prefill attention is dense causal by
+default; a layer that has been given a look-up table (`DecoderLayer.lut`, per head) runs its
+prefill through sparse_attention(q, k, v, scaling, lut, LT=True) as the reference's OPT
+attention does (test/nvidia/module/opt/modeling_opt_ours.py:435-438).
 """
 import math
 import time
@@ -17,7 +20,8 @@ import time
 import torch
 from torch import nn
 
-from . import capi
+from . import capi, lut_layout
+from .block_sparse_attention_lut import sparse_attention
 from .qlinear import WALinear
 
 
@@ -57,6 +61,8 @@ class DecoderLayer(nn.Module):
         self.fc2 = _random_walinear(ffn, hidden, g, dev, gen, scale_std, scale_min)
         self.qkv_proj = None
         self.fuse_ln = True  # LayerNorm inside the q/k/v and fc1 launches
+        self.lut = None      # int [heads, ceil(T / 64), nnz]: prefill attention through the LUT kernel
+        self.capture = None  # a dict: the prefill's q, k, v and attention output are left in it (tests)
 
     def forward(self, x, kc, vc, pos0):
         """x [B, T, H]; kc, vc [B, heads, Lmax, hd]; writes cache rows pos0 .. pos0+T-1."""
@@ -78,8 +84,13 @@ class DecoderLayer(nn.Module):
         if isinstance(pos0, int):
             kc[:, :, pos0:pos0 + t] = k
             vc[:, :, pos0:pos0 + t] = v
-            a = nn.functional.scaled_dot_product_attention(q, kc[:, :, :pos0 + t], vc[:, :, :pos0 + t],
-                                                           is_causal=(t > 1))
+            if self.lut is not None and pos0 == 0 and t > 1:
+                a = sparse_attention(q, k, v, 1.0 / math.sqrt(self.hd), self.lut, LT=True)
+            else:
+                a = nn.functional.scaled_dot_product_attention(q, kc[:, :, :pos0 + t], vc[:, :, :pos0 + t],
+                                                               is_causal=(t > 1))
+            if self.capture is not None:
+                self.capture.update(q=q.detach().clone(), k=k.detach().clone(), v=v.detach().clone(), a=a.detach().clone())
             a = a.transpose(1, 2).reshape(1, b * t, hdim)
         else:
             # graph-captured decode step: the position lives in a device tensor; one kernel appends the
@@ -108,16 +119,30 @@ class DecoderLayer(nn.Module):
 
 class OPTDecoder(nn.Module):
     def __init__(self, layers=32, hidden=4096, heads=32, ffn=16384, vocab=50272, max_pos=2048, group=128,
-                 dev="cuda", seed=0):
+                 dev="cuda", seed=0, scale_std=E2E_SCALE_STD, scale_min=E2E_SCALE_MIN):
         super().__init__()
         gen = torch.Generator(device=dev)
         gen.manual_seed(seed)
         self.hidden, self.heads = hidden, heads
         self.embed = (torch.randn((vocab, hidden), device=dev, generator=gen) * 0.02).half()
         self.pos = (torch.randn((max_pos + 2, hidden), device=dev, generator=gen) * 0.02).half()
-        self.layers = nn.ModuleList([DecoderLayer(hidden, heads, ffn, group, dev, gen) for _ in range(layers)])
+        self.layers = nn.ModuleList([DecoderLayer(hidden, heads, ffn, group, dev, gen, scale_std, scale_min)
+                                     for _ in range(layers)])
         self.final_ln = nn.LayerNorm(hidden, device=dev, dtype=torch.float16)
         self.lm_head = (torch.randn((vocab, hidden), device=dev, generator=gen) * 0.02).half()
+
+    def set_prefill_lut(self, tokens, density, seed=0):
+        """Give every layer a causal look-up table of the given block density for prompts of `tokens` tokens
+        (diagonal block always kept, the others drawn from a seed, a table per layer and head), or none
+        (density None): the reference loads such tables from a file (`--lut_path`,
+        test/eval_compress_opt_support_3090.sh:35: density 26 %)."""
+        nb = (tokens + 63) // 64
+        for idx, layer in enumerate(self.layers):
+            if density is None:
+                layer.lut = None
+                continue
+            layout = lut_layout.synth_layout(self.heads, nb, density, causal=True, seed=seed + idx)
+            layer.lut = lut_layout.layout2lut_single_density(layout[None])[0].to(self.embed.device)
 
     def new_cache(self, batch, max_len):
         hd = self.hidden // self.heads
@@ -140,10 +165,10 @@ class OPTDecoder(nn.Module):
 
 @torch.no_grad()
 def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed=0, fuse_qkv=True,
-            return_tokens=False):
+            return_tokens=False, lut_density=0.26, scale_std=E2E_SCALE_STD, scale_min=E2E_SCALE_MIN):
     """Greedy generation on random token ids; returns timing and throughput figures."""
     dev = "cuda"
-    model = OPTDecoder(layers=layers, dev=dev, seed=seed)
+    model = OPTDecoder(layers=layers, dev=dev, seed=seed, scale_std=scale_std, scale_min=scale_min)
     if fuse_qkv:
         for layer in model.layers:
             layer.fuse_qkv()
@@ -155,6 +180,18 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
 
     model(ids, cache, 0)  # untimed first pass: code objects, library handles and workspaces come into being here
     torch.cuda.synchronize()
+    # The same prefill with the attention of every layer through the LUT kernel (causal tables of the
+    # reference's OPT density); the dense pass that follows rewrites the cache, decode starts from that one.
+    prefill_lut_s = None
+    if lut_density is not None and prompt >= 128:
+        model.set_prefill_lut(prompt, lut_density, seed=seed)
+        model(ids, cache, 0)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        model(ids, cache, 0)
+        torch.cuda.synchronize()
+        prefill_lut_s = time.perf_counter() - t0
+        model.set_prefill_lut(prompt, None)
     t0 = time.perf_counter()
     logits = model(ids, cache, 0)
     nxt = logits.argmax(-1)
@@ -210,13 +247,18 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
         **extra,
         "weights": "random packed int4, zeros U{0..15}, scales |N(0,%g)|+%g (smaller than the single-linear "
                    "benchmark's |N(0,0.02)|+1e-3 so that 32 random layers stay finite in fp16)"
-                   % (E2E_SCALE_STD, E2E_SCALE_MIN),
+                   % (scale_std, scale_min),
         "batch": batch, "prompt": prompt, "new_tokens": new_tokens, "layers": layers,
         "launch": "hip-graph replay" if graph is not None else "eager",
         "fused": "bias+relu+residual in the GEMM store" + ("; q/k/v one launch" if fuse_qkv else "") +
                  "; both LayerNorms inside the q/k/v and fc1 kernels at decode; decode attention appends K/V in the same "
                  "launch",
         "prefill_ms": round(prefill_s * 1e3, 2),
+        "prefill_attention": "dense causal (torch SDPA)",
+        "prefill_lut_ms": None if prefill_lut_s is None else round(prefill_lut_s * 1e3, 2),
+        "prefill_lut_attention": None if prefill_lut_s is None else
+        "sparse_attention(q, k, v, scaling, lut, LT=True) in every layer: causal per-head tables, block density %.2f, "
+        "D = 128 (sq_lut_attention_fwd)" % lut_density,
         "prefill_tok_per_s": round(batch * prompt / prefill_s, 1),
         "decode_ms_per_step": round(decode_s * 1e3 / steps, 4),
         "decode_tok_per_s": round(batch * steps / decode_s, 1),
@@ -227,6 +269,7 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
         "parity": "covered by tests/test_gpu_full_size.py: one full-width decoder layer against the oracle composition, "
                   "eager and HIP-graph decode steps generate identical tokens",
         "tokens_checksum": int(torch.stack(generated).sum().item()),
+        "logits_finite": bool(torch.isfinite(logits).all().item()),
     }
 
 
