@@ -102,11 +102,13 @@ int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y,
  * results; the workspace is a buffer of SQ_STATIC_WS_BYTES (16 MiB + 64 KiB) that lives inside
  * the library's device code, one copy per GPU for the life of the process, so the call
  * allocates and frees nothing.  The caller still passes inputs and the output.
- * Limit: shapes with sq_w4a16_workspace_bytes(M, N, K) > SQ_STATIC_WS_BYTES are rejected with
- * SQ_ERR_STATIC_WS and nothing is launched (every decode batch of up to 32 tokens with
- * N <= 16384 fits; so do the K splits of the tiled GEMM up to that size).
- * The first call on a device looks the buffer's address up and enqueues a small kernel on
- * `stream` that clears its counter region; make that first call outside graph capture.
+ * Limit: a call whose kernels would take more than SQ_STATIC_WS_BYTES from a workspace is rejected
+ * with SQ_ERR_STATIC_WS and nothing is launched: the split-K decode kernels at 3..32 tokens (every
+ * such batch with N <= 16384 fits) and the K splits of the tiled GEMM beyond 32 tokens.  One or two
+ * tokens, and a GEMM whose grid fills the chip without a K split, use no workspace and are never
+ * rejected, whatever N is.
+ * The first call on a device looks the buffer's address up (hipGetSymbolAddress); nothing is
+ * cleared, the array is zero when the library is loaded and every kernel leaves its counters zero.
  * Every call on a GPU shares that GPU's buffer: calls that overlap in time on one GPU (two
  * streams, two threads) race; calls on one stream are ordered and safe.  The buffer keeps the
  * last call's partial sums; the kernels overwrite what they read and leave the counters zero. */

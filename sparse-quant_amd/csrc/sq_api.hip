@@ -20,33 +20,22 @@ __global__ void zero_words_kernel(unsigned* p, int n) {
 }
 
 constexpr int MAX_DEVICES = 64;
-struct ScratchState {
-    void* ptr = nullptr;
-    bool cleared = false;
-};
-ScratchState g_scratch[MAX_DEVICES];
+void* g_scratch[MAX_DEVICES];
 std::mutex g_scratch_mutex;
 
-// Device address of `scratch` on the current device; on the first call per device the counter
-// region (the part every kernel expects to find zero and leaves zero) is cleared by a small fill
-// kernel on `st`, ahead of the first use.  Returns null on failure.
-void* static_workspace(hipStream_t st) {
+// Device address of `scratch` on the current device (null on failure).  The array needs no clearing: a
+// file-scope __device__ array without an initialiser is zero when its code object is loaded, and every kernel
+// leaves the counters at its start zero.
+void* static_workspace() {
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
-    ScratchState& s = g_scratch[dev];
-    if (!s.ptr) {
+    if (!g_scratch[dev]) {
         void* p = nullptr;
         if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
-        s.ptr = p;
+        g_scratch[dev] = p;
     }
-    if (!s.cleared) {
-        constexpr int words = 64 * 1024 / 4;
-        hipLaunchKernelGGL(zero_words_kernel, dim3(words / 256), dim3(256), 0, st, static_cast<unsigned*>(s.ptr), words);
-        if (hipGetLastError() != hipSuccess) return nullptr;
-        s.cleared = true;
-    }
-    return s.ptr;
+    return g_scratch[dev];
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -228,17 +217,21 @@ int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y, int 
 
 int sq_w4a16_gemm_static_ws(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
                             int layout, int algo, void* stream) {
-    if (M > 0 && N > 0 && K > 0 && sq_w4a16_workspace_bytes(M, N, K) > (size_t)SQ_STATIC_WS_BYTES) return SQ_ERR_STATIC_WS;
-    // Validate before touching the device, so that argument errors launch nothing (not even the
-    // one-time clearing of the counters).
+    // Validate before touching the device, so that argument errors launch nothing.
     if (M < 0) return SQ_ERR_BAD_SHAPE;
     const int rc = check_weight(N, K, group_size, layout);
     if (rc != SQ_OK) return rc;
     if (layout != SQ_LAYOUT_L1) return SQ_ERR_BAD_LAYOUT;
+    // What the kernels of this token count would take from a workspace: nothing up to 2 tokens (the GEMV has
+    // no workspace form), the split-K decode kernels' counters and partial tiles up to 32, the tiled GEMM's K
+    // split beyond.  A shape that wants more than the static buffer is refused rather than served by a slower
+    // workspace-free kernel behind the caller's back.
+    const size_t need = M <= 2 ? 0 : (M <= 32 ? sq::skinny2_workspace_bytes(M, N, K) : sq::gemm_workspace_bytes(M, N, K));
+    if (need > (size_t)SQ_STATIC_WS_BYTES) return SQ_ERR_STATIC_WS;
     if (M == 0) return SQ_OK;
     if (!x || !w || !zs || !y) return SQ_ERR_NULL_POINTER;
     if (!aligned16(x) || !aligned16(w) || !aligned16(zs) || !aligned16(y)) return SQ_ERR_MISALIGNED;
-    void* ws = static_workspace(static_cast<hipStream_t>(stream));
+    void* ws = static_workspace();
     if (!ws) return SQ_ERR_LAUNCH;
     return gemm_dispatch(x, w, zs, y, M, N, K, group_size, layout, algo, sq::Epilogue{nullptr, nullptr, 0}, ws,
                          (size_t)SQ_STATIC_WS_BYTES, stream);

@@ -30,7 +30,10 @@ def test_static_workspace_entry_point_matches_the_caller_workspace_one(capi):
     before = torch.cuda.memory_allocated()
     # (M, N, K): split-K decode kernel on a large weight, then a smaller problem on a small weight, then a
     # K-split tiled GEMM and a shape that needs no workspace at all
-    cases = [(16, 8192, 4096), (20, 1024, 2048), (8, 8192, 4096), (96, 1024, 4096), (3, 512, 1024)]
+    # (the last two: a single token and 2048 tokens on an lm_head-sized weight, N = 50272, which need no workspace
+    # although the query for decode batches on that weight exceeds the static buffer)
+    cases = [(16, 8192, 4096), (20, 1024, 2048), (8, 8192, 4096), (96, 1024, 4096), (3, 512, 1024), (1, 50272, 1024),
+             (2048, 50272, 1024)]
     data = {}
     for m, n, k in cases:
         if (n, k) not in data:
@@ -62,6 +65,7 @@ def test_static_workspace_entry_point_rejects_what_does_not_fit(capi):
     # 32 tokens on N = 32768 need 32 MiB of partial sums: beyond the static buffer
     assert L.sq_w4a16_workspace_bytes(32, 32768, 4096) > capi.SQ_STATIC_WS_BYTES
     assert L.sq_w4a16_gemm_static_ws(p, p, p, p, 32, 32768, 4096, 128, 1, 0, None) == capi.SQ_ERR_STATIC_WS
+    assert L.sq_w4a16_workspace_bytes(32, 50272, 1024) > capi.SQ_STATIC_WS_BYTES  # yet one token on it is served (above)
     assert "static" in capi.strerror(capi.SQ_ERR_STATIC_WS)
     assert L.sq_w4a16_gemm_static_ws(None, p, p, p, 8, 4096, 4096, 128, 1, 0, None) == capi.SQ_ERR_NULL_POINTER
     assert L.sq_w4a16_gemm_static_ws(p, p, p, p, 8, 4096, 4096, 100, 1, 0, None) == capi.SQ_ERR_BAD_GROUP
