@@ -51,6 +51,16 @@ OPT67_LAYER = [("q_proj", 4096, 4096), ("k_proj", 4096, 4096), ("v_proj", 4096, 
                ("fc1", 16384, 4096), ("fc2", 4096, 16384)]  # (name, N, K)
 
 
+def decode_kernel_source_sha16():
+    """First 16 hex digits of the SHA-256 over the sources of the single-token decode kernel."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in ("sq_gemv2.hip", "sq_common.h"):
+        with open(os.path.join(REPO, "sparse-quant_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def algorithmic_bytes(m, n, k, g):
     return n * k // 2 + (k // g) * n * 4 + m * k * 2 + m * n * 2
 
@@ -439,11 +449,21 @@ def main():
     launch_us = gpu_ms * 1e3 / (steps * launches_per_step)
     achieved = (bytes_per_step / launches_per_step) / (launch_us * 1e-6) / 1e9
 
-    traffic = None
+    # HBM traffic per launch comes from a counter run of this command (rocprofv3 --pmc cannot run inside the timed
+    # process); the stored figure is used only while the decode kernel's source is the one it was measured on.
+    traffic, traffic_note = None, "no stored counter run"
     tfile = os.path.join(REPO, "profiles", "gemv_decode_traffic.json")
-    if os.path.exists(tfile) and m == 1 and g == 128:
+    if os.path.exists(tfile) and m == 1 and g == 128 and use_sequence:
         try:
-            traffic = json.load(open(tfile)).get("hbm_bytes_per_launch")
+            stored = json.load(open(tfile))
+            if stored.get("decode_kernel_source_sha16") == decode_kernel_source_sha16():
+                traffic = stored.get("hbm_bytes_per_launch")
+                traffic_note = ("stored from profiles/gemv_decode_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                                "of this command, scaled by a 256 MiB copy; same decode kernel source), not measured in "
+                                "this run")
+            else:
+                traffic_note = ("profiles/gemv_decode_traffic.json was measured on another version of the decode "
+                                "kernel's source: not reported")
         except Exception:
             traffic = None
 
@@ -467,9 +487,7 @@ def main():
                               "weights; every other leg below carries its own parity_max_rel_err, checked the same way "
                               "before it is timed"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "traffic_source": "stored from profiles/gemv_decode_traffic.json (rocprofv3 --pmc FETCH_SIZE / "
-                                       "WRITE_SIZE of this command, scaled by a 256 MiB copy), not measured in this run",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_note,
                      "kernel": "sq::gemv2_kernel / sq::gemv2_group_kernel (decode GEMV)",
                      "launches_per_step": launches_per_step, "avg_launch_us": round(launch_us, 3),
                      "bytes_per_launch": bytes_per_step // launches_per_step},
@@ -523,6 +541,7 @@ def main():
             pair["decode_ratio"] = round(pair["baseline_scales"]["decode_ms_per_step"] /
                                          pair["harness_scales"]["decode_ms_per_step"], 4)
             out["e2e_opt67"]["two_layers_either_scale_distribution"] = pair
+            out["kernel_picker"] = picker_leg(torch, capi, g, dev, gen, stream)  # last: it records choices
         except ParityError:
             raise
         except Exception as exc:  # an extra leg must never hide the headline line
@@ -962,6 +981,43 @@ def sequence_leg(torch, capi, pool, shapes, m, g, dev, gen, stream, bytes_per_st
         res[label] = {"depends": dep, "us_per_step": round(us, 2), "gbs": round(bytes_per_step / us / 1e3, 1),
                       "frac_of_hbm_peak": round(bytes_per_step / us / 1e3 / HBM_PEAK_GBS, 4),
                       "parity_max_rel_err": round(worst, 6), "wait_timeouts": sum(sq.error_flag() for sq in seqs)}
+    return res
+
+
+def picker_leg(torch, capi, g, dev, gen, stream):
+    """The measured kernel picker (sq_w4a16_autotune) on shapes the built-in rules were swept on and on shapes they
+    were not: per shape and token count the launch time of the built-in choice, of the fastest candidate, and that
+    candidate's kernel word (0 = the built-in choice stands).  Weights rotate through a pool beyond the last-level
+    cache.  The recorded choices are dropped again at the end."""
+    res = {}
+    shapes = (("opt_fc1", 16384, 4096), ("opt_fc2", 4096, 16384), ("llama13b_up", 13824, 5120),
+              ("llama13b_down", 5120, 13824), ("n1024_k8192", 1024, 8192))
+    try:
+        for name, n, k in shapes:
+            copies = max(2, int(600e6 / (n * k / 2)))
+            w = torch.randint(0, 256, (copies, n, k // 2), dtype=torch.uint8, device=dev, generator=gen)
+            z = torch.randint(0, 16, (copies, n, k // g), device=dev, generator=gen).half() + 64
+            sc = (torch.randn((copies, n, k // g), device=dev, generator=gen).abs() * 0.02 + 1e-3).half()
+            zs = torch.stack([z, sc], dim=-1).reshape(copies, n, 2 * (k // g)).contiguous()
+            per = {}
+            for m in (1, 8, 32, 128, 1024):
+                x = torch.randn((m, k), device=dev, generator=gen).half()
+                y = torch.empty((m, n), dtype=torch.float16, device=dev)
+                ws = capi.workspace(m, n, k, dev, stream)
+                torch.cuda.synchronize()
+                with torch.cuda.stream(stream):
+                    word, t_best, t_auto = capi.autotune(x, w, zs, n, k, g, ws=ws, reps=max(copies, 20), out=y, stream=stream)
+                    # the product path now takes the recorded choice: check it like every other leg
+                    capi.gemm_ws(x, w[0], zs[0], n, k, g, out=y, stream=stream, ws=ws)
+                    stream.synchronize()
+                    err = gate(parity_linear(torch, w[0], zs[0], n, k, g, x, y, seed=m), "picker %s at M=%d" % (name, m))
+                per["m%d" % m] = {"builtin_us": round(t_auto, 2), "best_us": round(t_best, 2),
+                                  "best_kernel_word": "0x%x" % word, "gain": round(t_auto / t_best, 3),
+                                  "parity_max_rel_err": round(err, 6)}
+            res[name] = per
+            del w, z, sc, zs
+    finally:
+        res["choices_recorded"] = capi.autotune_clear()
     return res
 
 

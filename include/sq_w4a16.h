@@ -96,6 +96,35 @@ int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y,
                      int M, int N, int K, int group_size, int layout, int algo,
                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* Measured kernel choice.  In the role of TurboMind's measuring mode, which times its 17 tile
+ * configurations on the shape at hand and keeps the fastest (reference:
+ * quantization/nvidia/kernel/gemm_s4_f16/gemm_s4_f16.cu:92-197, gemm_s4_f16_kernel.h:83-134);
+ * SQ_ALGO_AUTO's built-in rules are constants from sweeps of the OPT-6.7B / Llama-2-7B shapes.
+ * sq_w4a16_autotune runs the product x * W_hat^T with every kernel family and tuning that can
+ * serve (M, N, K, group_size) -- the decode GEMV's workgroup shapes, the streaming kernel's row
+ * blocks and K splits, the split-K kernel's splits, the tiled GEMM's tile heights, K splits and
+ * staging variants -- `reps` launches each between two HIP events on `stream`, and records the
+ * fastest in a process-wide table that SQ_ALGO_AUTO consults first from then on, for exactly
+ * this (M, N, K, group_size) and workspace situation (a workspace of at least
+ * sq_w4a16_workspace_bytes(M, N, K) bytes present or not).  This is the one GEMM entry point
+ * that SYNCHRONISES (once per candidate) and creates host-side event objects; it allocates no
+ * device memory.  y is written by every candidate and holds the chosen kernel's result at the end.
+ *   copies, w_stride, zs_stride  copies > 1: candidate launch i reads the weight at
+ *             w + (i % copies) * w_stride and its zeros/scales at zs + (i % copies) * zs_stride
+ *             (bytes, multiples of 16), so that a pool larger than the 256 MB last-level cache is
+ *             timed from HBM, as a decode step meets its weights; copies = 1 times one weight,
+ *             which stays in that cache when it is smaller.
+ *   best_algo  (may be NULL) the chosen kernel word for sq_w4a16_gemm_ex / _ws, 0 when the built-in
+ *             choice was not beaten (then nothing is recorded); best_us, auto_us (may be NULL) the
+ *             average launch time of the chosen and of the built-in choice.
+ * sq_w4a16_autotune_clear forgets every recorded choice and returns how many there were.  The table
+ * is append-only (1024 recordings per process; later ones are measured but not kept). */
+int sq_w4a16_autotune(const void* x, const void* w, const void* zs, void* y, int M, int N, int K,
+                      int group_size, int layout, void* workspace, size_t workspace_bytes, int copies,
+                      size_t w_stride, size_t zs_stride, int reps, void* stream, int* best_algo,
+                      float* best_us, float* auto_us);
+int sq_w4a16_autotune_clear(void);
+
 /* sq_w4a16_gemm_ws for callers that cannot allocate device memory: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the
  * reference.  Same product, same kernels and the same automatic kernel choice, bit-identical

@@ -2,6 +2,7 @@
 // and the contract of every entry point are in include/sq_w4a16.h.
 #include "../../include/sq_w4a16.h"
 
+#include <atomic>
 #include <mutex>
 
 #include "sq_kernels.h"
@@ -59,6 +60,31 @@ int check_weight(int N, int K, int g, int layout) {
 
 // One dispatcher behind every GEMM entry point.  `workspace` may be null: then the kernels
 // that need one are not considered (and an explicit SQ_ALGO_SKINNY_WS is an error).
+// Measured kernel choices (sq_w4a16_autotune): shape -> kernel word, consulted before the built-in rules.
+// Entries are only ever appended (under the mutex); readers scan without it up to the published count.
+struct TunedEntry {
+    int M, N, K, g, has_ws, algo;
+    float us;
+};
+constexpr int TUNED_MAX = 1024;
+TunedEntry g_tuned[TUNED_MAX];
+std::atomic<int> g_tuned_count{0};
+std::mutex g_tuned_mutex;
+
+inline bool full_workspace(const void* workspace, size_t workspace_bytes, int M, int N, int K) {
+    return workspace && (reinterpret_cast<uintptr_t>(workspace) & 15u) == 0 &&
+           workspace_bytes >= sq_w4a16_workspace_bytes(M, N, K);
+}
+
+int tuned_lookup(int M, int N, int K, int g, bool has_ws) {
+    const int n = g_tuned_count.load(std::memory_order_acquire);
+    for (int i = n - 1; i >= 0; i--) {  // the latest measurement of a shape wins
+        const TunedEntry& e = g_tuned[i];
+        if (e.M == M && e.N == N && e.K == K && e.g == g && e.has_ws == (int)has_ws) return e.algo;
+    }
+    return 0;
+}
+
 int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
                   int layout, int algo, sq::Epilogue epi, void* workspace, size_t workspace_bytes, void* stream) {
     if (M < 0) return SQ_ERR_BAD_SHAPE;
@@ -74,7 +100,14 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
     hipStream_t st = static_cast<hipStream_t>(stream);
 
     int kernel = algo & 0xFF;
-    const int tune = (algo >> 8) & 0xFFFF;
+    int tune = (algo >> 8) & 0xFFFF;
+    if (kernel == SQ_ALGO_AUTO && g_tuned_count.load(std::memory_order_relaxed) > 0) {
+        const int word = tuned_lookup(M, N, K, group_size, full_workspace(workspace, workspace_bytes, M, N, K));
+        if (word != 0) {
+            kernel = word & 0xFF;
+            tune = (word >> 8) & 0xFFFF;
+        }
+    }
     if (kernel == SQ_ALGO_AUTO) {
         // Measured on OPT-6.7B shapes.  With a workspace the split-K kernel wins for 5..32
         // tokens once the weight is large enough (fc1/fc2 class) or K is long, and for 17..32
@@ -213,6 +246,152 @@ int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y, int 
                      int layout, int algo, void* workspace, size_t workspace_bytes, void* stream) {
     return gemm_dispatch(x, w, zs, y, M, N, K, group_size, layout, algo, sq::Epilogue{nullptr, nullptr, 0}, workspace,
                          workspace_bytes, stream);
+}
+
+// Kernel words worth timing for a shape: every family that can run it, with the tunings its launcher accepts.
+// A word the launcher refuses (a K split that does not divide, a missing workspace) is skipped by the caller.
+static int autotune_candidates(int M, int K, int g, bool has_ws, int* out, int cap) {
+    int n = 0;
+    auto add = [&](int kernel, int tune) {
+        if (n < cap) out[n++] = kernel | (tune << 8);
+    };
+    if (M <= 8)
+        for (int ks = 1; ks <= 4; ks *= 2)
+            for (int nr = 2; nr <= 8; nr *= 2)
+                if (nr * ks <= 16) add(SQ_ALGO_GEMV_FIXUP, nr | (ks << 4));
+    if (M <= 16 && (g == 128 || g == 64) && K % 128 == 0) {
+        const int rows[3] = {1, 3, 4};
+        for (int r = 0; r < 3; r++)
+            for (int ks = 1; ks <= 8; ks *= 2)
+                if (ks == 1 ? K <= 4096 : (has_ws && K / ks >= 1024 && K / ks <= 4096)) add(SQ_ALGO_STREAM, rows[r] | (ks << 4));
+    }
+    if (M > 16 && M <= 32 && g == 128) add(SQ_ALGO_STREAM, 0);
+    if (M > 2 && M <= 32 && has_ws)
+        for (int ks = 1; ks <= 8; ks *= 2) add(SQ_ALGO_SKINNY_WS, ks);
+    if (M > 2 && M <= 64) add(SQ_ALGO_SKINNY, 0);
+    if (M > 16) {
+        for (int lds = 0; lds <= (K % 256 == 0 ? 1 : 0); lds++)
+            for (int mi = 1; mi <= 4; mi *= 2) {
+                if (M <= 64 && mi == 4) continue;
+                for (int ks = 1; ks <= (has_ws ? 8 : 1); ks *= 2) add(SQ_ALGO_GEMM, mi | (lds ? 0x80 : 0) | (ks << 8));
+            }
+        if (M > 64)
+            for (int v = 8; v <= 10; v++) add(SQ_ALGO_GEMM, v);
+    }
+    return n;
+}
+
+int sq_w4a16_autotune(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
+                      int layout, void* workspace, size_t workspace_bytes, int copies, size_t w_stride, size_t zs_stride,
+                      int reps, void* stream, int* best_algo, float* best_us, float* auto_us) {
+    if (M <= 0) return SQ_ERR_BAD_SHAPE;
+    if (copies < 1 || copies > 4096 || reps < 1 || reps > 100000) return SQ_ERR_BAD_SHAPE;
+    if (copies > 1 && (w_stride % 16 != 0 || zs_stride % 16 != 0 || w_stride < (size_t)N * K / 2)) return SQ_ERR_MISALIGNED;
+    const sq::Epilogue none{nullptr, nullptr, 0};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool has_ws = full_workspace(workspace, workspace_bytes, M, N, K);
+    if (!has_ws) {
+        workspace = nullptr;
+        workspace_bytes = 0;
+    }
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
+        if (e0) (void)hipEventDestroy(e0);
+        return SQ_ERR_LAUNCH;
+    }
+    // One candidate: a launch that has to succeed, a short warm-up, then `reps` launches between two events,
+    // walking through the `copies` weights so that a pool larger than the last-level cache is read from HBM.
+    auto run = [&](int word, int i) {
+        const size_t c = (size_t)(i % copies);
+        return gemm_dispatch(x, static_cast<const uint8_t*>(w) + c * w_stride, static_cast<const uint8_t*>(zs) + c * zs_stride,
+                             y, M, N, K, group_size, layout, word, none, workspace, workspace_bytes, stream);
+    };
+    int status = SQ_OK;
+    auto time_word = [&](int word, float* us) {
+        int rc = run(word, 0);
+        if (rc != SQ_OK) return rc;
+        // as many untimed launches as timed ones: clocks and caches are in the candidate's own steady state
+        for (int i = 1; i < reps; i++) (void)run(word, i);
+        if (hipEventRecord(e0, st) != hipSuccess) return (int)SQ_ERR_LAUNCH;
+        for (int i = 0; i < reps; i++) rc |= run(word, i + reps);
+        if (hipEventRecord(e1, st) != hipSuccess || hipEventSynchronize(e1) != hipSuccess) return (int)SQ_ERR_LAUNCH;
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess) return (int)SQ_ERR_LAUNCH;
+        *us = ms * 1000.f / (float)reps;
+        return rc;
+    };
+    // the built-in choice first (with any earlier measurement of this shape out of the way)
+    float t_auto = 0.f;
+    {
+        std::lock_guard<std::mutex> lock(g_tuned_mutex);
+        const int n = g_tuned_count.load(std::memory_order_relaxed);
+        for (int i = 0; i < n; i++) {
+            TunedEntry& e = g_tuned[i];
+            if (e.M == M && e.N == N && e.K == K && e.g == group_size && e.has_ws == (int)has_ws) e.M = -1;
+        }
+    }
+    for (int i = 0; i < 2 * reps; i++) (void)run(SQ_ALGO_AUTO, i);  // out of the idle state before anything is timed
+    status = time_word(SQ_ALGO_AUTO, &t_auto);
+    int best = 0;
+    float t_best = t_auto;
+    if (status == SQ_OK) {
+        int words[96];
+        const int n = autotune_candidates(M, K, group_size, has_ws, words, 96);
+        for (int i = 0; i < n; i++) {
+            float t = 0.f;
+            const int rc = time_word(words[i], &t);
+            if (rc == SQ_ERR_LAUNCH) {
+                status = rc;
+                break;
+            }
+            if (rc == SQ_OK && t < t_best) {
+                t_best = t;
+                best = words[i];
+            }
+        }
+    }
+    if (status == SQ_OK && best != 0) {
+        // A candidate has to beat the built-in choice twice, the second time against a fresh timing of both (the
+        // clocks of this part move with the load, and an early window can read a few percent off).
+        float t_auto2 = 0.f, t_best2 = 0.f;
+        if (time_word(SQ_ALGO_AUTO, &t_auto2) == SQ_OK && time_word(best, &t_best2) == SQ_OK) {
+            if (t_auto2 < t_auto) t_auto = t_auto2;
+            if (t_best2 > t_best) t_best = t_best2;
+            if (t_best >= 0.99f * t_auto) {
+                best = 0;
+                t_best = t_auto;
+            }
+        }
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (status != SQ_OK) return status;
+    // leave the caller's output as the chosen kernel writes it
+    status = run(best, 0);
+    if (status != SQ_OK) return status;
+    if (best != 0) {
+        std::lock_guard<std::mutex> lock(g_tuned_mutex);
+        const int n = g_tuned_count.load(std::memory_order_relaxed);
+        if (n < TUNED_MAX) {
+            g_tuned[n] = TunedEntry{M, N, K, group_size, (int)has_ws, best, t_best};
+            g_tuned_count.store(n + 1, std::memory_order_release);
+        }
+    }
+    if (best_algo) *best_algo = best;
+    if (best_us) *best_us = t_best;
+    if (auto_us) *auto_us = t_auto;
+    return SQ_OK;
+}
+
+int sq_w4a16_autotune_clear(void) {
+    std::lock_guard<std::mutex> lock(g_tuned_mutex);
+    const int n = g_tuned_count.load(std::memory_order_relaxed);
+    int live = 0;
+    for (int i = 0; i < n; i++) {  // readers may be scanning: entries are voided, never moved
+        if (g_tuned[i].M >= 0) live++;
+        g_tuned[i].M = -1;
+    }
+    return live;
 }
 
 int sq_w4a16_gemm_static_ws(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,

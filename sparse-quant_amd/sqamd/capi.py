@@ -31,6 +31,10 @@ SIGNATURES = {
     "sq_w4a16_gemm_fused": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, ctypes.c_size_t, _vp]),
     "sq_w4a16_gemm_silu_dot": (_i, [_vp] * 7 + [_i] * 5 + [_vp, ctypes.c_size_t, _vp]),
     "sq_w4a16_workspace_bytes": (ctypes.c_size_t, [_i, _i, _i]),
+    "sq_w4a16_autotune": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, ctypes.c_size_t, _i, ctypes.c_size_t,
+                               ctypes.c_size_t, _i, _vp, ctypes.POINTER(_i), ctypes.POINTER(ctypes.c_float),
+                               ctypes.POINTER(ctypes.c_float)]),
+    "sq_w4a16_autotune_clear": (_i, []),
     "sq_workspace_reset": (_i, [_vp, ctypes.c_size_t, _vp]),
     "sq_workspace_check": (_i, [_vp, ctypes.c_size_t, _vp]),
     "sq_w4a16_dequant": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
@@ -192,6 +196,26 @@ def gemm_ws(x, w, zs, n, k, group_size, algo=SQ_ALGO_AUTO, out=None, stream=None
     _check(lib().sq_w4a16_gemm_ws(_ptr(x), _ptr(w), _ptr(zs), _ptr(out), m, n, k, group_size, SQ_LAYOUT_L1, algo,
                                   _ptr(ws), ws.numel(), _stream(stream)), "sq_w4a16_gemm_ws")
     return out
+
+
+def autotune(x, w, zs, n, k, group_size, ws=None, reps=20, out=None, stream=None):
+    """Time every kernel that can serve this shape (sq_w4a16_autotune; synchronises) and record the fastest for
+    SQ_ALGO_AUTO.  w uint8 [N, K/2] or a pool [copies, N, K/2] with zs [copies, N, 2K/g] (timed in rotation, i.e.
+    from HBM when the pool exceeds the last-level cache).  Returns (kernel word or 0, best us, built-in us)."""
+    m = x.numel() // k
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
+    copies = w.shape[0] if w.dim() == 3 else 1
+    best, t_best, t_auto = ctypes.c_int(0), ctypes.c_float(0), ctypes.c_float(0)
+    _check(lib().sq_w4a16_autotune(_ptr(x), _ptr(w), _ptr(zs), _ptr(out), m, n, k, group_size, SQ_LAYOUT_L1, _ptr(ws),
+                                   0 if ws is None else ws.numel(), copies, n * k // 2, n * (k // group_size) * 4,
+                                   int(reps), _stream(stream), ctypes.byref(best), ctypes.byref(t_best),
+                                   ctypes.byref(t_auto)), "sq_w4a16_autotune")
+    return best.value, t_best.value, t_auto.value
+
+
+def autotune_clear():
+    return lib().sq_w4a16_autotune_clear()
 
 
 SQ_ERR_STATIC_WS = 9

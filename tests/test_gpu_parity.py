@@ -857,3 +857,30 @@ def test_read_probe_runs_on_every_reference_shape(capi):
         assert rc == 0
     torch.cuda.synchronize()
     assert capi.probes().sq_read_probe(None, None, out.data_ptr(), 4096, 4096, 128, None) == capi.SQ_ERR_NULL_POINTER
+
+
+def test_measured_kernel_choice_is_recorded_and_used(capi):
+    """sq_w4a16_autotune times every kernel that can serve a shape and records the fastest for SQ_ALGO_AUTO: the
+    recorded word is one sq_w4a16_gemm_ex accepts, the automatic path then gives that kernel's result bit for bit
+    and stays within the bar of the oracle; clearing forgets the choice."""
+    g = 128
+    capi.autotune_clear()
+    for m, n, k in ((8, 1024, 8192), (32, 2048, 2048), (96, 1536, 4096)):
+        d = orc.synth_linear(n, k, g, seed=m + n)
+        w, zs = to_dev(d["w_l1"]), to_dev(d["zs_l1"])
+        x = to_dev(orc.synth_x(m, k, seed=m))
+        ws = capi.workspace(m, n, k, DEV)
+        y_tuned = torch.empty((m, n), dtype=torch.float16, device=DEV)
+        word, t_best, t_auto = capi.autotune(x, w, zs, n, k, g, ws=ws, reps=5, out=y_tuned)
+        assert 0 < t_best <= t_auto
+        y_ref = orc.gemm_ref(orc.synth_x(m, k, seed=m), orc.dequant_l1(d["w_l1"], d["zs_l1"], g))
+        assert np.max(np.abs(y_tuned.float().cpu().numpy() - y_ref)) <= TOL * np.max(np.abs(y_ref))
+        y_auto = capi.gemm_ws(x, w, zs, n, k, g, ws=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(y_auto, y_tuned)
+        if word:
+            y_ex = capi.gemm_ws(x, w, zs, n, k, g, algo=word, ws=ws)
+            torch.cuda.synchronize()
+            assert torch.equal(y_ex, y_tuned)
+    capi.autotune_clear()
+    assert capi.autotune_clear() == 0
