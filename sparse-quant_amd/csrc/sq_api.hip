@@ -85,6 +85,79 @@ int tuned_lookup(int M, int N, int K, int g, bool has_ws) {
     return 0;
 }
 
+// The built-in kernel choice as a table: the first row whose token range contains M, whose `need` properties all
+// hold and whose `forbid` properties all fail names the kernel.  Every row carries the measurement it rests on
+// (MI355X, cold weights, OPT-6.7B / Llama-2-7B shapes, us per launch).  sq_w4a16_autotune overrides the table per
+// shape with a measurement of that shape.
+enum : unsigned {
+    P_LARGE = 1u << 0,      // N * K >= 2^25 elements (fc1 / fc2 class)
+    P_WS = 1u << 1,         // a workspace for the decode kernels' K split is at hand
+    P_GEMM_WS = 1u << 2,    // a workspace for the tiled GEMM's K split is at hand
+    P_G128 = 1u << 3,       // group size 128
+    P_G128_64 = 1u << 4,    // group size 128 or 64
+    P_K128 = 1u << 5,       // K a multiple of 128
+    P_K256 = 1u << 6,       // K a multiple of 256
+    P_K_LE_4096 = 1u << 7,
+    P_K_LE_8192 = 1u << 8,
+    P_K_LE_32768 = 1u << 9,
+    P_WIDE = 1u << 10,      // 64-row blocks (times the K split) of the two-tile streaming kernel fill half the chip
+};
+constexpr int ALGO_TWO_BLOCKS = 100;  // internal: the split-K decode kernel on two blocks of up to 32 tokens
+struct ChoiceRule {
+    int m_lo, m_hi;
+    unsigned need, forbid;
+    int kernel;
+    const char* measured;
+};
+const ChoiceRule kChoiceRules[] = {
+    // the streaming decode kernel, 5..16 tokens (3..4 on large weights); K beyond 4096 is split through the workspace
+    {5, 16, P_G128_64 | P_K128 | P_K_LE_4096, 0, SQ_ALGO_STREAM,
+     "8 tokens: fc1 10.0 vs 13.3 (split-K kernel), q/k/v in one launch 8.6 vs 12.1, 4096x4096 4.9 vs 6.5 (GEMV)"},
+    {5, 16, P_G128_64 | P_K128 | P_WS | P_K_LE_32768, 0, SQ_ALGO_STREAM, "8 tokens: fc2 12.7 vs 14.6 (split-K kernel)"},
+    {3, 4, P_LARGE | P_G128_64 | P_K128 | P_K_LE_4096, 0, SQ_ALGO_STREAM, "4 tokens: fc1 9.7 vs 10.7 (GEMV)"},
+    {3, 4, P_LARGE | P_G128_64 | P_K128 | P_WS | P_K_LE_32768, 0, SQ_ALGO_STREAM, "4 tokens: fc2 11.9 vs 13.6 (GEMV)"},
+    // its two-tile variant, 17..32 tokens
+    {17, 32, P_G128 | P_WIDE, 0, SQ_ALGO_STREAM,
+     "32 tokens: fc1 16.5 vs 17.2 (split-K kernel), q/k/v-sized 14.3 vs 15.5, fc2 18.1 vs 19.0"},
+    // the tiled GEMM with every operand through LDS and K split through the workspace, beyond 32 tokens
+    {33, 1 << 30, P_K256 | P_GEMM_WS, 0, SQ_ALGO_GEMM,
+     "48 tokens: 4096x4096 14.5 vs 17.2 (two blocks of the split-K kernel), fc1 24.7 vs 28.2, fc2 27.0 vs 32.3; "
+     "64 tokens: 14.5 vs 20.5 (16-column kernel)"},
+    // the split-K decode kernel: where the streaming kernels do not apply (group size 32, K no multiple of 128,
+    // grids that leave the two-tile kernel under half the chip such as 4096x4096 at 17..32 tokens)
+    {5, 32, P_WS | P_LARGE, 0, SQ_ALGO_SKINNY_WS, "16 tokens: fc1 12.5, fc2 14.7 vs 16-column kernel 19.6 / 21.7"},
+    {17, 32, P_WS, 0, SQ_ALGO_SKINNY_WS, "32 tokens: 4096x4096 9.8 vs 10.2 (two-tile kernel at 64 rows x 2048 columns)"},
+    {5, 32, P_WS, P_K_LE_8192, SQ_ALGO_SKINNY_WS, "long K: one workgroup per 16 rows cannot stage the activations in one round"},
+    {33, 48, P_WS | P_LARGE, 0, ALGO_TWO_BLOCKS, "33..48 tokens without the GEMM's workspace: fc1 30 vs 31 (tiled GEMM), fc2 35 vs 37"},
+    {33, 48, P_WS, P_K_LE_8192, ALGO_TWO_BLOCKS, "as above, long K"},
+    // the decode GEMV: up to 4 tokens, up to 8 while its staged activations fit one round
+    {1, 4, 0, 0, SQ_ALGO_GEMV_FIXUP, "1 token: the four-launch layer step 27.3 per step; 4096x4096 at 4 tokens 4.4"},
+    {5, 8, P_K_LE_8192, 0, SQ_ALGO_GEMV_FIXUP, "8 tokens at group size 32 (no streaming kernel): 6.5 vs 8.1 (16-column kernel)"},
+    // the 16-column kernel: no workspace, or small weights at 33..64 tokens
+    {5, 32, 0, 0, SQ_ALGO_SKINNY, "no workspace: the only kernel of this range that needs none"},
+    {33, 64, P_K_LE_8192, P_LARGE, SQ_ALGO_SKINNY, "4096x4096 at 64 tokens without the GEMM's workspace: 21 vs 46 (unsplit GEMM)"},
+    {33, 64, 0, P_GEMM_WS | P_K_LE_8192, SQ_ALGO_SKINNY, "4096x16384 at 64 tokens without a workspace: 70 vs 170 (unsplit GEMM)"},
+    {1, 1 << 30, 0, 0, SQ_ALGO_GEMM, "everything else: the tiled GEMM (plan_gemm picks tile height, staging and split)"},
+};
+
+int builtin_choice(int M, int N, int K, int g, bool ws_ok, bool gemm_ws) {
+    unsigned p = 0;
+    if ((long)N * (long)K >= (1L << 25)) p |= P_LARGE;
+    if (ws_ok) p |= P_WS;
+    if (gemm_ws) p |= P_GEMM_WS;
+    if (g == 128) p |= P_G128;
+    if (g == 128 || g == 64) p |= P_G128_64;
+    if (K % 128 == 0) p |= P_K128;
+    if (K % 256 == 0) p |= P_K256;
+    if (K <= 4096) p |= P_K_LE_4096;
+    if (K <= 8192) p |= P_K_LE_8192;
+    if (K <= 32768) p |= P_K_LE_32768;
+    if (M > 16 && M <= 32 && g == 128 && sq::skinny3_wide_applies(N, K, ws_ok)) p |= P_WIDE;
+    for (const ChoiceRule& r : kChoiceRules)
+        if (M >= r.m_lo && M <= r.m_hi && (p & r.need) == r.need && (p & r.forbid) == 0) return r.kernel;
+    return SQ_ALGO_GEMM;
+}
+
 int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, int N, int K, int group_size,
                   int layout, int algo, sq::Epilogue epi, void* workspace, size_t workspace_bytes, void* stream) {
     if (M < 0) return SQ_ERR_BAD_SHAPE;
@@ -109,44 +182,13 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
         }
     }
     if (kernel == SQ_ALGO_AUTO) {
-        // Measured on OPT-6.7B shapes.  With a workspace the split-K kernel wins for 5..32
-        // tokens once the weight is large enough (fc1/fc2 class) or K is long, and for 17..32
-        // tokens on any weight.  Without one: the GEMV up to 4 tokens (up to 8 when K is short: its staged
-        // activations would otherwise need several sequential rounds), the 16-column kernel up
-        // to 32, the tiled GEMM beyond.
-        const bool large = (long)N * (long)K >= (1L << 25);
         const bool ws_ok = workspace && aligned16(workspace) &&
                            workspace_bytes >= sq::skinny2_workspace_bytes(M > 32 ? 32 : M, N, K) &&
                            (N + 63) / 64 <= 16384;
         const bool gemm_ws = workspace && aligned16(workspace) && M > 32 &&
                              workspace_bytes >= sq::gemm_workspace_bytes(M, N, K);
-        // 5..16 tokens at group size 128: the streaming kernel wherever its K range fits (a K beyond 4096
-        // needs the workspace).  Against the split-K kernel at 8 tokens: fc1 10.0 against 13.3 us, q/k/v in
-        // one launch 8.6 against 12.1, fc2 12.7 against 14.6; against the GEMV on 4096 x 4096: 4.9 against 6.5.
-        // With 3 or 4 tokens it also beats the GEMV on fc1 / fc2-class weights (9.7 against 10.7 us, 11.9 against
-        // 13.6 us at 4 tokens); on 4096 x 4096 and with 1 or 2 tokens the GEMV stays ahead.
-        const bool stream_ok = (M > 4 || (M >= 3 && large)) && M <= 16 && (group_size == 128 || group_size == 64) &&
-                               K % 128 == 0 &&
-                               (K <= 4096 || (ws_ok && K <= 32768));
-        // 17..32 tokens at group size 128: the two-tile variant of the streaming kernel where 64-row blocks (times the
-        // K split) fill at least half the chip (fc1 at 32 tokens 16.5 against 17.2 us, q/k/v-sized 14.3 against 15.5,
-        // fc2 18.1 against 19.0)
-        const bool wide_ok = M > 16 && M <= 32 && group_size == 128 && sq::skinny3_wide_applies(N, K, ws_ok);
-        // more than 32 tokens at group size 32, 64 or 128: the tiled kernel with both operands through LDS and K split
-        // through the workspace (4096 x 4096 at 48 tokens 14.5 us against 17.2 for two blocks of the split-K
-        // decode kernel, fc1 24.7 against 28.2, fc2 27.0 against 32.3; at 64 tokens 14.5 against 20.5 for the
-        // 16-column kernel)
-        const bool lds_ok = M > 32 && (group_size == 128 || group_size == 64 || group_size == 32) && K % 256 == 0 && gemm_ws;
-        if (stream_ok || wide_ok) {
-            kernel = SQ_ALGO_STREAM;
-        } else if (lds_ok) {
-            kernel = SQ_ALGO_GEMM;
-        } else if (ws_ok && M > 4 && M <= 32 && (large || M > 16 || K > 8192)) {
-            kernel = SQ_ALGO_SKINNY_WS;
-        } else if (ws_ok && M > 32 && M <= 48 && (large || K > 8192)) {
-            // 33..48 tokens on a large weight: two blocks through the split-K decode kernel are
-            // still a little faster than the tiled GEMM with K split (fc1: 30 us against 31 us,
-            // fc2: 35 us against 37 us); beyond that the GEMM takes over.
+        kernel = builtin_choice(M, N, K, group_size, ws_ok, gemm_ws);
+        if (kernel == ALGO_TWO_BLOCKS) {
             for (int m0 = 0; m0 < M; m0 += 32) {
                 const int mb = M - m0 < 32 ? M - m0 : 32;
                 sq::Epilogue e = epi;
@@ -158,15 +200,6 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
                 if (err != hipSuccess) return SQ_ERR_LAUNCH;
             }
             return SQ_OK;
-        } else if (M <= 4 || (M <= 8 && K <= 8192)) {
-            kernel = SQ_ALGO_GEMV_FIXUP;
-        } else if (M <= 32 || (M <= 64 && ((!large && K <= 8192) || (!gemm_ws && K > 8192)))) {
-            // 33..64 tokens: the 16-column kernel on small weights (4096 x 4096: 21 us against
-            // 19 us for the GEMM with K split, 46 us without), and on long K when no workspace
-            // allows the GEMM to split K (4096 x 16384: 70 us against 170 us unsplit).
-            kernel = SQ_ALGO_SKINNY;
-        } else {
-            kernel = SQ_ALGO_GEMM;
         }
     }
     switch (kernel) {
