@@ -245,9 +245,10 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
     step_s = decode_s / steps
     return {
         **extra,
-        "weights": "random packed int4, zeros U{0..15}, scales |N(0,%g)|+%g (smaller than the single-linear "
-                   "benchmark's |N(0,0.02)|+1e-3 so that 32 random layers stay finite in fp16)"
-                   % (scale_std, scale_min),
+        "weights": "random packed int4, zeros U{0..15}, scales |N(0,%g)|+%g%s" % (
+            scale_std, scale_min,
+            " (smaller than the single-linear benchmark's |N(0,0.02)|+1e-3 so that 32 random layers stay finite in fp16)"
+            if scale_std < 0.02 else " (the single-linear benchmark's distribution)"),
         "batch": batch, "prompt": prompt, "new_tokens": new_tokens, "layers": layers,
         "launch": "hip-graph replay" if graph is not None else "eager",
         "fused": "bias+relu+residual in the GEMM store" + ("; q/k/v one launch" if fuse_qkv else "") +
