@@ -884,3 +884,46 @@ def test_measured_kernel_choice_is_recorded_and_used(capi):
             assert torch.equal(y_ex, y_tuned)
     capi.autotune_clear()
     assert capi.autotune_clear() == 0
+
+
+# ------------------------------------------------------------------ seeded random shapes through the built-in choice
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_shapes_fused_auto_dispatch(capi, seed):
+    """Eighty seeded random (M, N, K, group, bias, residual, activation) cases per seed through SQ_ALGO_AUTO, each
+    with and without a workspace (so that every kernel family the rule table can pick is reached at shapes nobody
+    tuned), against the oracle's fp32 result and the fp32 epilogue formula."""
+    rng = np.random.default_rng(seed)
+    for c in range(80):
+        g = int(rng.choice([32, 64, 128]))
+        if rng.random() < 0.7:
+            k = max(g, 128) * int(rng.choice([1, 2, 3, 4, 5, 8, 11, 16, 32, 43]))
+        else:
+            k = g * int(rng.integers(1, 40))
+        k = max((k + 31) // 32 * 32, g)
+        n = int(rng.choice([8, 16, 24, 40, 64, 72, 128, 136, 256, 264, 520, 1024, 1032, 2048, 4096]))
+        m = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 24, 31, 32, 33, 48, 64, 65, 100, 128, 129, 200, 257,
+                            512, 700]))
+        if n * k > 4096 * 8192:
+            k = 1024
+        d = orc.synth_linear(n, k, g, seed=1000 * seed + c)
+        w_hat = orc.dequant_l1(d["w_l1"], d["zs_l1"], g)
+        x = orc.synth_x(m, k, seed=1000 * seed + c + 500)
+        use_b, use_r, act = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), int(rng.integers(0, 3))
+        bias = (rng.standard_normal(n) * 2).astype(np.float16) if use_b else None
+        res = (rng.standard_normal((m, n)) * 2).astype(np.float16) if use_r else None
+        z = orc.gemm_ref(x, w_hat) + (bias.astype(np.float32) if use_b else 0)
+        if act == capi.SQ_ACT_RELU:
+            z = np.maximum(z, 0)
+        elif act == capi.SQ_ACT_SILU:
+            z = z / (1 + np.exp(-z))
+        y_ref = z + (res.astype(np.float32) if use_r else 0)
+        xd, wd, zd = to_dev(x), to_dev(d["w_l1"]), to_dev(d["zs_l1"])
+        bd = to_dev(bias) if use_b else None
+        rd = to_dev(res) if use_r else None
+        for use_ws in (False, True):
+            y = capi.gemm_fused(xd, wd, zd, n, k, g, bias=bd, residual=rd, act=act, use_workspace=use_ws)
+            torch.cuda.synchronize()
+            y = y.float().cpu().numpy()
+            what = (seed, c, m, n, k, g, use_b, use_r, act, use_ws)
+            assert np.all(np.isfinite(y)), what
+            assert np.max(np.abs(y - y_ref)) <= TOL * max(np.max(np.abs(y_ref)), 1e-6), what
