@@ -180,7 +180,13 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     // (fused LayerNorm, while the first weights are on their way: thread t holds columns 8t .. 8t+7 of every
     // token.  Per-thread partial sums go to LDS (the activations' space, not yet in use), wave w adds up the 512
     // partials of token w and leaves the statistic where every thread reads it; mean first, then the squared
-    // deviations around it.  The normalised row replaces the raw one before it is parked.)
+    // deviations around it.  Every workgroup normalises all MROWS x K activations itself, so this is vector
+    // arithmetic on the critical path of every CU: it runs on fp16 pairs.  Sums are two-wide dot products with
+    // fp32 accumulation; the deviations are taken in fp16 around the fp16-rounded mean mh (the difference of two
+    // fp16 numbers loses nothing that matters), the statistics correct for delta = mean - mh exactly
+    // (var = E[(x - mh)^2] - delta^2, normalised value = (x - mh) * r - delta * r), and 1 / sigma enters as a
+    // sum of two fp16 numbers so that its rounding does not scale the whole row.  The normalised row replaces
+    // the raw one before it is parked.)
     if (LN) {
         float* scr = (float*)sk3_lds;                    // [MROWS][512] partials
         float* stat = (float*)(sk3_lds + L::LN_OFF);     // [2][MROWS]: mean, 1 / sqrt(var + eps)
@@ -199,42 +205,59 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
                                    bit_cast<float>(__builtin_amdgcn_readlane(bit_cast<int>(a), 16))) +
                                   (bit_cast<float>(__builtin_amdgcn_readlane(bit_cast<int>(a), 32)) +
                                    bit_cast<float>(__builtin_amdgcn_readlane(bit_cast<int>(a), 48)));
-                if (lane == 0) stat[which * MROWS + wave] = finish_var ? rsqrtf(tot * inv_k + ln.eps) : tot * inv_k;
+                if (lane == 0) {
+                    if (finish_var) {
+                        const float mean_w = stat[wave];
+                        const float dl = mean_w - (float)(half_t)mean_w;
+                        stat[MROWS + wave] = rsqrtf(fmaxf(tot * inv_k - dl * dl, 0.f) + ln.eps);
+                    } else {
+                        stat[wave] = tot * inv_k;
+                    }
+                }
             }
             sk3_barrier();
         };
-        float part[XPT], mean[XPT];
+        const half2_t one2 = {(half_t)1.f, (half_t)1.f};
+        float part[XPT], delta[XPT];
 #pragma unroll
         for (int p = 0; p < XPT; p++) {
-            const half8_t h = bit_cast<half8_t>(xr[p]);
             float a = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; e++) a += (float)h[e];
+            for (int e = 0; e < 4; e++) a = __builtin_amdgcn_fdot2(bit_cast<half2_t>(xr[p][e]), one2, a, false);
             part[p] = a;  // zero where the token or the column does not exist
         }
         token_sums(part, 0, false);
 #pragma unroll
         for (int p = 0; p < XPT; p++) {
-            mean[p] = stat[p];
-            const half8_t h = bit_cast<half8_t>(xr[p]);
+            const float mean = stat[p];
+            const half_t mh = (half_t)mean;
+            delta[p] = mean - (float)mh;
+            const half2_t mh2 = {mh, mh};
             float q = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const float dlt = (float)h[e] - mean[p];
-                q += dlt * dlt;
+            for (int e = 0; e < 4; e++) {
+                const half2_t d = bit_cast<half2_t>(xr[p][e]) - mh2;
+                xr[p][e] = bit_cast<uint32_t>(d);
+                q = __builtin_amdgcn_fdot2(d, d, q, false);
             }
             part[p] = cok ? q : 0.f;
         }
         token_sums(part, 1, true);
-        const half8_t g8 = bit_cast<half8_t>(lg), b8 = bit_cast<half8_t>(lb);
 #pragma unroll
         for (int p = 0; p < XPT; p++) {
             const float rstd = stat[MROWS + p];
-            const half8_t h = bit_cast<half8_t>(xr[p]);
-            half8_t o;
+            const half_t rh = (half_t)rstd;
+            const half_t rl = (half_t)(rstd - (float)rh);
+            const half_t ch = (half_t)(-delta[p] * rstd);
+            const half2_t rh2 = {rh, rh}, rl2 = {rl, rl}, c2 = {ch, ch};
+            u32x4_t o;
 #pragma unroll
-            for (int e = 0; e < 8; e++) o[e] = (half_t)(((float)h[e] - mean[p]) * rstd * (float)g8[e] + (float)b8[e]);
-            xr[p] = (cok && p < M) ? bit_cast<u32x4_t>(o) : (u32x4_t){0u, 0u, 0u, 0u};
+            for (int e = 0; e < 4; e++) {
+                const half2_t d = bit_cast<half2_t>(xr[p][e]);
+                const half2_t t = d * rh2 + (d * rl2 + c2);
+                o[e] = bit_cast<uint32_t>(t * bit_cast<half2_t>(lg[e]) + bit_cast<half2_t>(lb[e]));
+            }
+            xr[p] = (cok && p < M) ? o : (u32x4_t){0u, 0u, 0u, 0u};
         }
         sk3_barrier();  // the partials' space becomes the activations' space
     }
