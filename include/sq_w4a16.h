@@ -386,9 +386,11 @@ int sq_layernorm(const void* x, const void* gamma, const void* beta, void* y, in
  * and no LayerNorm launch, no normalised copy in memory and no second read of it exist; x_norm is then not
  * touched and may be NULL.  Otherwise sq_layernorm writes x_norm [M, K] (fp16, caller-allocated, must not be NULL)
  * and the linear runs on it through the automatic dispatch (workspace as for sq_w4a16_gemm_fused, may be NULL).
- * Same arithmetic as sq_layernorm (fp32 statistics, mean first, then the variance around it, one rounding to
- * fp16); the summation order of the statistics differs, so the normalised row can differ from sq_layernorm's by
- * one fp16 ulp in rare elements.  ln_gamma / ln_beta fp16 [K] or NULL. */
+ * Inside the kernel the statistics are fp32 (mean first, then the variance around it) and the normalisation
+ * runs on fp16 pairs: the deviations are taken around the fp16-rounded mean with the remainder carried exactly,
+ * 1 / sigma enters as the sum of two fp16 numbers, gamma and beta are applied in fp16; the normalised row can
+ * differ from sq_layernorm's (one rounding from fp32) by an fp16 ulp or two per element.  ln_gamma / ln_beta
+ * fp16 [K] or NULL. */
 int sq_w4a16_ln_fusable(int M, int N, int K, int group_size, int layout);
 int sq_w4a16_gemm_ln_fused(const void* x, const void* ln_gamma, const void* ln_beta, float ln_eps, void* x_norm,
                            const void* w, const void* zs, const void* bias, const void* residual, void* y, int M, int N,

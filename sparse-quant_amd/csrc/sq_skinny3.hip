@@ -172,7 +172,12 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     };
     // (in front of a fused LayerNorm a 16-row workgroup, whose units are two loads, sends two of them: measured)
     constexpr int PRE = (LN && RT == 1) ? 2 : SK3_DEPTH_PRE;
-    constexpr int STEADY = LN ? (DEPTH > PRE ? DEPTH : PRE) : DEPTH;
+    // (and 48-row workgroups one more once the activations have arrived, ahead of the LayerNorm arithmetic: the
+    // memory system otherwise runs dry while every wave works on the activations.  Measured at 8 tokens:
+    // 12288 x 4096 in 48-row workgroups 9.3 -> 8.8 us; 16384 x 4096 in 64-row workgroups 11.5 -> 12.0 us, so
+    // those keep one unit.)
+    constexpr int MID = (LN && RT == 3) ? 1 : 0;
+    constexpr int STEADY = LN ? (DEPTH > PRE + MID ? DEPTH : PRE + MID) : DEPTH;
 #pragma unroll
     for (int un = 0; un < NU; un++)
         if (un < PRE) issue_unit(un);
@@ -226,6 +231,11 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
             for (int e = 0; e < 4; e++) a = __builtin_amdgcn_fdot2(bit_cast<half2_t>(xr[p][e]), one2, a, false);
             part[p] = a;  // zero where the token or the column does not exist
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int un = PRE; un < NU; un++)
+            if (un < PRE + MID) issue_unit(un);
+        __builtin_amdgcn_sched_barrier(0);
         token_sums(part, 0, false);
 #pragma unroll
         for (int p = 0; p < XPT; p++) {
@@ -285,7 +295,7 @@ __device__ __forceinline__ void skinny3_body(const uint8_t* __restrict__ W, cons
     const half8_t m960 = {(half_t)-960.f, (half_t)-960.f, (half_t)0.f, (half_t)0.f,
                           (half_t)-960.f, (half_t)-960.f, (half_t)0.f, (half_t)0.f};
 #pragma unroll
-    for (int un = PRE; un < NU; un++)
+    for (int un = PRE + MID; un < NU; un++)
         if (un < STEADY) issue_unit(un);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
