@@ -488,15 +488,10 @@ struct GemmPlan {
     int mi, ksplit, pipe;
     int lds = 0;  // 1: gemm_lds_kernel (group size 32, 64 or 128, K a multiple of 256)
 };
-// Group size 32, 64 or 128 with K a multiple of 256 and more than 32 tokens: gemm_lds_kernel, whose choices
-// come from a sweep of tile height x split over 4096 x 4096, 16384 x 4096, 4096 x 16384,
-// 11008 x 4096, 4096 x 11008 and 12288 x 4096 at 48..4096 tokens (within a few percent of the best
-// swept configuration on all of them): 32-row tiles up to 64 tokens on narrow weights (up to 128
-// when K is short as well), 128-row tiles beyond 256 tokens when the weight is wide or K long and
-// always beyond 1024, 64-row tiles between; K split while the grid stays within one round of 256
-// workgroups and every part keeps 8 steps.  Only a long K whose 256 x 256 tiles fill whole rounds
-// stays with the pipelined kernel (4096 x 16384 at 4096 tokens: 497 against 530 us); at group size 32, where
-// this kernel refills its zeros/scales every step, any K does (fc1 at 2048 tokens: 285 against 302 us).
+// Group size 32, 64 or 128 with K a multiple of 256 and more than 32 tokens: gemm_lds_kernel; tile height and K
+// split come from the cost model below.  Only a long K whose 256 x 256 tiles fill whole rounds stays with the
+// pipelined kernel (4096 x 16384 at 4096 tokens: 497 against 530 us); at group size 32, where this kernel refills
+// its zeros/scales every step, any K does (fc1 at 2048 tokens: 285 against 302 us).
 static GemmPlan plan_gemm_lds(int M, long ncol, int nit, int g, bool have_ws) {
     GemmPlan p = {1, 1, -1};
     const long t256 = ncol * ((M + 255) / 256);
@@ -506,18 +501,40 @@ static GemmPlan plan_gemm_lds(int M, long ncol, int nit, int g, bool have_ws) {
         return p;
     }
     p.lds = 1;
-    const bool wide_or_long = ncol >= 32 || nit >= 128;
-    if (M <= 64)
-        p.mi = ncol >= 32 ? 2 : 1;
-    else if (M <= 128)
-        p.mi = wide_or_long ? 2 : 1;
-    else if (M <= 256)
-        p.mi = 2;
-    else
-        p.mi = (wide_or_long || M > 1024) ? 4 : 2;
-    const long t = ncol * ((M + 32 * p.mi - 1) / (32 * p.mi));
-    if (have_ws && t <= 16384)
-        while (p.ksplit < 8 && t * p.ksplit * 2 <= 256 && nit / (p.ksplit * 2) >= 8) p.ksplit *= 2;
+    // Tile height (32 mi rows) and K split by a cost model fitted to timings of all twelve combinations on 17 weights
+    // x 7 token counts (48..2048 tokens; 768 x 3072 to 8192 x 28672): a workgroup alone on its CU takes
+    // a1[mi] us per K step, one that shares its CU a2[mi] (two fit), plus b[mi] per workgroup; W workgroups run in
+    // rounds of 512; a K split adds the exchange of the partial tiles.  The model's choice is within 1 % of the best
+    // combination in the geometric mean over those 119 points (worst case 12 %); the rule it replaces (tile height by
+    // token count, K split only below 128 tiles) was within 5 % (worst 81 %: 1024 x 1024 at 2048 tokens ran 64
+    // workgroups).
+    static const float a1[3] = {0.456f, 0.528f, 0.821f}, a2[3] = {0.965f, 1.275f, 1.992f}, b[3] = {3.49f, 4.53f, 5.77f};
+    float best = 3.4e38f;
+    for (int i = 0; i < 3; i++) {
+        const int mi = 1 << i;
+        const long t = ncol * ((M + 32 * mi - 1) / (32 * mi));
+        for (int ks = 1; ks <= 8; ks *= 2) {
+            if (ks > 1 && (!have_ws || t > 16384 || nit / ks < 4 || t * ks * (32 * mi) * 256 * 4 > (256L << 20))) break;
+            const long W = t * ks;
+            const int steps = ((nit + ks - 1) / ks + 3) & ~3;
+            const float t1 = a1[i] * steps + b[i], t2 = a2[i] * steps + b[i];
+            float cost;
+            if (W <= 256) {
+                cost = t1;
+            } else if (W <= 512) {
+                cost = t2;
+            } else {
+                const long full = W / 512, rem = W - full * 512;
+                cost = full * t2 + (rem == 0 ? 0.f : (rem > 256 ? t2 : t1));
+            }
+            if (ks > 1) cost += 1.3f + 2.56f * mi;
+            if (cost < best) {
+                best = cost;
+                p.mi = mi;
+                p.ksplit = ks;
+            }
+        }
+    }
     return p;
 }
 
