@@ -101,6 +101,7 @@ enum : unsigned {
     P_K_LE_8192 = 1u << 8,
     P_K_LE_32768 = 1u << 9,
     P_WIDE = 1u << 10,      // 64-row blocks (times the K split) of the two-tile streaming kernel fill half the chip
+    P_SMALL = 1u << 11,     // N * K <= 2^22 elements and K <= 2048
 };
 constexpr int ALGO_TWO_BLOCKS = 100;  // internal: the split-K decode kernel on two blocks of up to 32 tokens
 struct ChoiceRule {
@@ -116,6 +117,9 @@ const ChoiceRule kChoiceRules[] = {
     {5, 16, P_G128_64 | P_K128 | P_WS | P_K_LE_32768, 0, SQ_ALGO_STREAM, "8 tokens: fc2 12.7 vs 14.6 (split-K kernel)"},
     {3, 4, P_LARGE | P_G128_64 | P_K128 | P_K_LE_4096, 0, SQ_ALGO_STREAM, "4 tokens: fc1 9.7 vs 10.7 (GEMV)"},
     {3, 4, P_LARGE | P_G128_64 | P_K128 | P_WS | P_K_LE_32768, 0, SQ_ALGO_STREAM, "4 tokens: fc2 11.9 vs 13.6 (GEMV)"},
+    // small weights at 17..32 tokens: the 16-column kernel (one launch, no exchange between workgroups)
+    {17, 32, P_SMALL, 0, SQ_ALGO_SKINNY,
+     "32 tokens: 2048x2048 7.4 vs 8.6 (split-K kernel), 1024x1024 4.9 vs 6.9, 3072x768 4.8 vs 6.6"},
     // its two-tile variant, 17..32 tokens
     {17, 32, P_G128 | P_WIDE, 0, SQ_ALGO_STREAM,
      "32 tokens: fc1 16.5 vs 17.2 (split-K kernel), q/k/v-sized 14.3 vs 15.5, fc2 18.1 vs 19.0"},
@@ -149,6 +153,7 @@ int builtin_choice(int M, int N, int K, int g, bool ws_ok, bool gemm_ws) {
     if (g == 128 || g == 64) p |= P_G128_64;
     if (K % 128 == 0) p |= P_K128;
     if (K % 256 == 0) p |= P_K256;
+    if ((long)N * (long)K <= (1L << 22) && K <= 2048) p |= P_SMALL;
     if (K <= 4096) p |= P_K_LE_4096;
     if (K <= 8192) p |= P_K_LE_8192;
     if (K <= 32768) p |= P_K_LE_32768;
