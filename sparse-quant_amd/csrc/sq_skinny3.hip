@@ -830,35 +830,65 @@ struct Sk3Plan {
     int rt, ch, ksplit;
 };
 
-Sk3Plan plan(const int* rows, int count, int K, bool have_ws, int tune) {
+Sk3Plan plan(const int* rows, int count, int K, bool have_ws, int tune, int M) {
     const int groups = K / 128;
-    Sk3Plan p{4, 4, (groups + 31) / 32};
-    if ((tune >> 4) & 0xF) p.ksplit = (tune >> 4) & 0xF;
-    const int cps = (groups + p.ksplit - 1) / p.ksplit;
-    p.ch = cps <= 8 ? 1 : cps <= 16 ? 2 : 4;
-    if (cps > 32 || (p.ksplit > 1 && !have_ws) || p.ksplit > 8 || (p.ksplit - 1) * cps >= groups) {
-        p.ksplit = 0;  // does not fit
+    const int ks0 = (groups + 31) / 32;  // the least split: a workgroup covers at most 32 chunks
+    Sk3Plan none{4, 4, 0};
+    auto shape = [&](int ks, Sk3Plan* p) {
+        p->ksplit = ks;
+        const int cps = (groups + ks - 1) / ks;
+        p->ch = cps <= 8 ? 1 : cps <= 16 ? 2 : 4;
+        return !(cps > 32 || (ks > 1 && !have_ws) || ks > 8 || (ks - 1) * cps >= groups);
+    };
+    if ((tune >> 4) & 0xF) {
+        Sk3Plan p{4, 4, 0};
+        if (!shape((tune >> 4) & 0xF, &p)) return none;
+        p.rt = (tune & 0xF) == 1 ? 1 : ((tune & 0xF) == 3 && p.ksplit == 1 && p.ch == 4) ? 3 : 4;
+        if ((tune & 0xF) == 0) {
+            // rows per workgroup by the count below, at the given split
+            int best = 1 << 30;
+            for (int rt : {4, 3, 1}) {
+                if (rt == 3 && (p.ksplit != 1 || p.ch != 4)) continue;
+                long blocks = 0;
+                for (int l = 0; l < count; l++) blocks += (rows[l] + 16 * rt - 1) / (16 * rt);
+                const long cost = (blocks * p.ksplit + 255) / 256 * (rt + 2);
+                if (cost < best) best = (int)cost, p.rt = rt;
+            }
+        }
         return p;
     }
-    // Rows per workgroup: 64, 48 or 16, whichever needs the least time by this count: rounds of 256 workgroups
-    // (one per CU) times the row tiles of a workgroup plus two for its activations (at 8 tokens the staged
-    // activations weigh as much as two row tiles of weights).  OPT-6.7B: 4096 rows -> 16 (256 workgroups),
-    // 12288 and 11008 -> 48 (256 and 230), 16384 -> 64 (256).  48-row workgroups only without a K split (their
-    // partial tiles do not fit the workspace layout) and with full-length K ranges.
-    int best = 1 << 30;
-    for (int rt : {4, 3, 1}) {
-        if (rt == 3 && (p.ksplit != 1 || p.ch != 4)) continue;
-        long blocks = 0;
-        for (int l = 0; l < count; l++) blocks += (rows[l] + 16 * rt - 1) / (16 * rt);
-        const long rounds = (blocks * p.ksplit + 255) / 256;
-        const long cost = rounds * (rt + 2);
-        if (cost < best) {
-            best = (int)cost;
-            p.rt = rt;
+    // Rows per workgroup (64, 48 or 16) and K split (the least one, or two or four times as fine) by a count of
+    // time calibrated on timed launches at 8 and 16 tokens, in units of 1.75 us (what a CU needs to stream one
+    // 16-row tile over a full range of 32 chunks): rounds of 256 workgroups (one per CU) x ((row tiles + M / 24 for
+    // the activations, which come from L2 at a sixth of the price per byte) x the part of a full range a workgroup
+    // covers + 1 for a workgroup's start: its activations must be there before its first matrix instruction),
+    // + 1.54 (2.7 us) where partial tiles are exchanged.  OPT-6.7B: 4096 rows -> 16 (256 workgroups), 12288 and
+    // 11008 -> 48 (256 and 230), 16384 -> 64 (256), 4096 x 16384 -> 64 rows x 4 ranges.  A finer split pays where
+    // the least one leaves rounds half empty: 5120 x 13824 at 16 tokens 80 x 4 = 320 workgroups (18.7 us) -> 80 x 8
+    // (15.7); 1024 x 8192 64 x 2 -> 64 x 4 with 16 rows (7.3 -> 6.4).  48-row workgroups only without a K split
+    // (their partial tiles do not fit the workspace layout) and with full-length K ranges.
+    Sk3Plan bestp = none;
+    float best = 3.4e38f;
+    for (int ks = ks0; ks <= 8 && ks <= 4 * ks0; ks *= 2) {
+        Sk3Plan p{4, 4, 0};
+        if (!shape(ks, &p)) continue;
+        const int cps = (groups + ks - 1) / ks;
+        for (int rt : {4, 3, 1}) {
+            if (rt == 3 && (ks != 1 || p.ch != 4)) continue;
+            long blocks = 0;
+            for (int l = 0; l < count; l++) blocks += (rows[l] + 16 * rt - 1) / (16 * rt);
+            const long rounds = (blocks * ks + 255) / 256;
+            const float cost = rounds * ((rt + M / 24.f) * (cps / 32.f) + 1.f) + (ks > 1 ? 1.54f : 0.f);
+            if (cost < best - 1e-3f) {
+                best = cost;
+                bestp = p;
+                bestp.rt = rt;
+            }
         }
     }
-    if (tune & 0xF) p.rt = (tune & 0xF) == 1 ? 1 : ((tune & 0xF) == 3 && p.ksplit == 1 && p.ch == 4) ? 3 : 4;
-    return p;
+    if ((tune & 0xF) && bestp.ksplit)
+        bestp.rt = (tune & 0xF) == 1 ? 1 : ((tune & 0xF) == 3 && bestp.ksplit == 1 && bestp.ch == 4) ? 3 : 4;
+    return bestp;
 }
 
 }  // namespace
@@ -870,7 +900,7 @@ Sk3Plan plan(const int* rows, int count, int K, bool have_ws, int tune) {
 hipError_t launch_skinny3_tuned(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                                 int g, int tune, Epilogue epi, const LnPre* ln, hipStream_t st) {
     if (M < 1 || M > 16 || K % 128 != 0 || (g != 128 && g != 64)) return hipErrorInvalidValue;
-    Sk3Plan p = plan(&N, 1, K, ws != nullptr, tune);
+    Sk3Plan p = plan(&N, 1, K, ws != nullptr, tune, M);
     if (p.ksplit == 0) return hipErrorInvalidValue;
     if (g == 64 && p.rt == 3) p.rt = 4;  // group size 64: 16- and 64-row workgroups only
     if (p.ksplit > 1 && (N + 16 * p.rt - 1) / (16 * p.rt) > 16384) return hipErrorInvalidValue;
@@ -1010,7 +1040,7 @@ hipError_t launch_skinny3_group(const SeqProblem* probs, int count, int M, void*
         rows[p] = probs[p].N;
         blocks64 += (probs[p].N + 63) / 64;
     }
-    const Sk3Plan pl = plan(rows, count, K, ws != nullptr, 0);
+    const Sk3Plan pl = plan(rows, count, K, ws != nullptr, 0, M);
     if (pl.ksplit == 0) return hipErrorInvalidValue;
     if (pl.ksplit > 1 && (blocks64 * (4 / pl.rt) > 16384 || ws_bytes < skinny2_group_workspace_bytes(probs, count, M)))
         return hipErrorInvalidValue;
