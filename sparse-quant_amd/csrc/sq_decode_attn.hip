@@ -165,17 +165,19 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
         m = mx;
     };
     // Two register sets take turns (a loop that copied "next" into "current" would have to wait for the
-    // requests it has just made); two batches per trip, one past the end of the share is all probability zero.
+    // requests it has just made); two batches per trip while two are left, then the odd one (a trip's last
+    // request may lie past the end of the share: it re-reads the last row and nobody consumes it).
     int base = r0 + wave * RPI * DA_U;
     if (base < r1) {
         request(base, ka, va, ma);
-        do {
+        while (base + STEP < r1) {
             request(base + STEP, kb, vb, mb_);
             consume(base, ka, va, ma);
             request(base + 2 * STEP, ka, va, ma);
             consume(base + STEP, kb, vb, mb_);
             base += 2 * STEP;
-        } while (base < r1);
+        }
+        if (base < r1) consume(base, ka, va, ma);
     }
 
     // Merge the row slots of a wave (lanes with equal c), then the waves.
