@@ -397,6 +397,28 @@ int sq_w4a16_gemm_ln_fused(const void* x, const void* ln_gamma, const void* ln_b
                            int K, int group_size, int layout, int act, void* workspace, size_t workspace_bytes,
                            void* stream);
 
+/* The ends of a greedy decode step around the quantised layers, for the end-to-end configuration (random-init
+ * OPT-6.7B, batch 8): what the reference runs as torch modules and ops -- embed_tokens + embed_positions
+ * (test/nvidia/module/opt/modeling_opt_ours.py:900-913), the fp16 lm_head (:1097, :1229), the argmax of greedy
+ * generation and the bookkeeping between two steps -- as three launches that a HIP graph can hold whole.
+ *
+ * sq_embed_rows:      out[r, :] = embed[tok[r], :] + pos_table[*pos + pos_offset, :], fp16 [rows, hidden],
+ *                     hidden % 8 == 0; tok int64 [rows], pos int64 [1] on the device; indices are clamped to
+ *                     [0, vocab) and [0, positions).  The sum is rounded once, as torch's fp16 add.
+ * sq_f16_gemv:        y[M, N] = x[M, K] w[N, K]^T, fp16 in and out, fp32 sums; M <= 8, K % 512 == 0, K <= 8192.
+ *                     part_val (float) / part_idx (int32), both or neither, [8][sq_f16_gemv_parts(N)]: per token the
+ *                     largest stored value and its row for every workgroup of the kernel's fixed grid (two per
+ *                     CU; the lowest row among equals).
+ * sq_greedy_feedback: tok[m] = the row of the best candidate of token m (lowest row among equals: torch.argmax's
+ *                     rule; NaN never wins); if history and step are given and *step < history_rows,
+ *                     history[*step, m] = tok[m]; then *pos += 1 and *step += 1 where given (int64 on the device). */
+int sq_embed_rows(const void* embed, const void* pos_table, const void* tok, const void* pos, long long pos_offset,
+                  void* out, int rows, int hidden, long long vocab, long long positions, void* stream);
+int sq_f16_gemv_parts(int N);
+int sq_f16_gemv(const void* x, const void* w, void* y, void* part_val, void* part_idx, int M, int N, int K, void* stream);
+int sq_greedy_feedback(const void* part_val, const void* part_idx, int parts, int M, void* tok, void* pos, void* history,
+                       void* step, long long history_rows, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

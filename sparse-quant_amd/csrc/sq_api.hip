@@ -829,4 +829,42 @@ int sq_w4a16_gemm_ln_fused(const void* x, const void* ln_gamma, const void* ln_b
                          stream);
 }
 
+int sq_embed_rows(const void* embed, const void* pos_table, const void* tok, const void* pos, long long pos_offset,
+                  void* out, int rows, int hidden, long long vocab, long long positions, void* stream) {
+    if (rows < 0 || hidden <= 0 || hidden % 8 != 0 || vocab <= 0 || positions <= 0) return SQ_ERR_BAD_SHAPE;
+    if (rows == 0) return SQ_OK;
+    if (!embed || !pos_table || !tok || !pos || !out) return SQ_ERR_NULL_POINTER;
+    if (!aligned16(embed) || !aligned16(pos_table) || !aligned16(out) || (reinterpret_cast<uintptr_t>(tok) & 7u) ||
+        (reinterpret_cast<uintptr_t>(pos) & 7u))
+        return SQ_ERR_MISALIGNED;
+    return launch_code(sq::launch_embed_rows(embed, pos_table, tok, pos, pos_offset, out, rows, hidden, vocab, positions,
+                                             static_cast<hipStream_t>(stream)));
+}
+
+int sq_f16_gemv_parts(int N) { return N > 0 ? sq::f16_gemv_parts(N) : 0; }
+
+int sq_f16_gemv(const void* x, const void* w, void* y, void* part_val, void* part_idx, int M, int N, int K, void* stream) {
+    if (M < 0 || M > 8 || N <= 0 || K < 512 || K % 512 != 0 || K > 8192) return SQ_ERR_BAD_SHAPE;
+    if (M == 0) return SQ_OK;
+    if (!x || !w || !y || ((part_val == nullptr) != (part_idx == nullptr))) return SQ_ERR_NULL_POINTER;
+    if (!aligned16(x) || !aligned16(w) || (reinterpret_cast<uintptr_t>(y) & 1u) ||
+        (reinterpret_cast<uintptr_t>(part_val) & 3u) || (reinterpret_cast<uintptr_t>(part_idx) & 3u))
+        return SQ_ERR_MISALIGNED;
+    return launch_code(sq::launch_f16_gemv(x, w, y, static_cast<float*>(part_val), static_cast<int*>(part_idx), M, N, K,
+                                           static_cast<hipStream_t>(stream)));
+}
+
+int sq_greedy_feedback(const void* part_val, const void* part_idx, int parts, int M, void* tok, void* pos, void* history,
+                       void* step, long long history_rows, void* stream) {
+    if (M < 0 || M > 8 || parts <= 0 || history_rows < 0) return SQ_ERR_BAD_SHAPE;
+    if (M == 0) return SQ_OK;
+    if (!part_val || !part_idx || !tok) return SQ_ERR_NULL_POINTER;
+    if ((reinterpret_cast<uintptr_t>(tok) & 7u) || (reinterpret_cast<uintptr_t>(pos) & 7u) ||
+        (reinterpret_cast<uintptr_t>(history) & 7u) || (reinterpret_cast<uintptr_t>(step) & 7u))
+        return SQ_ERR_MISALIGNED;
+    return launch_code(sq::launch_greedy_feedback(static_cast<const float*>(part_val), static_cast<const int*>(part_idx),
+                                                  parts, M, tok, pos, history, step, history_rows,
+                                                  static_cast<hipStream_t>(stream)));
+}
+
 }  // extern "C"

@@ -106,6 +106,20 @@ hipError_t launch_decode_attention(const void* q, const void* k_new, const void*
 constexpr int DECODE_ATTN_MAX_SPLIT = 16;
 size_t decode_attention_workspace_bytes(int B, int H, int D);
 
+// sq_lm_head.hip: the ends of a greedy decode step around the W4A16 layers (the end-to-end harness).
+// out[r, :] = embed[tok[r], :] + pos_table[*pos + pos_offset, :] (fp16; indices clamped to their tables).
+hipError_t launch_embed_rows(const void* embed, const void* pos_table, const void* tok, const void* pos, long long pos_offset,
+                             void* out, int rows, int hidden, long long vocab, long long positions, hipStream_t st);
+// y[M, N] = x[M, K] w[N, K]^T in fp16 with fp32 sums, M <= 8, K % 512 == 0, K <= 8192; part_val / part_idx (both or
+// neither): per token the best value and row of every workgroup, [8][f16_gemv_parts(N)].
+int f16_gemv_parts(int N);
+hipError_t launch_f16_gemv(const void* x, const void* w, void* y, float* part_val, int* part_idx, int M, int N, int K,
+                           hipStream_t st);
+// tok[m] = the row of the best candidate of token m (lowest row among equals); history[*step, m] = tok[m] when both
+// are given and *step < history_rows; then *pos += 1 and *step += 1 (each where given).
+hipError_t launch_greedy_feedback(const float* part_val, const int* part_idx, int parts, int M, void* tok, void* pos,
+                                  void* history, void* step, long long history_rows, hipStream_t st);
+
 // sq_layernorm.hip: LayerNorm over the last dimension, fp16 in/out, fp32 statistics; cols % 8 == 0,
 // cols <= 16384.
 hipError_t launch_layernorm(const void* x, const void* gamma, const void* beta, void* y, int rows, int cols, float eps,

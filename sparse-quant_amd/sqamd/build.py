@@ -28,7 +28,8 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 PROBES_PATH = os.path.join(PKG_ROOT, "libsq_probes.so")
 
 HIP_SOURCES = ["sq_api.hip", "sq_dequant.hip", "sq_repack.hip", "sq_gemv2.hip", "sq_gemv_seq.hip", "sq_skinny.hip", "sq_skinny2.hip",
-               "sq_skinny3.hip", "sq_gemm.hip", "sq_gemm2.hip", "sq_attn.hip", "sq_decode_attn.hip", "sq_layernorm.hip"]
+               "sq_skinny3.hip", "sq_gemm.hip", "sq_gemm2.hip", "sq_attn.hip", "sq_decode_attn.hip", "sq_layernorm.hip",
+               "sq_lm_head.hip"]
 PROBE_SOURCES = ["sq_probes.hip"]  # diagnostic kernels, a library of their own (include/sq_probes.h)
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
              # keep the compiler from forming packed-fp32 instructions

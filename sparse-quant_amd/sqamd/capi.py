@@ -53,6 +53,10 @@ SIGNATURES = {
     "sq_w4a16_gemm_ln_fused": (_i, [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
                                     _vp, ctypes.c_size_t, _vp]),
     "sq_lut_attention_fwd": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, ctypes.c_float, _i, _vp]),
+    "sq_embed_rows": (_i, [_vp, _vp, _vp, _vp, ctypes.c_longlong, _vp, _i, _i, ctypes.c_longlong, ctypes.c_longlong, _vp]),
+    "sq_f16_gemv_parts": (_i, [_i]),
+    "sq_f16_gemv": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "sq_greedy_feedback": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _vp, ctypes.c_longlong, _vp]),
 }
 
 # include/sq_probes.h (libsq_probes.so): diagnostic kernels used by the benchmark only.
@@ -447,6 +451,43 @@ def decode_attention(q, k_cache, v_cache, cache_len, sm_scale, k_new=None, v_new
                                      len_host, len_dev, float(sm_scale), _ptr(ws), 0 if ws is None else ws.numel(),
                                      _stream(stream)), "sq_decode_attention")
     return out
+
+
+def embed_rows(embed, pos_table, tok, pos, pos_offset=0, out=None, stream=None):
+    """out[r] = embed[tok[r]] + pos_table[pos[0] + pos_offset] through sq_embed_rows; tok int64 [rows], pos int64 [1]."""
+    rows, hidden = tok.numel(), embed.shape[1]
+    if out is None:
+        out = torch.empty((rows, hidden), dtype=torch.float16, device=embed.device)
+    _check(lib().sq_embed_rows(_ptr(embed), _ptr(pos_table), _ptr(tok), _ptr(pos), int(pos_offset), _ptr(out), rows, hidden,
+                               embed.shape[0], pos_table.shape[0], _stream(stream)), "sq_embed_rows")
+    return out
+
+
+def f16_gemv(x, w, out=None, parts=None, stream=None):
+    """y [M, N] = x [M, K] w[N, K]^T in fp16 through sq_f16_gemv (M <= 8).  parts: None, or a (values, rows) pair of
+    float32 / int32 tensors [8, sq_f16_gemv_parts(N)] that receive every workgroup's best candidate per token."""
+    n, k = w.shape
+    m = x.numel() // k
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.float16, device=x.device)
+    pv, pi = parts if parts is not None else (None, None)
+    _check(lib().sq_f16_gemv(_ptr(x), _ptr(w), _ptr(out), _ptr(pv), _ptr(pi), m, n, k, _stream(stream)), "sq_f16_gemv")
+    return out
+
+
+def f16_gemv_parts(n, device):
+    """The (values, rows) pair sq_f16_gemv fills for a weight of n rows."""
+    p = lib().sq_f16_gemv_parts(n)
+    return (torch.empty((8, p), dtype=torch.float32, device=device), torch.empty((8, p), dtype=torch.int32, device=device))
+
+
+def greedy_feedback(parts, m, tok, pos=None, history=None, step=None, stream=None):
+    """tok[i] = argmax of token i from the candidates of f16_gemv; optional history[step] = tok, pos += 1, step += 1
+    (all int64 on the device) through sq_greedy_feedback."""
+    pv, pi = parts
+    _check(lib().sq_greedy_feedback(_ptr(pv), _ptr(pi), pv.shape[1], m, _ptr(tok), _ptr(pos), _ptr(history), _ptr(step),
+                                    0 if history is None else history.shape[0], _stream(stream)), "sq_greedy_feedback")
+    return tok
 
 
 def layernorm(x, gamma, beta, eps=1e-5, out=None, stream=None):

@@ -162,10 +162,29 @@ class OPTDecoder(nn.Module):
         x = _layernorm(self.final_ln, x[:, -1:])
         return torch.matmul(x, self.lm_head.t())  # [B, 1, vocab]
 
+    @torch.no_grad()
+    def greedy_step(self, tok, cache, pos_t, history=None, step_t=None):
+        """One greedy decode step for up to 8 sequences with nothing but library launches, so that a HIP graph
+        holds the whole of it: tok int64 [B, 1] is read at the start and replaced by the chosen tokens at the
+        end, pos_t int64 [1] (the cache row the new keys and values go to) is advanced, and with history int64
+        [T, B] and step_t int64 [1] the chosen tokens are also written to history[step_t].  Embeddings, final
+        LayerNorm, fp16 lm_head and argmax are what forward() computes with torch ops (the embeddings bit for bit;
+        the logits with fp32 sums in another order).  Returns the logits [B, vocab]."""
+        b = tok.shape[0]
+        if getattr(self, "_parts", None) is None:
+            self._parts = capi.f16_gemv_parts(self.lm_head.shape[0], self.lm_head.device)
+        x = capi.embed_rows(self.embed, self.pos, tok.view(-1), pos_t, 2).view(b, 1, self.hidden)
+        for layer, (kc, vc) in zip(self.layers, cache):
+            x = layer(x, kc, vc, pos_t)
+        x = _layernorm(self.final_ln, x.view(b, self.hidden))
+        logits = capi.f16_gemv(x, self.lm_head, parts=self._parts)
+        capi.greedy_feedback(self._parts, b, tok.view(-1), pos=pos_t, history=history, step=step_t)
+        return logits
+
 
 @torch.no_grad()
 def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed=0, fuse_qkv=True,
-            return_tokens=False, lut_density=0.26, scale_std=E2E_SCALE_STD, scale_min=E2E_SCALE_MIN):
+            return_tokens=False, lut_density=0.26, scale_std=E2E_SCALE_STD, scale_min=E2E_SCALE_MIN, fused_ends=True):
     """Greedy generation on random token ids; returns timing and throughput figures."""
     dev = "cuda"
     model = OPTDecoder(layers=layers, dev=dev, seed=seed, scale_std=scale_std, scale_min=scale_min)
@@ -198,14 +217,30 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
 
-    # One decode step with device-side position so that it can be replayed as a graph.
+    # One decode step with device-side position so that it can be replayed as a graph.  fused_ends: embeddings,
+    # lm_head, argmax and the feedback of the chosen token are library launches inside the step (greedy_step);
+    # otherwise they are torch ops, three of them between two replays.
     pos_t = torch.tensor([prompt], device=dev, dtype=torch.long)
     tok = nxt.clone()
     out_tok = torch.empty_like(tok)
+    fused_ends = fused_ends and batch <= 8
+    history = torch.zeros((new_tokens, batch), dtype=torch.long, device=dev) if fused_ends else None
+    step_t = torch.zeros(1, dtype=torch.long, device=dev) if fused_ends else None
+    first_tok = tok.clone()
 
     def step():
-        lg = model(tok, cache, pos_t, pos_ids=pos_t + 2)
-        out_tok.copy_(lg.argmax(-1))
+        if fused_ends:
+            model.greedy_step(tok, cache, pos_t, history, step_t)
+        else:
+            lg = model(tok, cache, pos_t, pos_ids=pos_t + 2)
+            out_tok.copy_(lg.argmax(-1))
+
+    def rewind():
+        # the warm-up and the capture run a step each: put token, position and step counter back
+        tok.copy_(first_tok)
+        pos_t.fill_(prompt)
+        if step_t is not None:
+            step_t.zero_()
 
     graph = None
     if use_graph:
@@ -213,11 +248,13 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             step()  # warm-up outside capture
+            rewind()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=side):  # same stream as the warm-up: per-stream workspaces exist
             step()
+        rewind()
     generated = [tok.clone()]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -226,12 +263,15 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
             graph.replay()
         else:
             step()
-        tok.copy_(out_tok)
-        pos_t += 1
-        generated.append(tok.clone())
+        if not fused_ends:
+            tok.copy_(out_tok)
+            pos_t += 1
+            generated.append(tok.clone())
     torch.cuda.synchronize()
     decode_s = time.perf_counter() - t0
     steps = new_tokens - 1
+    if fused_ends:
+        generated += [history[i].view(batch, 1).clone() for i in range(steps)]
     extra = {"tokens": torch.stack(generated).cpu()} if return_tokens else {}
     # Algorithmic bytes of one decode step: every packed weight with its zeros/scales and the batch's
     # activations (N*K/2 + (K/g)*N*4 + M*K*2 + M*N*2 per linear, q/k/v as one linear), the valid K/V cache
@@ -253,7 +293,8 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
         "launch": "hip-graph replay" if graph is not None else "eager",
         "fused": "bias+relu+residual in the GEMM store" + ("; q/k/v one launch" if fuse_qkv else "") +
                  "; both LayerNorms inside the q/k/v and fc1 kernels at decode; decode attention appends K/V in the same "
-                 "launch",
+                 "launch" + ("; embeddings, fp16 lm_head + argmax, token feedback as three launches inside the step"
+                             if fused_ends else ""),
         "prefill_ms": round(prefill_s * 1e3, 2),
         "prefill_attention": "dense causal (torch SDPA)",
         "prefill_lut_ms": None if prefill_lut_s is None else round(prefill_lut_s * 1e3, 2),
@@ -268,7 +309,8 @@ def run_e2e(batch=8, prompt=512, new_tokens=128, layers=32, use_graph=True, seed
                      "what": "int4 weights + zeros/scales + activations of the %d x 4 linears, K/V cache rows read once "
                              "(%.0f rows on average), fp16 lm_head; per decode step" % (layers, rows_avg)},
         "parity": "covered by tests/test_gpu_full_size.py: one full-width decoder layer against the oracle composition, "
-                  "eager and HIP-graph decode steps generate identical tokens",
+                  "eager and HIP-graph decode steps generate identical tokens; tests/test_gpu_step_ends.py: the step "
+                  "with library launches at its ends generates the tokens of the step with torch ops there",
         "tokens_checksum": int(torch.stack(generated).sum().item()),
         "logits_finite": bool(torch.isfinite(logits).all().item()),
     }
