@@ -98,7 +98,7 @@ __global__ __launch_bounds__(64 * DA_WAVES) void decode_attn_kernel(DecodeAttnAr
         for (int u = 0; u < DA_U; u++) {
             const int j = imin(base + u * RPI + r, r1 - 1);
             const half_t* src = (append && j == n0) ? fresh : cache + (long)j * D;
-            dst[u] = *(const u32x4_t*)src;
+            dst[u] = __builtin_nontemporal_load((const u32x4_t*)src);
         }
     };
     // The appended row goes into the cache once, up front, by the lanes of the workgroup whose share holds it
