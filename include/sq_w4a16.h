@@ -89,7 +89,9 @@ int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y,
  * decode kernel for 5..32 tokens otherwise on weights of 2^25 elements or more or with
  * K > 8192 and for 17..32 tokens on any weight, the same kernel in two blocks for 33..48
  * tokens on such weights, and a K split of the tiled GEMM for larger M whose grid would
- * leave most CUs idle.  A workspace that is NULL, misaligned or too small is ignored under
+ * leave most CUs idle and for 17..32 tokens on weights of 2^25 elements or more that the
+ * two-tile streaming kernel would serve in part-empty rounds of workgroups (K a multiple
+ * of 256; at group size 64 and 32, N >= 8192).  A workspace that is NULL, misaligned or too small is ignored under
  * SQ_ALGO_AUTO (the workspace-free kernels run); an explicit SQ_ALGO_SKINNY_WS then
  * returns SQ_ERR_WORKSPACE. */
 int sq_w4a16_gemm_ws(const void* x, const void* w, const void* zs, void* y,
@@ -133,7 +135,7 @@ int sq_w4a16_autotune_clear(void);
  * allocates and frees nothing.  The caller still passes inputs and the output.
  * Limit: a call whose kernels would take more than SQ_STATIC_WS_BYTES from a workspace is rejected
  * with SQ_ERR_STATIC_WS and nothing is launched: the split-K decode kernels at 3..32 tokens (every
- * such batch with N <= 16384 fits) and the K splits of the tiled GEMM beyond 32 tokens.  One or two
+ * such batch with N <= 16384 fits) and the K splits of the tiled GEMM beyond 16 tokens.  One or two
  * tokens, and a GEMM whose grid fills the chip without a K split, use no workspace and are never
  * rejected, whatever N is.
  * The first call on a device looks the buffer's address up (hipGetSymbolAddress); nothing is

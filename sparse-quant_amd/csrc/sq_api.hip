@@ -100,8 +100,9 @@ enum : unsigned {
     P_K_LE_4096 = 1u << 7,
     P_K_LE_8192 = 1u << 8,
     P_K_LE_32768 = 1u << 9,
-    P_WIDE = 1u << 10,      // 64-row blocks (times the K split) of the two-tile streaming kernel fill half the chip
+    P_WIDE = 1u << 10,      // the two-tile streaming kernel applies and its workgroups come in one round or fill their rounds
     P_SMALL = 1u << 11,     // N * K <= 2^22 elements and K <= 2048
+    P_N_GE_8192 = 1u << 12, // 32 or more 256-column tiles: a K split of up to 8 gives every CU a workgroup of the tiled GEMM
 };
 constexpr int ALGO_TWO_BLOCKS = 100;  // internal: the split-K decode kernel on two blocks of up to 32 tokens
 struct ChoiceRule {
@@ -123,6 +124,15 @@ const ChoiceRule kChoiceRules[] = {
     // its two-tile variant, 17..32 tokens
     {17, 32, P_G128 | P_WIDE, 0, SQ_ALGO_STREAM,
      "32 tokens: fc1 16.5 vs 17.2 (split-K kernel), q/k/v-sized 14.3 vs 15.5, fc2 18.1 vs 19.0"},
+    // large weights whose grid leaves the two-tile kernel's last round part empty or whose K leaves chunk slots of
+    // its workgroups unused: the tiled GEMM's 32-row tiles with K split through the workspace
+    {17, 32, P_LARGE | P_K256 | P_GEMM_WS | P_G128, 0, SQ_ALGO_GEMM,
+     "32 tokens: 13824x5120 20.2 vs 27.7 (two-tile kernel: 1.7 rounds of workgroups at 20 of 32 chunk slots), "
+     "28672x8192 47.2 vs 56.7, 8192x28672 45.6 vs 55.6, 5120x13824 23.3 vs 26.9, 22016x4096 24.3 vs 25.9"},
+    // the same at group size 64 and 32 (no two-tile kernel) on weights with enough columns of tiles; long K on few
+    // rows stays with the split-K kernel below (group size 64, 4096x16384: 19.6 vs 25.2 for the tiled GEMM)
+    {17, 32, P_LARGE | P_K256 | P_GEMM_WS | P_N_GE_8192, 0, SQ_ALGO_GEMM,
+     "32 tokens, group size 64: fc1 18.4, 12288x4096 16.0, 13824x5120 20.7, 28672x8192 53.6: no other kernel faster"},
     // the tiled GEMM with every operand through LDS and K split through the workspace, beyond 32 tokens
     {33, 1 << 30, P_K256 | P_GEMM_WS, 0, SQ_ALGO_GEMM,
      "48 tokens: 4096x4096 14.5 vs 17.2 (two blocks of the split-K kernel), fc1 24.7 vs 28.2, fc2 27.0 vs 32.3; "
@@ -154,10 +164,20 @@ int builtin_choice(int M, int N, int K, int g, bool ws_ok, bool gemm_ws) {
     if (K % 128 == 0) p |= P_K128;
     if (K % 256 == 0) p |= P_K256;
     if ((long)N * (long)K <= (1L << 22) && K <= 2048) p |= P_SMALL;
+    if (N >= 8192) p |= P_N_GE_8192;
     if (K <= 4096) p |= P_K_LE_4096;
     if (K <= 8192) p |= P_K_LE_8192;
     if (K <= 32768) p |= P_K_LE_32768;
-    if (M > 16 && M <= 32 && g == 128 && sq::skinny3_wide_applies(N, K, ws_ok)) p |= P_WIDE;
+    if (M > 16 && M <= 32 && g == 128) {
+        // One workgroup per CU: W workgroups take ceil(W / 256) rounds of about the same length whatever part of
+        // their 32 chunk slots the K range fills.
+        long wgs = 0;
+        int slots = 0;
+        if (sq::skinny3_wide_shape(N, K, ws_ok, &wgs, &slots)) {
+            const long rounds = (wgs + 255) / 256;
+            if (wgs <= 256 || wgs * slots * 100 >= rounds * 256 * 32 * 95) p |= P_WIDE;
+        }
+    }
     for (const ChoiceRule& r : kChoiceRules)
         if (M >= r.m_lo && M <= r.m_hi && (p & r.need) == r.need && (p & r.forbid) == 0) return r.kernel;
     return SQ_ALGO_GEMM;
@@ -190,7 +210,7 @@ int gemm_dispatch(const void* x, const void* w, const void* zs, void* y, int M, 
         const bool ws_ok = workspace && aligned16(workspace) &&
                            workspace_bytes >= sq::skinny2_workspace_bytes(M > 32 ? 32 : M, N, K) &&
                            (N + 63) / 64 <= 16384;
-        const bool gemm_ws = workspace && aligned16(workspace) && M > 32 &&
+        const bool gemm_ws = workspace && aligned16(workspace) && M > 16 &&
                              workspace_bytes >= sq::gemm_workspace_bytes(M, N, K);
         kernel = builtin_choice(M, N, K, group_size, ws_ok, gemm_ws);
         if (kernel == ALGO_TWO_BLOCKS) {
@@ -276,7 +296,7 @@ int sq_w4a16_gemm_ex(const void* x, const void* w, const void* zs, void* y, int 
 size_t sq_w4a16_workspace_bytes(int M, int N, int K) {
     if (M <= 0 || N <= 0 || K <= 0) return 0;
     const size_t a = sq::skinny2_workspace_bytes(M > 32 ? 32 : M, N, K);
-    const size_t b = M > 32 ? sq::gemm_workspace_bytes(M, N, K) : 0;
+    const size_t b = M > 16 ? sq::gemm_workspace_bytes(M, N, K) : 0;
     return a > b ? a : b;
 }
 
@@ -441,9 +461,13 @@ int sq_w4a16_gemm_static_ws(const void* x, const void* w, const void* zs, void* 
     if (layout != SQ_LAYOUT_L1) return SQ_ERR_BAD_LAYOUT;
     // What the kernels of this token count would take from a workspace: nothing up to 2 tokens (the GEMV has
     // no workspace form), the split-K decode kernels' counters and partial tiles up to 32, the tiled GEMM's K
-    // split beyond.  A shape that wants more than the static buffer is refused rather than served by a slower
-    // workspace-free kernel behind the caller's back.
-    const size_t need = M <= 2 ? 0 : (M <= 32 ? sq::skinny2_workspace_bytes(M, N, K) : sq::gemm_workspace_bytes(M, N, K));
+    // split beyond and where the automatic choice takes it at 17..32.  A shape that wants more than the static
+    // buffer is refused rather than served by a slower workspace-free kernel behind the caller's back.
+    size_t need = M <= 2 ? 0 : (M <= 32 ? sq::skinny2_workspace_bytes(M, N, K) : sq::gemm_workspace_bytes(M, N, K));
+    if (M > 16 && M <= 32 && builtin_choice(M, N, K, group_size, true, true) == SQ_ALGO_GEMM) {
+        const size_t b = sq::gemm_workspace_bytes(M, N, K);
+        if (b > need) need = b;
+    }
     if (need > (size_t)SQ_STATIC_WS_BYTES) return SQ_ERR_STATIC_WS;
     if (M == 0) return SQ_OK;
     if (!x || !w || !zs || !y) return SQ_ERR_NULL_POINTER;

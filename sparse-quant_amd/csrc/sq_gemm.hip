@@ -488,7 +488,7 @@ struct GemmPlan {
     int mi, ksplit, pipe;
     int lds = 0;  // 1: gemm_lds_kernel (group size 32, 64 or 128, K a multiple of 256)
 };
-// Group size 32, 64 or 128 with K a multiple of 256 and more than 32 tokens: gemm_lds_kernel; tile height and K
+// Group size 32, 64 or 128 with K a multiple of 256 and more than 16 tokens: gemm_lds_kernel; tile height and K
 // split come from the cost model below.  Only a long K whose 256 x 256 tiles fill whole rounds stays with the
 // pipelined kernel (4096 x 16384 at 4096 tokens: 497 against 530 us); at group size 32, where this kernel refills
 // its zeros/scales every step, any K does (fc1 at 2048 tokens: 285 against 302 us).
@@ -545,7 +545,7 @@ static GemmPlan plan_gemm(int M, int N, int K, int g, bool have_ws) {
     const long t256 = ntiles(256);
     const long rounds = (t256 + 255) / 256;
     const int nit = (K + GEMM_BK - 1) / GEMM_BK;
-    if ((g == 128 || g == 64 || g == 32) && K % 256 == 0 && M > 32) return plan_gemm_lds(M, ncol, nit, g, have_ws);
+    if ((g == 128 || g == 64 || g == 32) && K % 256 == 0 && M > 16) return plan_gemm_lds(M, ncol, nit, g, have_ws);
     if (M > 64 && t256 * 10 >= rounds * 256 * 6) {
         p.pipe = 2;  // 256 x 256 tiles pay from about 60 % of the CUs (5120 x 13696 at M = 2048: 338 us against 390 us)
     } else if (M > 64 && ntiles(128) >= 160) {

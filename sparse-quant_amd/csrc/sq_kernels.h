@@ -80,6 +80,7 @@ hipError_t launch_skinny3_group(const SeqProblem* probs, int count, int M, void*
 hipError_t launch_skinny3_wide(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                                Epilogue epi, hipStream_t st);
 bool skinny3_wide_applies(int N, int K, bool have_ws);
+bool skinny3_wide_shape(int N, int K, bool have_ws, long* workgroups, int* slots_in_use);
 hipError_t launch_skinny3_wide_group(const SeqProblem* probs, int count, int M, void* ws, size_t ws_bytes,
                                      hipStream_t st);
 // sq_gemm.hip: any M.  tune = 32-row tiles per workgroup (1,2,4) | ksplit << 8; ws may be null.

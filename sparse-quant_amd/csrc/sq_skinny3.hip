@@ -980,6 +980,16 @@ bool skinny3_wide_applies(int N, int K, bool have_ws) {
     return wide_fits((N + 63) / 64, K, have_ws, &ks);
 }
 
+// The same with the grid it would run: workgroups, and how many of a workgroup's 32 chunk slots its K range fills.
+bool skinny3_wide_shape(int N, int K, bool have_ws, long* workgroups, int* slots_in_use) {
+    int ks;
+    const long blocks64 = (N + 63) / 64;
+    if (!wide_fits(blocks64, K, have_ws, &ks)) return false;
+    *workgroups = blocks64 * ks;
+    *slots_in_use = (K / 128 + ks - 1) / ks;
+    return true;
+}
+
 // ws = the caller's workspace or null (then K is never split); it must hold skinny2_workspace_bytes(M, N, K).
 hipError_t launch_skinny3_wide(const void* x, const void* w, const void* zs, void* y, void* ws, int M, int N, int K,
                                Epilogue epi, hipStream_t st) {

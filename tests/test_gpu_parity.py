@@ -927,3 +927,30 @@ def test_random_shapes_fused_auto_dispatch(capi, seed):
             what = (seed, c, m, n, k, g, use_b, use_r, act, use_ws)
             assert np.all(np.isfinite(y)), what
             assert np.max(np.abs(y - y_ref)) <= TOL * max(np.max(np.abs(y_ref)), 1e-6), what
+
+
+@pytest.mark.parametrize("m,n,k,g", [(32, 13824, 5120, 128), (17, 13824, 5120, 128), (24, 5120, 13824, 128),
+                                     (32, 8192, 4352, 64), (20, 8192, 4352, 32)])
+def test_large_weights_17_to_32_tokens_auto_dispatch(capi, m, n, k, g):
+    """Large weights whose K is no multiple of 4096 at 17..32 tokens, which the automatic choice serves with the tiled
+    GEMM's 32-row tiles and a K split through the workspace: every output element against the oracle with bias,
+    ReLU and residual in the store, and against the split-K decode kernel asked for by name on the same operands."""
+    d = orc.synth_linear(n, k, g, seed=n + k + m)
+    w_hat = orc.dequant_l1(d["w_l1"], d["zs_l1"], g)
+    x = orc.synth_x(m, k, seed=m + 3)
+    rng = np.random.default_rng(m + n)
+    bias = (rng.standard_normal(n) * 2).astype(np.float16)
+    res = (rng.standard_normal((m, n)) * 2).astype(np.float16)
+    y_ref = np.maximum(orc.gemm_ref(x, w_hat) + bias.astype(np.float32), 0) + res.astype(np.float32)
+    xd, wd, zd, bd, rd = to_dev(x), to_dev(d["w_l1"]), to_dev(d["zs_l1"]), to_dev(bias), to_dev(res)
+    scale = np.max(np.abs(y_ref))
+    for use_ws in (True, False):
+        y = capi.gemm_fused(xd, wd, zd, n, k, g, bias=bd, residual=rd, act=capi.SQ_ACT_RELU, use_workspace=use_ws)
+        torch.cuda.synchronize()
+        y = y.float().cpu().numpy()
+        assert np.all(np.isfinite(y))
+        assert np.max(np.abs(y - y_ref)) <= TOL * scale, (m, n, k, g, use_ws)
+    y_named = capi.gemm_fused(xd, wd, zd, n, k, g, bias=bd, residual=rd, act=capi.SQ_ACT_RELU,
+                              algo=capi.SQ_ALGO_SKINNY_WS, use_workspace=True)
+    torch.cuda.synchronize()
+    assert np.max(np.abs(y_named.float().cpu().numpy() - y_ref)) <= TOL * scale

@@ -31,9 +31,10 @@ def test_static_workspace_entry_point_matches_the_caller_workspace_one(capi):
     # (M, N, K): split-K decode kernel on a large weight, then a smaller problem on a small weight, then a
     # K-split tiled GEMM and a shape that needs no workspace at all
     # (the last two: a single token and 2048 tokens on an lm_head-sized weight, N = 50272, which need no workspace
-    # although the query for decode batches on that weight exceeds the static buffer)
+    # although the query for decode batches on that weight exceeds the static buffer); 24 tokens on 13824 x 5120 take
+    # the tiled GEMM with K split four ways (7 MiB of partial tiles)
     cases = [(16, 8192, 4096), (20, 1024, 2048), (8, 8192, 4096), (96, 1024, 4096), (3, 512, 1024), (1, 50272, 1024),
-             (2048, 50272, 1024)]
+             (2048, 50272, 1024), (24, 13824, 5120)]
     data = {}
     for m, n, k in cases:
         if (n, k) not in data:
