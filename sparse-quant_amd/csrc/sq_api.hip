@@ -103,6 +103,7 @@ enum : unsigned {
     P_WIDE = 1u << 10,      // the two-tile streaming kernel applies and its workgroups come in one round or fill their rounds
     P_SMALL = 1u << 11,     // N * K <= 2^22 elements and K <= 2048
     P_N_GE_8192 = 1u << 12, // 32 or more 256-column tiles: a K split of up to 8 gives every CU a workgroup of the tiled GEMM
+    P_K_LE_1536 = 1u << 13,
 };
 constexpr int ALGO_TWO_BLOCKS = 100;  // internal: the split-K decode kernel on two blocks of up to 32 tokens
 struct ChoiceRule {
@@ -133,6 +134,10 @@ const ChoiceRule kChoiceRules[] = {
     // rows stays with the split-K kernel below (group size 64, 4096x16384: 19.6 vs 25.2 for the tiled GEMM)
     {17, 32, P_LARGE | P_K256 | P_GEMM_WS | P_N_GE_8192, 0, SQ_ALGO_GEMM,
      "32 tokens, group size 64: fc1 18.4, 12288x4096 16.0, 13824x5120 20.7, 28672x8192 53.6: no other kernel faster"},
+    // small weights with a short K at 33..64 tokens: still the 16-column kernel (from K = 2048 on the GEMM wins)
+    {33, 64, P_SMALL | P_K_LE_1536, 0, SQ_ALGO_SKINNY,
+     "48 tokens: 3072x768 5.6 vs 8.6 (tiled GEMM), 4096x1024 6.3 vs 8.6, 1024x1024 5.9 vs 8.1, 1536x1536 7.8 vs 9.9; "
+     "64 tokens: 6.8 vs 8.6, 7.3 vs 8.7, 6.9 vs 8.1, 9.2 vs 10.0; 2048x2048 at 64 tokens 12.0 vs 10.7"},
     // the tiled GEMM with every operand through LDS and K split through the workspace, beyond 32 tokens
     {33, 1 << 30, P_K256 | P_GEMM_WS, 0, SQ_ALGO_GEMM,
      "48 tokens: 4096x4096 14.5 vs 17.2 (two blocks of the split-K kernel), fc1 24.7 vs 28.2, fc2 27.0 vs 32.3; "
@@ -165,6 +170,7 @@ int builtin_choice(int M, int N, int K, int g, bool ws_ok, bool gemm_ws) {
     if (K % 256 == 0) p |= P_K256;
     if ((long)N * (long)K <= (1L << 22) && K <= 2048) p |= P_SMALL;
     if (N >= 8192) p |= P_N_GE_8192;
+    if (K <= 1536) p |= P_K_LE_1536;
     if (K <= 4096) p |= P_K_LE_4096;
     if (K <= 8192) p |= P_K_LE_8192;
     if (K <= 32768) p |= P_K_LE_32768;

@@ -368,19 +368,20 @@ hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void
     const int nsteps = (K + 511) / 512;
     // Measured on MI355X (cold weights, M = 1): K = 16384 wants 4 k ranges x 2 row groups,
     // 16384 x 4096 wants 2 x 4, 4096 x 4096 wants 1 x 4.
+    // A wave issues its k-steps in rounds of 2, 4 or 8: the k-step slots a split into k_ ranges streams.
+    const int smax = M <= 2 ? 8 : 4;
+    auto slots = [&](int k_) {
+        const int spw_ = (nsteps + k_ - 1) / k_;
+        const int s_ = (spw_ >= 8 && smax >= 8) ? 8 : (spw_ >= 4 ? 4 : 2);
+        return (spw_ + s_ - 1) / s_ * s_ * k_;
+    };
     if (ks != 1 && ks != 2 && ks != 4) {
         // (two ranges from 24 M weights up: 5120 x 5120 at M = 1 7.3 -> 6.7 us; 4096 x 4096 stays at one)
         ks = nsteps > 16 ? 4 : (((long)N * K >= (3L << 23) && nsteps >= 8) ? 2 : 1);
         if (M >= 3 && M <= 4 && ks == 1 && nsteps >= 8) ks = 2;  // 4096 x 4096 with 3..4 tokens: 4.5 vs 5.6 us
-        // A wave issues its k-steps in rounds of 2, 4 or 8; a K whose steps do not fill the rounds of that choice
-        // (11008 = 21.5 steps: 4 ranges x 2 rounds x 4 = 32 slots) streams padding.  Take the split that wastes
-        // least when the first choice wastes more than an eighth (4096 x 11008 at M = 1: 8.9 -> 7.9 us).
-        const int smax = M <= 2 ? 8 : 4;
-        auto slots = [&](int k_) {
-            const int spw_ = (nsteps + k_ - 1) / k_;
-            const int s_ = (spw_ >= 8 && smax >= 8) ? 8 : (spw_ >= 4 ? 4 : 2);
-            return (spw_ + s_ - 1) / s_ * s_ * k_;
-        };
+        // A K whose steps do not fill the rounds of that choice (11008 = 21.5 steps: 4 ranges x 2 rounds x 4 = 32
+        // slots) streams padding.  Take the split that wastes least when the first choice wastes more than an
+        // eighth (4096 x 11008 at M = 1: 8.9 -> 7.9 us).
         if (slots(ks) * 8 > nsteps * 9) {
             int best = ks;
             for (int k_ : {4, 2, 1})
@@ -389,7 +390,10 @@ hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void
         }
     }
     if (nr != 2 && nr != 4 && nr != 8) {
-        nr = (ks == 4 && M <= 1) ? 2 : 4;  // 4096 x 16384 at M = 4: 12.8 vs 13.7 us
+        // (one token on a split K >= 8192: two row groups, i.e. twice as many workgroups of half the size -- 8192 x 8192
+        // 9.2 -> 8.8 us, 16384 x 8192 16.0 -> 14.7, 28672 x 8192 26.4 -> 23.9; 4096 x 16384 at M = 4 wants four:
+        // 12.8 vs 13.7 us)
+        nr = ((ks == 4 || (ks == 2 && nsteps >= 16)) && M <= 1) ? 2 : 4;
         // The busiest CU gets ceil(workgroups / 256) workgroups of 4 nr rows each: where halving the workgroup
         // lowers that product, halve it (5120 rows: 320 workgroups of 16 rows are two rounds for a quarter of the
         // CUs; 5120 x 13824 at M = 2: 16.0 -> 12.6 us.  1024 rows: 64 workgroups leave three CUs in four idle).
@@ -398,7 +402,9 @@ hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void
         // and a weight that gives the chip less than one wave per SIMD splits K further, down to two k-steps
         // per wave (M = 1: 1024 x 8192 5.0 -> 3.4 us, 768 x 3072 3.4 -> 2.8, 2048 x 2048 at 2 tokens 3.05 -> 2.7)
         if (((tune >> 4) & 0xF) == 0)
-            while (ks < 4 && (long)((N + 4 * nr - 1) / (4 * nr)) * nr * ks < 1024 && nsteps > 2 * ks) ks *= 2;
+            while (ks < 4 && (long)((N + 4 * nr - 1) / (4 * nr)) * nr * ks < 1024 && nsteps > 2 * ks &&
+                   slots(2 * ks) <= slots(ks))  // (not into padding: 2560 x 10240, 20 k-steps, 8.2 -> 7.3 us unsplit)
+                ks *= 2;
     }
     const int spw = (nsteps + ks - 1) / ks;
     if (M <= 1) return launch_rows<1>(nr, ks, spw, x, w, zs, y, M, N, K, gshift, fixup, epi, st);

@@ -859,7 +859,7 @@ Sk3Plan plan(const int* rows, int count, int K, bool have_ws, int tune, int M) {
     }
     // Rows per workgroup (64, 48 or 16) and K split (the least one, or two or four times as fine) by a count of
     // time calibrated on timed launches at 8 and 16 tokens, in units of 1.75 us (what a CU needs to stream one
-    // 16-row tile over a full range of 32 chunks): rounds of 256 workgroups (one per CU) x ((row tiles + M / 24 for
+    // 16-row tile over a full range of 32 chunks): rounds of 256 workgroups (one per CU; 512 below) x ((row tiles + M / 24 for
     // the activations, which come from L2 at a sixth of the price per byte) x the part of a full range a workgroup
     // covers + 1 for a workgroup's start: its activations must be there before its first matrix instruction),
     // + 1.54 (2.7 us) where partial tiles are exchanged.  OPT-6.7B: 4096 rows -> 16 (256 workgroups), 12288 and
@@ -877,7 +877,10 @@ Sk3Plan plan(const int* rows, int count, int K, bool have_ws, int tune, int M) {
             if (rt == 3 && (ks != 1 || p.ch != 4)) continue;
             long blocks = 0;
             for (int l = 0; l < count; l++) blocks += (rows[l] + 16 * rt - 1) / (16 * rt);
-            const long rounds = (blocks * ks + 255) / 256;
+            // (an unsplit K of at most 2048 leaves room for two workgroups per CU: 6144 x 2048 at 8 tokens in
+            // 16-row workgroups 4.6 against 5.8 us in 64-row ones, 8192 x 1024 3.4 against 3.8)
+            const int per_round = (ks == 1 && p.ch <= 2) ? 512 : 256;
+            const long rounds = (blocks * ks + per_round - 1) / per_round;
             const float cost = rounds * ((rt + M / 24.f) * (cps / 32.f) + 1.f) + (ks > 1 ? 1.54f : 0.f);
             if (cost < best - 1e-3f) {
                 best = cost;
