@@ -104,6 +104,7 @@ enum : unsigned {
     P_SMALL = 1u << 11,     // N * K <= 2^22 elements and K <= 2048
     P_N_GE_8192 = 1u << 12, // 32 or more 256-column tiles: a K split of up to 8 gives every CU a workgroup of the tiled GEMM
     P_K_LE_1536 = 1u << 13,
+    P_CHUNK_FILL = 1u << 14,  // the least K split of the streaming kernel fills 3/4 or more of a workgroup's 32 chunks
 };
 constexpr int ALGO_TWO_BLOCKS = 100;  // internal: the split-K decode kernel on two blocks of up to 32 tokens
 struct ChoiceRule {
@@ -118,7 +119,8 @@ const ChoiceRule kChoiceRules[] = {
      "8 tokens: fc1 10.0 vs 13.3 (split-K kernel), q/k/v in one launch 8.6 vs 12.1, 4096x4096 4.9 vs 6.5 (GEMV)"},
     {5, 16, P_G128_64 | P_K128 | P_WS | P_K_LE_32768, 0, SQ_ALGO_STREAM, "8 tokens: fc2 12.7 vs 14.6 (split-K kernel)"},
     {3, 4, P_LARGE | P_G128_64 | P_K128 | P_K_LE_4096, 0, SQ_ALGO_STREAM, "4 tokens: fc1 9.7 vs 10.7 (GEMV)"},
-    {3, 4, P_LARGE | P_G128_64 | P_K128 | P_WS | P_K_LE_32768, 0, SQ_ALGO_STREAM, "4 tokens: fc2 11.9 vs 13.6 (GEMV)"},
+    {3, 4, P_LARGE | P_G128_64 | P_K128 | P_WS | P_K_LE_32768 | P_CHUNK_FILL, 0, SQ_ALGO_STREAM,
+     "4 tokens: fc2 11.9 vs 13.6 (GEMV); 13824x5120, whose K ranges fill 20 of a workgroup's 32 chunks: 14.6 vs 13.9 (GEMV)"},
     // small weights at 17..32 tokens: the 16-column kernel (one launch, no exchange between workgroups)
     {17, 32, P_SMALL, 0, SQ_ALGO_SKINNY,
      "32 tokens: 2048x2048 7.4 vs 8.6 (split-K kernel), 1024x1024 4.9 vs 6.9, 3072x768 4.8 vs 6.6"},
@@ -171,6 +173,10 @@ int builtin_choice(int M, int N, int K, int g, bool ws_ok, bool gemm_ws) {
     if ((long)N * (long)K <= (1L << 22) && K <= 2048) p |= P_SMALL;
     if (N >= 8192) p |= P_N_GE_8192;
     if (K <= 1536) p |= P_K_LE_1536;
+    {
+        const int chunks = K / 128, ks0 = (chunks + 31) / 32;
+        if (ks0 > 0 && chunks * 4 >= ks0 * 32 * 3) p |= P_CHUNK_FILL;
+    }
     if (K <= 4096) p |= P_K_LE_4096;
     if (K <= 8192) p |= P_K_LE_8192;
     if (K <= 32768) p |= P_K_LE_32768;

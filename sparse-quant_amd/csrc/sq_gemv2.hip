@@ -398,7 +398,10 @@ hipError_t launch_gemv2_tuned(const void* x, const void* w, const void* zs, void
         // lowers that product, halve it (5120 rows: 320 workgroups of 16 rows are two rounds for a quarter of the
         // CUs; 5120 x 13824 at M = 2: 16.0 -> 12.6 us.  1024 rows: 64 workgroups leave three CUs in four idle).
         auto busiest = [&](int r) { return ((N + 4 * r - 1) / (4 * r) + 255) / 256 * r; };
-        if (nr == 4 && busiest(2) < busiest(4)) nr = 2;
+        // (with 3..4 tokens every workgroup stages that many activation rows, and halving only pays where 16-row
+        // workgroups leave CUs without one: 5120 x 5120 at 4 tokens 10.3 -> 8.8 us with four row groups, 6144 x 2048
+        // 5.2 -> 4.2; 2048 x 8192 5.8 with two against 6.7)
+        if (nr == 4 && busiest(2) < busiest(4) && (M <= 2 || (N + 15) / 16 < 256)) nr = 2;
         // and a weight that gives the chip less than one wave per SIMD splits K further, down to two k-steps
         // per wave (M = 1: 1024 x 8192 5.0 -> 3.4 us, 768 x 3072 3.4 -> 2.8, 2048 x 2048 at 2 tokens 3.05 -> 2.7)
         if (((tune >> 4) & 0xF) == 0)
